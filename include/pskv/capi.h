@@ -1,0 +1,172 @@
+/*
+ * pskv C ABI: the MI355X (gfx950) server-side key-value data path of a
+ * ps-lite style parameter server, as a plain-C boundary.
+ *
+ * What sits behind it: an open-addressing hash table resident in HBM
+ * (find-or-insert + accumulate on push, gather on pull), row accumulation for
+ * fixed-length and variable-length values, and the worker-side key-range
+ * slicer (boundary search + lens scan). All kernels are HIP for gfx950.
+ *
+ * Conventions
+ *  - Every function returns an int status: 0 on success, a negative PSKV_E*
+ *    code otherwise; pskv_last_error() gives the text for the calling thread.
+ *    Nothing throws across this boundary.
+ *  - `memkind` says where the caller's buffers live. PSKV_MEM_DEVICE pointers
+ *    are device memory on the table's device and are used in place;
+ *    PSKV_MEM_HOST pointers are ordinary host memory and are staged through
+ *    pinned buffers owned by the library.
+ *  - Calls with PSKV_MEM_DEVICE buffers are asynchronous: work is enqueued on
+ *    the table's stream in call order and the caller's buffers must stay valid
+ *    until pskv_sync(). Input buffers written by other streams must be complete
+ *    before the call. Calls with PSKV_MEM_HOST buffers return when done.
+ *  - Keys within one request must be unique (ps-lite requires sorted unique
+ *    keys, include/ps/kv_app.h:17); requests on one table are applied in call
+ *    order. A table must not be used from two threads at once (the reference
+ *    runs the handle on one Customer thread, src/customer.cc:49-63).
+ *    pskv_slice is re-entrant.
+ *
+ * Reference lines are relative to the root of dmlc/ps-lite.
+ */
+#ifndef PSKV_CAPI_H_
+#define PSKV_CAPI_H_
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PSKV_OK 0
+#define PSKV_EUNCOVERED_KEY (-1) /* a key lies beyond the last range: kv_app.h:542 */
+#define PSKV_ESIZE_MISMATCH (-2) /* kv_app.h:447,489,549,551; sarray.h:249; output too small */
+#define PSKV_ENOMEM (-3)
+#define PSKV_EHIP (-4)           /* a HIP runtime call failed */
+#define PSKV_EINVAL (-5)
+#define PSKV_ERANGE_GAP (-6)     /* ranges[i-1].end != ranges[i].begin: kv_app.h:533 */
+#define PSKV_ELEN_CHANGED (-7)   /* var-len push with a length that differs from the stored row */
+
+#define PSKV_MEM_HOST 0
+#define PSKV_MEM_DEVICE 1
+
+#define PSKV_MODE_SCALAR 0 /* one float per key: KVServerDefaultHandle, kv_app.h:440-463 */
+#define PSKV_MODE_FIXED 1  /* k floats per key, k = vals/keys: KVPairs layout kv_app.h:17-22 */
+#define PSKV_MODE_VARLEN 2 /* lens[i] floats per key: KVPairs layout kv_app.h:24-31 */
+
+/* longest row a PSKV_MODE_VARLEN table stores, in floats */
+#define PSKV_MAX_VARLEN_ROW ((1u << 28) - 1)
+
+/* kernels whose device time pskv_prof_read reports */
+#define PSKV_KERNEL_PUSH_SCALAR 0
+#define PSKV_KERNEL_PULL_SCALAR 1
+#define PSKV_KERNEL_ROWS_ACC 2    /* push accumulate of rows (fixed-k and var-len) */
+#define PSKV_KERNEL_ROWS_GATHER 3 /* pull gather of rows */
+#define PSKV_KERNEL_LOOKUP 4      /* key -> row lookup / insert of the row modes */
+#define PSKV_KERNEL_REHASH 5
+#define PSKV_KERNEL_COUNT 6
+
+typedef struct pskv_table pskv_table;
+
+typedef struct pskv_opts {
+  int32_t device;            /* HIP device ordinal */
+  int32_t mode;              /* PSKV_MODE_* */
+  uint64_t initial_capacity; /* keys the table should hold before its first growth; 0 = default */
+  uint64_t row_len;          /* PSKV_MODE_FIXED: floats per key, 0 = taken from the first push */
+  uint64_t arena_floats;     /* row modes: initial value storage in floats, 0 = default */
+  float max_load;            /* highest fill of the slot array, 0 = 0.5 */
+  uint32_t reserved;
+  void* stream;              /* hipStream_t to run on, NULL = the table creates its own */
+} pskv_opts;
+
+/* Replaces the construction of KVServerDefaultHandle and its std::unordered_map
+ * store (kv_app.h:441,462; tests/test_kv_app.cc:10-11). */
+int pskv_table_create(pskv_table** out, const pskv_opts* opts);
+int pskv_table_destroy(pskv_table* t);
+
+/* Push half of the request handle: `store[keys[i]] += vals[i]` with an absent
+ * key starting from 0 (kv_app.h:444-455). lens is NULL unless the table is
+ * PSKV_MODE_VARLEN (then nlens must equal n, kv_app.h:489). */
+int pskv_push(pskv_table* t, const uint64_t* keys, size_t n, const float* vals, size_t nvals,
+              const int32_t* lens, size_t nlens, int memkind);
+
+/* Pull half of the request handle: `out[i] = store[keys[i]]`, where an absent key
+ * is inserted with value 0 (kv_app.h:448-450,456-458). Row modes write the rows
+ * back to back in request order; PSKV_MODE_VARLEN also writes out_lens[n] and
+ * answers an absent key with length 0 without inserting it. If the response
+ * does not fit out_cap floats the status is PSKV_ESIZE_MISMATCH and *out_nvals
+ * (a host pointer, may be NULL) holds the needed size; out/out_lens are then
+ * unspecified. In PSKV_MODE_VARLEN the call waits for the device even with
+ * PSKV_MEM_DEVICE buffers because the response size is data dependent. */
+int pskv_pull(pskv_table* t, const uint64_t* keys, size_t n, float* out, size_t out_cap,
+              int32_t* out_lens, size_t* out_nvals, int memkind);
+
+/* A request with push and pull both set: per key the push is applied first,
+ * then the value is read back (kv_app.h:451-459). */
+int pskv_pushpull(pskv_table* t, const uint64_t* keys, size_t n, const float* vals, size_t nvals,
+                  const int32_t* lens, size_t nlens, float* out, size_t out_cap,
+                  int32_t* out_lens, size_t* out_nvals, int memkind);
+
+/* Waits for everything enqueued on the table and reports a deferred device-side
+ * error (PSKV_ELEN_CHANGED) of an earlier asynchronous push, once. */
+int pskv_sync(pskv_table* t);
+
+/* Number of keys held: unordered_map::size() of the reference store (kv_app.h:462).
+ * Waits for the device. */
+int pskv_size(pskv_table* t, uint64_t* n_keys, uint64_t* n_vals);
+
+/* All stored pairs sorted by key, for stored-key parity checks (the reference has
+ * no such call; it is the equivalent of iterating the store, kv_app.h:462).
+ * Host buffers only. lens may be NULL. Too small a buffer gives
+ * PSKV_ESIZE_MISMATCH with the needed sizes in *n_keys / *n_vals. */
+int pskv_dump(pskv_table* t, uint64_t* keys, int32_t* lens, size_t cap_keys, float* vals,
+              size_t cap_vals, size_t* n_keys, size_t* n_vals);
+
+/* KVWorker::DefaultSlicer (kv_app.h:517-572): partitions sorted keys over S
+ * contiguous key ranges [range_begin[i], range_end[i]) (host arrays, as returned by
+ * Postoffice::GetServerKeyRanges, src/postoffice.cc:169-180).
+ * Outputs are host arrays: pos[S+1] so that slice i holds keys [pos[i], pos[i+1]),
+ * val_pos[S+1] so that it holds vals [val_pos[i], val_pos[i+1]), used[S] = the
+ * `first` flag of the slice (0 for an empty slice). keys/lens follow memkind;
+ * lens == NULL or nlens == 0 means no lens (value length k = nvals / n).
+ * `device` selects the GPU for PSKV_MEM_HOST inputs and must be the device that
+ * holds PSKV_MEM_DEVICE inputs. */
+int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, size_t nlens,
+               size_t nvals, const uint64_t* range_begin, const uint64_t* range_end, size_t S,
+               uint64_t* pos, uint64_t* val_pos, uint8_t* used, int memkind);
+
+/* Postoffice::GetServerKeyRanges (src/postoffice.cc:169-180) for num_servers
+ * servers; host arrays of num_servers entries each. */
+int pskv_server_ranges(uint64_t num_servers, uint64_t* range_begin, uint64_t* range_end);
+
+/* Worker-side pull reassembly, the callback of KVWorker::AddPullCB
+ * (kv_app.h:663-714): R per-server responses, in any order, are checked against
+ * the request keys, ordered by first key and concatenated into out (and
+ * out_lens when resp_lens is not NULL). The pointer tables and the size tables are
+ * host arrays; what they point to follows memkind, as do req_keys/out/out_lens. */
+int pskv_assemble_pull(int device, const uint64_t* req_keys, size_t n, size_t R,
+                       const uint64_t* const* resp_keys, const size_t* resp_nkeys,
+                       const float* const* resp_vals, const size_t* resp_nvals,
+                       const int32_t* const* resp_lens, float* out, size_t out_cap,
+                       int32_t* out_lens, size_t* out_nvals, int memkind);
+
+/* Device-time accounting for roofline figures (no counterpart in the reference).
+ * While enabled, every launch of the kernels listed above is bracketed by HIP
+ * events on the table's stream. pskv_prof_read waits for the stream and returns
+ * the launch count and the summed duration since the last pskv_prof_reset. */
+int pskv_prof_enable(pskv_table* t, int on);
+int pskv_prof_reset(pskv_table* t);
+int pskv_prof_read(pskv_table* t, int kernel, uint64_t* launches, double* total_ms);
+
+/* Plain device-to-device copy kernel of `bytes` bytes (multiple of 16) on the
+ * table's stream; used to calibrate memory-traffic counters and as the measured
+ * copy ceiling next to the accumulate kernels. No counterpart in the reference. */
+int pskv_copy_probe(pskv_table* t, void* dst, const void* src, size_t bytes);
+
+/* Text of the last error on the calling thread ("" if none). */
+const char* pskv_last_error(void);
+/* "pskv <major>.<minor> gfx950" */
+const char* pskv_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PSKV_CAPI_H_ */

@@ -1,0 +1,267 @@
+"""ctypes binding of libpskv.so, the C ABI declared in include/pskv/capi.h.
+
+Buffers are either numpy arrays (host memory, PSKV_MEM_HOST) or torch tensors
+on the table's device (PSKV_MEM_DEVICE). torch is only the owner of device
+memory here; every computation happens inside libpskv.so.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+from . import build as _build
+
+OK = 0
+EUNCOVERED_KEY = -1
+ESIZE_MISMATCH = -2
+ENOMEM = -3
+EHIP = -4
+EINVAL = -5
+ERANGE_GAP = -6
+ELEN_CHANGED = -7
+MEM_HOST = 0
+MEM_DEVICE = 1
+MODE_SCALAR = 0
+MODE_FIXED = 1
+MODE_VARLEN = 2
+MAX_VARLEN_ROW = (1 << 28) - 1
+KERNEL_PUSH_SCALAR, KERNEL_PULL_SCALAR, KERNEL_ROWS_ACC, KERNEL_ROWS_GATHER, KERNEL_LOOKUP, \
+    KERNEL_REHASH = range(6)
+
+ERROR_NAMES = {
+    EUNCOVERED_KEY: "PSKV_EUNCOVERED_KEY", ESIZE_MISMATCH: "PSKV_ESIZE_MISMATCH",
+    ENOMEM: "PSKV_ENOMEM", EHIP: "PSKV_EHIP", EINVAL: "PSKV_EINVAL",
+    ERANGE_GAP: "PSKV_ERANGE_GAP", ELEN_CHANGED: "PSKV_ELEN_CHANGED",
+}
+
+# every symbol include/pskv/capi.h declares
+SYMBOLS = [
+    "pskv_table_create", "pskv_table_destroy", "pskv_push", "pskv_pull", "pskv_pushpull",
+    "pskv_sync", "pskv_size", "pskv_dump", "pskv_slice", "pskv_server_ranges",
+    "pskv_assemble_pull", "pskv_prof_enable", "pskv_prof_reset", "pskv_prof_read",
+    "pskv_copy_probe", "pskv_last_error", "pskv_version",
+]
+
+
+class PskvError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__("%s: %s" % (ERROR_NAMES.get(code, code), text))
+        self.code = code
+
+
+class Opts(ctypes.Structure):
+    _fields_ = [
+        ("device", ctypes.c_int32), ("mode", ctypes.c_int32),
+        ("initial_capacity", ctypes.c_uint64), ("row_len", ctypes.c_uint64),
+        ("arena_floats", ctypes.c_uint64), ("max_load", ctypes.c_float),
+        ("reserved", ctypes.c_uint32), ("stream", ctypes.c_void_p),
+    ]
+
+
+_lib = None
+
+
+def load():
+    """Loads the built library. There is no fallback: a missing library is an error."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = _build.lib_path()
+    if not os.path.exists(path):
+        raise RuntimeError(
+            "libpskv.so is not built (%s); run `python -c 'import __graft_entry__ as g; g.build()'`" % path)
+    try:
+        import torch  # noqa: F401  (so that one HIP runtime serves torch and this library)
+    except ImportError:
+        pass
+    lib = ctypes.CDLL(path)
+    vp, sz, i32, u64 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_uint64
+    lib.pskv_table_create.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(Opts)]
+    lib.pskv_table_destroy.argtypes = [vp]
+    lib.pskv_push.argtypes = [vp, vp, sz, vp, sz, vp, sz, i32]
+    lib.pskv_pull.argtypes = [vp, vp, sz, vp, sz, vp, ctypes.POINTER(sz), i32]
+    lib.pskv_pushpull.argtypes = [vp, vp, sz, vp, sz, vp, sz, vp, sz, vp, ctypes.POINTER(sz), i32]
+    lib.pskv_sync.argtypes = [vp]
+    lib.pskv_size.argtypes = [vp, ctypes.POINTER(u64), ctypes.POINTER(u64)]
+    lib.pskv_dump.argtypes = [vp, vp, vp, sz, vp, sz, ctypes.POINTER(sz), ctypes.POINTER(sz)]
+    lib.pskv_slice.argtypes = [i32, vp, sz, vp, sz, sz, vp, vp, sz, vp, vp, vp, i32]
+    lib.pskv_server_ranges.argtypes = [u64, vp, vp]
+    lib.pskv_assemble_pull.argtypes = [i32, vp, sz, sz, vp, vp, vp, vp, vp, vp, sz, vp,
+                                       ctypes.POINTER(sz), i32]
+    lib.pskv_prof_enable.argtypes = [vp, i32]
+    lib.pskv_prof_reset.argtypes = [vp]
+    lib.pskv_prof_read.argtypes = [vp, i32, ctypes.POINTER(u64), ctypes.POINTER(ctypes.c_double)]
+    lib.pskv_copy_probe.argtypes = [vp, vp, vp, sz]
+    lib.pskv_last_error.restype = ctypes.c_char_p
+    lib.pskv_version.restype = ctypes.c_char_p
+    _lib = lib
+    return lib
+
+
+def _check(rc):
+    if rc != OK:
+        raise PskvError(rc, load().pskv_last_error().decode())
+
+
+def _is_tensor(x):
+    return hasattr(x, "data_ptr")
+
+
+def _buf(x, dtype_np, dtype_name):
+    """(pointer, element count, memkind or None) of a numpy array / torch tensor / None."""
+    if x is None:
+        return None, 0, None
+    if _is_tensor(x):
+        assert str(x.dtype).endswith(dtype_name), (x.dtype, dtype_name)
+        assert x.is_contiguous()
+        kind = MEM_DEVICE if x.is_cuda else MEM_HOST
+        return (x.data_ptr() if x.numel() else None), x.numel(), kind
+    a = np.ascontiguousarray(x, dtype=dtype_np)
+    return (a.ctypes.data if a.size else None), a.size, MEM_HOST
+
+
+def _memkind(*kinds):
+    ks = {k for k in kinds if k is not None}
+    assert len(ks) <= 1, "all buffers of a call must live in the same kind of memory"
+    return ks.pop() if ks else MEM_HOST
+
+
+class Table:
+    """The store behind a KVServer request handle (kv_app.h:440-463)."""
+
+    def __init__(self, mode=MODE_SCALAR, device=0, initial_capacity=0, row_len=0, arena_floats=0,
+                 max_load=0.0, stream=None):
+        self._lib = load()
+        self._h = ctypes.c_void_p()
+        o = Opts(device, mode, initial_capacity, row_len, arena_floats, max_load, 0, stream)
+        _check(self._lib.pskv_table_create(ctypes.byref(self._h), ctypes.byref(o)))
+        self.mode = mode
+        self.device = device
+
+    def close(self):
+        if self._h:
+            self._lib.pskv_table_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def push(self, keys, vals, lens=None):
+        kp, n, k1 = _buf(keys, np.uint64, "int64")
+        vp, nv, k2 = _buf(vals, np.float32, "float32")
+        lp, nl, k3 = _buf(lens, np.int32, "int32")
+        _check(self._lib.pskv_push(self._h, kp, n, vp, nv, lp, nl, _memkind(k1, k2, k3)))
+
+    def pull(self, keys, out, out_lens=None):
+        """Returns the number of floats of the response."""
+        kp, n, k1 = _buf(keys, np.uint64, "int64")
+        op, cap, k2 = _buf(out, np.float32, "float32")
+        lp, _, k3 = _buf(out_lens, np.int32, "int32")
+        got = ctypes.c_size_t(0)
+        self.last_out_nvals = None
+        rc = self._lib.pskv_pull(self._h, kp, n, op, cap, lp, ctypes.byref(got), _memkind(k1, k2, k3))
+        self.last_out_nvals = got.value
+        _check(rc)
+        return got.value
+
+    def pushpull(self, keys, vals, out, lens=None, out_lens=None):
+        kp, n, k1 = _buf(keys, np.uint64, "int64")
+        vp, nv, k2 = _buf(vals, np.float32, "float32")
+        lp, nl, k3 = _buf(lens, np.int32, "int32")
+        op, cap, k4 = _buf(out, np.float32, "float32")
+        olp, _, k5 = _buf(out_lens, np.int32, "int32")
+        got = ctypes.c_size_t(0)
+        rc = self._lib.pskv_pushpull(self._h, kp, n, vp, nv, lp, nl, op, cap, olp, ctypes.byref(got),
+                                     _memkind(k1, k2, k3, k4, k5))
+        self.last_out_nvals = got.value
+        _check(rc)
+        return got.value
+
+    def sync(self):
+        _check(self._lib.pskv_sync(self._h))
+
+    def size(self):
+        nk, nv = ctypes.c_uint64(0), ctypes.c_uint64(0)
+        _check(self._lib.pskv_size(self._h, ctypes.byref(nk), ctypes.byref(nv)))
+        return nk.value, nv.value
+
+    def dump(self):
+        """(keys sorted, lens, vals) as numpy arrays."""
+        nk, nv = self.size()
+        keys = np.zeros(nk, np.uint64)
+        lens = np.zeros(nk, np.int32)
+        vals = np.zeros(nv, np.float32)
+        a, b = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        _check(self._lib.pskv_dump(self._h, keys.ctypes.data, lens.ctypes.data, nk, vals.ctypes.data,
+                                   nv, ctypes.byref(a), ctypes.byref(b)))
+        return keys, lens, vals
+
+    def prof_enable(self, on=True):
+        _check(self._lib.pskv_prof_enable(self._h, 1 if on else 0))
+
+    def prof_reset(self):
+        _check(self._lib.pskv_prof_reset(self._h))
+
+    def prof_read(self, kernel):
+        n, ms = ctypes.c_uint64(0), ctypes.c_double(0.0)
+        _check(self._lib.pskv_prof_read(self._h, kernel, ctypes.byref(n), ctypes.byref(ms)))
+        return n.value, ms.value
+
+    def copy_probe(self, dst, src):
+        assert dst.is_cuda and src.is_cuda
+        nbytes = src.numel() * src.element_size()
+        _check(self._lib.pskv_copy_probe(self._h, dst.data_ptr(), src.data_ptr(), nbytes))
+
+
+def server_ranges(num_servers):
+    """Postoffice::GetServerKeyRanges (src/postoffice.cc:169-180) as two uint64 arrays."""
+    b = np.zeros(num_servers, np.uint64)
+    e = np.zeros(num_servers, np.uint64)
+    _check(load().pskv_server_ranges(num_servers, b.ctypes.data, e.ctypes.data))
+    return b, e
+
+
+def slice_keys(keys, range_begin, range_end, lens=None, nvals=0, device=0):
+    """KVWorker::DefaultSlicer (kv_app.h:517-572): returns (pos, val_pos, used)."""
+    kp, n, k1 = _buf(keys, np.uint64, "int64")
+    lp, nl, k2 = _buf(lens, np.int32, "int32")
+    rb = np.ascontiguousarray(range_begin, dtype=np.uint64)
+    re = np.ascontiguousarray(range_end, dtype=np.uint64)
+    S = rb.size
+    pos = np.zeros(S + 1, np.uint64)
+    val_pos = np.zeros(S + 1, np.uint64)
+    used = np.zeros(max(S, 1), np.uint8)
+    _check(load().pskv_slice(device, kp, n, lp, nl, nvals, rb.ctypes.data, re.ctypes.data, S,
+                             pos.ctypes.data, val_pos.ctypes.data, used.ctypes.data,
+                             _memkind(k1, k2)))
+    return pos, val_pos, used[:S]
+
+
+def assemble_pull(req_keys, responses, out, out_lens=None, device=0):
+    """Device-side counterpart of the KVWorker::AddPullCB callback (kv_app.h:663-714).
+    responses: list of (keys, vals, lens-or-None) device tensors in arrival order."""
+    R = len(responses)
+    PA = ctypes.c_void_p * max(R, 1)
+    SA = ctypes.c_size_t * max(R, 1)
+    kptr, vptr, lptr, nk, nv = PA(), PA(), PA(), SA(), SA()
+    have_lens = R > 0 and all(r[2] is not None for r in responses)
+    for i, (k, v, l) in enumerate(responses):
+        kptr[i], nk[i] = k.data_ptr() if k.numel() else None, k.numel()
+        vptr[i], nv[i] = v.data_ptr() if v.numel() else None, v.numel()
+        if have_lens:
+            lptr[i] = l.data_ptr() if l.numel() else None
+    kp, n, _ = _buf(req_keys, np.uint64, "int64")
+    op, cap, _ = _buf(out, np.float32, "float32")
+    olp, _, _ = _buf(out_lens, np.int32, "int32")
+    got = ctypes.c_size_t(0)
+    _check(load().pskv_assemble_pull(device, kp, n, R, kptr, nk, vptr, nv,
+                                     lptr if have_lens else None, op, cap, olp, ctypes.byref(got),
+                                     MEM_DEVICE))
+    return got.value
+
+
+def version():
+    return load().pskv_version().decode()

@@ -1,0 +1,136 @@
+// Shared device-side definitions of the pskv library (gfx950 only).
+#ifndef PSKV_DEVICE_COMMON_H_
+#define PSKV_DEVICE_COMMON_H_
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pskv {
+
+// ps::kMaxKey (include/ps/base.h:18). The stock server ranges never cover it
+// (src/postoffice.cc:169-180), so it marks an empty slot; a caller that pushes it
+// directly is served from one side slot kept in DevState.
+constexpr uint64_t kEmptyKey = ~0ull;
+
+// Row reference handed from the lookup kernel to the row kernels.
+//   FIXED : low bits = row index
+//   VARLEN: bits [28,63) = arena offset in 16-byte units, bits [0,28) = row length in floats
+// bit 63 = the key was created by this request; all ones = key absent (var-len pull).
+constexpr uint64_t kRefNew = 1ull << 63;
+constexpr uint64_t kRefAbsent = ~0ull;
+constexpr int kLenBits = 28;
+constexpr uint64_t kLenMask = (1ull << kLenBits) - 1;
+
+// sticky device-side error bits (DevState::error)
+constexpr unsigned kDevErrLenChanged = 1u;  // var-len push: stored length differs
+constexpr unsigned kDevErrFull = 2u;        // probe sequence found no free slot (host sizing bug)
+constexpr unsigned kDevErrBadLen = 4u;      // negative or too long length
+constexpr unsigned kDevErrSizeMismatch = 8u;  // lens do not add up to the number of values
+
+constexpr int kBlock = 256;             // threads per workgroup of every kernel here (4 waves)
+constexpr unsigned kTileFloats = 4096;  // request-side floats handled by one workgroup of the row kernels
+constexpr unsigned kSpanMax = 1024;     // keys whose offsets a row-kernel workgroup stages in LDS
+
+struct __align__(16) Slot {
+  uint64_t key;
+  uint64_t payload;  // SCALAR: float bits in the low word; row modes: see above (without bit 63)
+};
+
+struct DevState {
+  unsigned long long count;            // keys held (slot array plus the side slot)
+  unsigned long long arena_top;        // FIXED: rows handed out; VARLEN: 16-byte units handed out
+  unsigned long long special_payload;  // payload of key 2^64-1
+  unsigned long long scan_total;       // grand total of the last lens scan
+  unsigned int special_present;
+  unsigned int error;                  // sticky error bits of finished requests
+  unsigned int req_error;              // error bits of the request in flight
+  unsigned int misaligned;             // OR of (len & 3) over the lens of the current request
+};
+
+// murmur3 finaliser: full avalanche, so evenly spaced keys (kMaxKey/n*i) spread out
+__device__ __forceinline__ uint64_t mix64(uint64_t x) {
+  x ^= x >> 33;
+  x *= 0xff51afd7ed558ccdull;
+  x ^= x >> 33;
+  x *= 0xc4ceb9fe1a85ec53ull;
+  x ^= x >> 33;
+  return x;
+}
+
+__device__ __forceinline__ unsigned wave_sum_u32(unsigned x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+  return x;
+}
+
+// Inclusive prefix sum over the 64 lanes of a wavefront. Every lane must call it.
+__device__ __forceinline__ unsigned long long wave_incl_scan_u64(unsigned long long x) {
+  const unsigned lane = __lane_id();
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    unsigned long long y = __shfl_up(x, d);
+    if (lane >= (unsigned)d) x += y;
+  }
+  return x;
+}
+
+// Finds `key` or claims an empty slot for it. Returns the address of the slot's
+// payload (nullptr if the table has no free slot, which the host-side sizing
+// rules out). `seen` is the payload read together with the key when the key was
+// already present.
+__device__ __forceinline__ uint64_t* find_or_insert(Slot* __restrict__ slots, uint64_t mask,
+                                                    DevState* st, uint64_t key, bool& is_new,
+                                                    uint64_t& seen) {
+  is_new = false;
+  seen = 0;
+  if (key == kEmptyKey) {
+    is_new = atomicExch(&st->special_present, 1u) == 0u;
+    seen = st->special_payload;
+    return reinterpret_cast<uint64_t*>(&st->special_payload);
+  }
+  uint64_t h = mix64(key) & mask;
+  for (uint64_t probes = 0; probes <= mask; ++probes) {
+    const ulonglong2 s = *reinterpret_cast<const ulonglong2*>(&slots[h]);
+    if (s.x == key) {
+      seen = s.y;
+      return &slots[h].payload;
+    }
+    if (s.x == kEmptyKey) {
+      unsigned long long old = atomicCAS(reinterpret_cast<unsigned long long*>(&slots[h].key),
+                                         (unsigned long long)kEmptyKey, (unsigned long long)key);
+      if (old == kEmptyKey) {
+        is_new = true;
+        return &slots[h].payload;
+      }
+      if (old == key) {  // same key twice in one request: undefined for callers, but stay sane
+        seen = slots[h].payload;
+        return &slots[h].payload;
+      }
+    }
+    h = (h + 1) & mask;
+  }
+  atomicOr(&st->error, kDevErrFull);
+  return nullptr;
+}
+
+// Lookup without insertion. Returns false when the key is absent.
+__device__ __forceinline__ bool find_only(const Slot* __restrict__ slots, uint64_t mask,
+                                          const DevState* st, uint64_t key, uint64_t& payload) {
+  if (key == kEmptyKey) {
+    payload = st->special_payload;
+    return st->special_present != 0u;
+  }
+  uint64_t h = mix64(key) & mask;
+  for (uint64_t probes = 0; probes <= mask; ++probes) {
+    const ulonglong2 s = *reinterpret_cast<const ulonglong2*>(&slots[h]);
+    if (s.x == key) {
+      payload = s.y;
+      return true;
+    }
+    if (s.x == kEmptyKey) return false;
+    h = (h + 1) & mask;
+  }
+  return false;
+}
+
+}  // namespace pskv
+#endif  // PSKV_DEVICE_COMMON_H_

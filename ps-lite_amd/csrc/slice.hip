@@ -1,0 +1,407 @@
+// Worker-side kernels: the key-range slicer that replaces KVWorker::DefaultSlicer
+// (include/ps/kv_app.h:517-572) and the device-side reassembly of pulled slices
+// that mirrors the callback of KVWorker::AddPullCB (kv_app.h:663-714).
+#include <algorithm>
+#include <limits>
+#include <mutex>
+#include <numeric>
+#include <vector>
+
+#include "device_common.h"
+#include "host_common.h"
+
+namespace pskv {
+namespace {
+
+// One wavefront per search target: a 64-ary lower_bound. Each round the 64 lanes probe
+// evenly spaced keys of the remaining interval, a ballot counts how many are below
+// the target (the probes are sorted, so the votes are a prefix of ones) and the
+// interval shrinks 64-fold: ceil(log64 n) dependent loads instead of ceil(log2 n).
+__global__ __launch_bounds__(kBlock) void k_bounds(const uint64_t* __restrict__ keys, uint64_t n,
+                                                  const uint64_t* __restrict__ targets,
+                                                  uint64_t ntargets, uint64_t* __restrict__ lb) {
+  const uint64_t w = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
+  const unsigned lane = threadIdx.x & 63;
+  if (w >= ntargets) return;  // whole wavefronts leave together
+  const uint64_t target = targets[w];
+  uint64_t lo = 0, hi = n;  // the answer lies in [lo, hi]; keys[lo..hi) are undecided
+  while (hi > lo) {
+    const uint64_t len = hi - lo;
+    if (len <= 64) {
+      const bool below = lane < len && keys[lo + lane] < target;
+      lo += __popcll(__ballot(below));
+      break;
+    }
+    const uint64_t step = (len + 63) / 64;
+    const uint64_t idx = lo + (uint64_t)(lane + 1) * step - 1;
+    const bool below = idx < hi && keys[idx] < target;
+    const uint64_t c = __popcll(__ballot(below));
+    // probes 0..c-1 are below the target, probe c (if any) is not
+    const uint64_t new_lo = lo + c * step;
+    const uint64_t cap = lo + (c + 1) * step - 1;
+    hi = cap < hi ? cap : hi;
+    lo = new_lo < hi ? new_lo : hi;
+  }
+  if (lane == 0) lb[w] = lo;
+}
+
+// kv_app.h:528-541: pos[0] = lower_bound(keys, ranges[0].begin); every further
+// boundary is searched in the suffix that starts at the previous one, which for
+// sorted keys is max(previous, lower_bound over the whole array).
+__global__ void k_bounds_chain(const uint64_t* __restrict__ lb, uint64_t S,
+                               uint64_t* __restrict__ pos) {
+  if (blockIdx.x != 0 || threadIdx.x != 0) return;
+  uint64_t p = lb[0];
+  pos[0] = p;
+  for (uint64_t i = 0; i < S; ++i) {
+    const uint64_t e = lb[i + 1];
+    p = e > p ? e : p;
+    pos[i + 1] = p;
+  }
+}
+
+// kv_app.h:565 `for (int l : kv.lens) val_end += l;` for every slice at once:
+// blockIdx.y is the slice, the workgroups of a slice stride over its lens.
+// Sums are taken modulo 2^64 over sign-extended lens, like size_t += int.
+__global__ __launch_bounds__(kBlock) void k_segment_sums(const int32_t* __restrict__ lens,
+                                                        const uint64_t* __restrict__ pos,
+                                                        unsigned long long* __restrict__ sums) {
+  __shared__ unsigned long long red[kBlock / 64];
+  const uint64_t begin = pos[blockIdx.y], end = pos[blockIdx.y + 1];
+  unsigned long long s = 0;
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t i = begin + (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < end; i += stride)
+    s += (unsigned long long)(long long)lens[i];
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long t = 0;
+    for (int w = 0; w < kBlock / 64; ++w) t += red[w];
+    if (t) atomicAdd(&sums[blockIdx.y], t);
+  }
+}
+
+// First key and last key + 1 of every response (FindRange arguments, kv_app.h:671).
+__global__ void k_response_ends(const uint64_t* const* __restrict__ resp_keys,
+                                const uint64_t* __restrict__ resp_nkeys, uint64_t R,
+                                uint64_t* __restrict__ targets) {
+  const uint64_t r = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= R) return;
+  targets[2 * r] = resp_keys[r][0];
+  targets[2 * r + 1] = resp_keys[r][resp_nkeys[r] - 1] + 1;  // wraps to 0 for kMaxKey, as Key does
+}
+
+// Per-call state of the slicer. Calls may come from any thread at once
+// (KVWorker::Push is thread-safe, kv_app.h:101-104), so each call takes a context
+// of its own from a pool and returns it afterwards.
+struct SliceCtx {
+  int device = -1;
+  hipStream_t stream = nullptr;
+  void* dev = nullptr;      // device scratch: targets, lower bounds, positions, sums
+  size_t dev_bytes = 0;
+  void* pinned = nullptr;   // host-visible copy of the small arrays
+  size_t pinned_bytes = 0;
+  void* stage = nullptr;    // device copy of host-resident keys / lens
+  size_t stage_bytes = 0;
+};
+
+std::mutex g_pool_mu;
+std::vector<SliceCtx*> g_pool;
+
+SliceCtx* take_ctx(int device) {
+  {
+    std::lock_guard<std::mutex> lk(g_pool_mu);
+    for (size_t i = 0; i < g_pool.size(); ++i) {
+      if (g_pool[i]->device == device) {
+        SliceCtx* c = g_pool[i];
+        g_pool.erase(g_pool.begin() + i);
+        return c;
+      }
+    }
+  }
+  SliceCtx* c = new (std::nothrow) SliceCtx();
+  if (!c) return nullptr;
+  c->device = device;
+  if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
+    delete c;
+    return nullptr;
+  }
+  return c;
+}
+
+void give_ctx(SliceCtx* c) {
+  std::lock_guard<std::mutex> lk(g_pool_mu);
+  g_pool.push_back(c);
+}
+
+struct CtxLease {
+  SliceCtx* c;
+  explicit CtxLease(int device) : c(take_ctx(device)) {}
+  ~CtxLease() {
+    if (c) give_ctx(c);
+  }
+};
+
+int ctx_reserve(SliceCtx* c, size_t dev_bytes, size_t pinned_bytes, size_t stage_bytes) {
+  if (dev_bytes > c->dev_bytes) {
+    if (c->dev) PSKV_HIP(hipFree(c->dev));
+    c->dev = nullptr;
+    c->dev_bytes = 0;
+    PSKV_HIP(hipMalloc(&c->dev, dev_bytes));
+    c->dev_bytes = dev_bytes;
+  }
+  if (pinned_bytes > c->pinned_bytes) {
+    if (c->pinned) PSKV_HIP(hipHostFree(c->pinned));
+    c->pinned = nullptr;
+    c->pinned_bytes = 0;
+    PSKV_HIP(hipHostMalloc(&c->pinned, pinned_bytes, hipHostMallocDefault));
+    c->pinned_bytes = pinned_bytes;
+  }
+  if (stage_bytes > c->stage_bytes) {
+    if (c->stage) PSKV_HIP(hipFree(c->stage));
+    c->stage = nullptr;
+    c->stage_bytes = 0;
+    PSKV_HIP(hipMalloc(&c->stage, stage_bytes));
+    c->stage_bytes = stage_bytes;
+  }
+  return PSKV_OK;
+}
+
+inline size_t pad256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+int launch_bounds_search(const uint64_t* keys, uint64_t n, const uint64_t* targets, uint64_t nt,
+                         uint64_t* lb, hipStream_t stream) {
+  const unsigned blocks = (unsigned)((nt * 64 + kBlock - 1) / kBlock);
+  k_bounds<<<dim3(blocks), dim3(kBlock), 0, stream>>>(keys, n, targets, nt, lb);
+  PSKV_HIP(hipGetLastError());
+  return PSKV_OK;
+}
+
+}  // namespace
+}  // namespace pskv
+
+using namespace pskv;
+
+extern "C" {
+
+int pskv_server_ranges(uint64_t num_servers, uint64_t* range_begin, uint64_t* range_end) {
+  clear_error();
+  if (num_servers == 0 || !range_begin || !range_end)
+    return set_error(PSKV_EINVAL, "need at least one server and two output arrays");
+  const uint64_t max_key = std::numeric_limits<uint64_t>::max();  // ps::kMaxKey, base.h:18
+  for (uint64_t i = 0; i < num_servers; ++i) {
+    range_begin[i] = max_key / num_servers * i;        // postoffice.cc:174
+    range_end[i] = max_key / num_servers * (i + 1);    // postoffice.cc:175
+  }
+  return PSKV_OK;
+}
+
+int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, size_t nlens,
+               size_t nvals, const uint64_t* range_begin, const uint64_t* range_end, size_t S,
+               uint64_t* pos, uint64_t* val_pos, uint8_t* used, int memkind) {
+  clear_error();
+  if (memkind != PSKV_MEM_HOST && memkind != PSKV_MEM_DEVICE)
+    return set_error(PSKV_EINVAL, "bad memkind %d", memkind);
+  if (!pos || !val_pos || (S && (!used || !range_begin || !range_end)))
+    return set_error(PSKV_EINVAL, "null argument");
+  if (n && !keys) return set_error(PSKV_EINVAL, "null keys");
+  for (size_t i = 0; i <= S; ++i) pos[i] = val_pos[i] = 0;
+  for (size_t i = 0; i < S; ++i) used[i] = 0;
+  // kv_app.h:533 CHECK_EQ(ranges[i-1].end(), ranges[i].begin()); it fires inside the
+  // loop, before the coverage check of :542
+  for (size_t i = 1; i < S; ++i) {
+    if (range_end[i - 1] != range_begin[i])
+      return set_error(PSKV_ERANGE_GAP, "ranges[%zu].end != ranges[%zu].begin", i - 1, i);
+  }
+  if (S == 0) {
+    if (n) return set_error(PSKV_EUNCOVERED_KEY, "no ranges for %zu keys", n);
+    return PSKV_OK;
+  }
+  const bool has_lens = lens != nullptr && nlens != 0;
+
+  if (n) {
+    DeviceGuard guard(device);
+    if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", device);
+    CtxLease lease(device);
+    SliceCtx* c = lease.c;
+    if (!c) return set_error(PSKV_EHIP, "cannot create a slicer context on device %d", device);
+    const bool do_sums = has_lens && nlens == n;
+    // small arrays: targets[S+1] | lb[S+1] | pos[S+1] | sums[S]
+    const size_t small = 4 * pad256((S + 1) * 8);
+    const bool host = memkind == PSKV_MEM_HOST;
+    const size_t stage_need = host ? pad256(n * 8) + (do_sums ? pad256(n * 4) : 0) : 0;
+    int rc = ctx_reserve(c, small, small, stage_need);
+    if (rc) return rc;
+    char* d = static_cast<char*>(c->dev);
+    uint64_t* d_targets = reinterpret_cast<uint64_t*>(d);
+    uint64_t* d_lb = reinterpret_cast<uint64_t*>(d + pad256((S + 1) * 8));
+    uint64_t* d_pos = reinterpret_cast<uint64_t*>(d + 2 * pad256((S + 1) * 8));
+    unsigned long long* d_sums = reinterpret_cast<unsigned long long*>(d + 3 * pad256((S + 1) * 8));
+    char* h = static_cast<char*>(c->pinned);
+    uint64_t* h_targets = reinterpret_cast<uint64_t*>(h);
+    uint64_t* h_pos = reinterpret_cast<uint64_t*>(h + 2 * pad256((S + 1) * 8));
+    unsigned long long* h_sums = reinterpret_cast<unsigned long long*>(h + 3 * pad256((S + 1) * 8));
+
+    const uint64_t* d_keys = keys;
+    const int32_t* d_lens = lens;
+    if (host) {
+      uint64_t* sk = static_cast<uint64_t*>(c->stage);
+      PSKV_HIP(hipMemcpyAsync(sk, keys, n * 8, hipMemcpyHostToDevice, c->stream));
+      d_keys = sk;
+      if (do_sums) {
+        int32_t* sl = reinterpret_cast<int32_t*>(static_cast<char*>(c->stage) + pad256(n * 8));
+        PSKV_HIP(hipMemcpyAsync(sl, lens, n * 4, hipMemcpyHostToDevice, c->stream));
+        d_lens = sl;
+      }
+    }
+    h_targets[0] = range_begin[0];
+    for (size_t i = 0; i < S; ++i) h_targets[i + 1] = range_end[i];
+    PSKV_HIP(hipMemcpyAsync(d_targets, h_targets, (S + 1) * 8, hipMemcpyHostToDevice, c->stream));
+    rc = launch_bounds_search(d_keys, n, d_targets, S + 1, d_lb, c->stream);
+    if (rc) return rc;
+    k_bounds_chain<<<dim3(1), dim3(64), 0, c->stream>>>(d_lb, S, d_pos);
+    PSKV_HIP(hipGetLastError());
+    if (do_sums) {
+      if (S > 65535) return set_error(PSKV_EINVAL, "more than 65535 ranges with lens");
+      PSKV_HIP(hipMemsetAsync(d_sums, 0, S * 8, c->stream));
+      uint64_t per = n / S / (kBlock * 8) + 1;
+      if (per > 1024) per = 1024;
+      k_segment_sums<<<dim3((unsigned)per, (unsigned)S), dim3(kBlock), 0, c->stream>>>(d_lens, d_pos,
+                                                                                      d_sums);
+      PSKV_HIP(hipGetLastError());
+      PSKV_HIP(hipMemcpyAsync(h_sums, d_sums, S * 8, hipMemcpyDeviceToHost, c->stream));
+    }
+    PSKV_HIP(hipMemcpyAsync(h_pos, d_pos, (S + 1) * 8, hipMemcpyDeviceToHost, c->stream));
+    PSKV_HIP(hipStreamSynchronize(c->stream));
+    for (size_t i = 0; i <= S; ++i) pos[i] = h_pos[i];
+    if (do_sums)
+      for (size_t i = 0; i < S; ++i) val_pos[i + 1] = h_sums[i];  // per-slice sums for now
+  }
+
+  for (size_t i = 0; i < S; ++i) used[i] = pos[i + 1] != pos[i];  // kv_app.h:540
+  if (pos[S] != n)  // kv_app.h:542
+    return set_error(PSKV_EUNCOVERED_KEY,
+                     "Check failed: (pos[n]) == (send.keys.size()): %llu keys fall in the ranges, "
+                     "%zu were given", (unsigned long long)pos[S], n);
+  if (n == 0) return PSKV_OK;  // kv_app.h:543
+
+  if (!has_lens) {
+    const size_t k = nvals / n;  // kv_app.h:548
+    if (k * n != nvals)          // kv_app.h:549
+      return set_error(PSKV_ESIZE_MISMATCH, "%zu values do not divide over %zu keys", nvals, n);
+    for (size_t i = 0; i <= S; ++i) val_pos[i] = pos[i] * k;  // kv_app.h:569
+    return PSKV_OK;
+  }
+  if (nlens != n)  // kv_app.h:551
+    return set_error(PSKV_ESIZE_MISMATCH, "%zu keys but %zu lens", n, nlens);
+  // kv_app.h:563-567 with the CHECKs of SArray::segment (sarray.h:249)
+  uint64_t val_begin = 0, val_end = 0;
+  for (size_t i = 0; i < S; ++i) {
+    const uint64_t sum = val_pos[i + 1];
+    val_pos[i] = val_begin;
+    if (pos[i + 1] != pos[i]) {
+      val_end += sum;
+      if (val_end < val_begin || val_end > nvals) {
+        val_pos[i + 1] = val_end;
+        return set_error(PSKV_ESIZE_MISMATCH, "lens of slice %zu reach past the %zu values", i, nvals);
+      }
+      val_begin = val_end;
+    }
+    val_pos[i + 1] = val_end;
+  }
+  return PSKV_OK;
+}
+
+int pskv_assemble_pull(int device, const uint64_t* req_keys, size_t n, size_t R,
+                       const uint64_t* const* resp_keys, const size_t* resp_nkeys,
+                       const float* const* resp_vals, const size_t* resp_nvals,
+                       const int32_t* const* resp_lens, float* out, size_t out_cap,
+                       int32_t* out_lens, size_t* out_nvals, int memkind) {
+  clear_error();
+  if (memkind != PSKV_MEM_DEVICE)
+    return set_error(PSKV_EINVAL,
+                     "pskv_assemble_pull concatenates device-resident slices; host-resident "
+                     "slices are reassembled by KVWorker itself");
+  if (out_nvals) *out_nvals = 0;
+  if (R && (!resp_keys || !resp_nkeys || !resp_vals || !resp_nvals))
+    return set_error(PSKV_EINVAL, "null argument");
+  size_t total_key = 0, total_val = 0;
+  for (size_t r = 0; r < R; ++r) {
+    if (resp_nkeys[r] == 0)  // front()/back() CHECK(!empty()), sarray.h:221-222
+      return set_error(PSKV_EINVAL, "response %zu has no keys", r);
+    total_key += resp_nkeys[r];
+    total_val += resp_nvals[r];
+  }
+  std::vector<uint64_t> ends(2 * R);
+  if (R) {
+    DeviceGuard guard(device);
+    if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", device);
+    CtxLease lease(device);
+    SliceCtx* c = lease.c;
+    if (!c) return set_error(PSKV_EHIP, "cannot create a context on device %d", device);
+    // device scratch: key pointers[R] | nkeys[R] | targets[2R] | lb[2R]
+    const size_t a = pad256(R * 8), b = pad256(2 * R * 8);
+    int rc = ctx_reserve(c, 2 * a + 2 * b, 2 * a + 2 * b, 0);
+    if (rc) return rc;
+    char* d = static_cast<char*>(c->dev);
+    char* h = static_cast<char*>(c->pinned);
+    const uint64_t** d_ptrs = reinterpret_cast<const uint64_t**>(d);
+    uint64_t* d_nk = reinterpret_cast<uint64_t*>(d + a);
+    uint64_t* d_targets = reinterpret_cast<uint64_t*>(d + 2 * a);
+    uint64_t* d_lb = reinterpret_cast<uint64_t*>(d + 2 * a + b);
+    const uint64_t** h_ptrs = reinterpret_cast<const uint64_t**>(h);
+    uint64_t* h_nk = reinterpret_cast<uint64_t*>(h + a);
+    uint64_t* h_targets = reinterpret_cast<uint64_t*>(h + 2 * a);
+    uint64_t* h_lb = reinterpret_cast<uint64_t*>(h + 2 * a + b);
+    for (size_t r = 0; r < R; ++r) {
+      h_ptrs[r] = resp_keys[r];
+      h_nk[r] = resp_nkeys[r];
+    }
+    PSKV_HIP(hipMemcpyAsync(d, h, 2 * a, hipMemcpyHostToDevice, c->stream));
+    k_response_ends<<<dim3((unsigned)((R + 63) / 64)), dim3(64), 0, c->stream>>>(d_ptrs, d_nk, R,
+                                                                                 d_targets);
+    PSKV_HIP(hipGetLastError());
+    rc = launch_bounds_search(req_keys, n, d_targets, 2 * R, d_lb, c->stream);
+    if (rc) return rc;
+    PSKV_HIP(hipMemcpyAsync(h_targets, d_targets, 2 * b, hipMemcpyDeviceToHost, c->stream));
+    PSKV_HIP(hipStreamSynchronize(c->stream));
+    for (size_t r = 0; r < R; ++r) {  // kv_app.h:670-677
+      const uint64_t lower = h_targets[2 * r], upper = h_targets[2 * r + 1];
+      const uint64_t size = upper <= lower ? 0 : h_lb[2 * r + 1] - h_lb[2 * r];  // sarray.h:283
+      if (size != resp_nkeys[r])
+        return set_error(PSKV_ESIZE_MISMATCH, "unmatched keys size from one server (response %zu)", r);
+      ends[2 * r] = lower;
+    }
+    if (total_key != n)  // kv_app.h:678
+      return set_error(PSKV_ESIZE_MISMATCH, "lost some servers? %zu of %zu keys answered", total_key, n);
+    if (out_nvals) *out_nvals = total_val;
+    if (total_val > out_cap)  // kv_app.h:686-690
+      return set_error(PSKV_ESIZE_MISMATCH, "response needs %zu floats, buffer holds %zu", total_val,
+                       out_cap);
+    std::vector<size_t> order(R);
+    std::iota(order.begin(), order.end(), (size_t)0);
+    std::sort(order.begin(), order.end(),  // kv_app.h:681-684
+              [&](size_t x, size_t y) { return ends[2 * x] < ends[2 * y]; });
+    size_t voff = 0, koff = 0;
+    for (size_t i = 0; i < R; ++i) {  // kv_app.h:701-708
+      const size_t r = order[i];
+      if (resp_nvals[r])
+        PSKV_HIP(hipMemcpyAsync(out + voff, resp_vals[r], resp_nvals[r] * sizeof(float),
+                                hipMemcpyDeviceToDevice, c->stream));
+      voff += resp_nvals[r];
+      if (out_lens && resp_lens)
+        PSKV_HIP(hipMemcpyAsync(out_lens + koff, resp_lens[r], resp_nkeys[r] * sizeof(int32_t),
+                                hipMemcpyDeviceToDevice, c->stream));
+      koff += resp_nkeys[r];
+    }
+    PSKV_HIP(hipStreamSynchronize(c->stream));
+    return PSKV_OK;
+  }
+  if (total_key != n)
+    return set_error(PSKV_ESIZE_MISMATCH, "lost some servers? %zu of %zu keys answered", total_key, n);
+  return PSKV_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,827 @@
+// Host side of the HBM-resident key-value store: owns the slot array, the row
+// arena and the per-request workspace, sizes them, and enqueues the kernels of
+// table_kernels.h in request order on one stream. This is what a ps-lite server
+// calls in place of KVServerDefaultHandle (include/ps/kv_app.h:440-463).
+#include <algorithm>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "host_common.h"
+#include "scan.h"
+#include "table_kernels.h"
+
+namespace pskv {
+
+static thread_local std::string g_last_error;
+
+int set_error(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+void clear_error() { g_last_error.clear(); }
+
+namespace {
+
+constexpr uint64_t kDefaultCapacity = 1u << 20;
+constexpr uint64_t kMinSlots = 1024;
+constexpr unsigned kMaxGrid = 1u << 20;
+
+// A device buffer that only grows. Contents are not kept across growth.
+struct GrowBuf {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+};
+
+struct EventPair {
+  hipEvent_t a, b;
+};
+
+}  // namespace
+}  // namespace pskv
+
+using namespace pskv;
+
+struct pskv_table {
+  int device = 0;
+  int mode = PSKV_MODE_SCALAR;
+  hipStream_t stream = nullptr;
+  bool own_stream = false;
+  float max_load = 0.5f;
+
+  Slot* slots = nullptr;
+  uint64_t cap = 0;        // slots, a power of two
+  uint64_t count_ub = 0;   // upper bound of DevState::count kept on the host
+  DevState* st = nullptr;  // device
+  DevState* st_host = nullptr;  // pinned mirror for read-backs
+
+  // row modes
+  float* arena = nullptr;
+  uint64_t arena_cap = 0;  // floats
+  uint64_t top_ub = 0;     // upper bound of DevState::arena_top (rows or 16-byte units)
+  uint64_t row_len = 0;    // FIXED
+
+  GrowBuf ws;         // per-request workspace (row references, offsets)
+  GrowBuf tiles;      // VARLEN: first key of every request-side tile
+  GrowBuf stage;      // device copies of host-resident request buffers
+  GrowBuf stage_out;  // device-side response of a host-resident or undersized pull
+  bool no_growth = false;  // set while dumping: every key is known to be present
+
+  bool prof = false;
+  std::vector<EventPair> pending[PSKV_KERNEL_COUNT];
+  std::vector<EventPair> free_events;
+  uint64_t launches[PSKV_KERNEL_COUNT] = {0};
+  double total_ms[PSKV_KERNEL_COUNT] = {0};
+};
+
+namespace {
+
+// ---- profiling -------------------------------------------------------------------
+struct ProfScope {
+  pskv_table* t;
+  int kernel;
+  EventPair ev;
+  bool on;
+  ProfScope(pskv_table* t_, int kernel_) : t(t_), kernel(kernel_), on(t_->prof) {
+    if (!on) return;
+    if (!t->free_events.empty()) {
+      ev = t->free_events.back();
+      t->free_events.pop_back();
+    } else if (hipEventCreate(&ev.a) != hipSuccess || hipEventCreate(&ev.b) != hipSuccess) {
+      on = false;
+      return;
+    }
+    (void)hipEventRecord(ev.a, t->stream);
+  }
+  ~ProfScope() {
+    if (!on) return;
+    (void)hipEventRecord(ev.b, t->stream);
+    t->pending[kernel].push_back(ev);
+  }
+};
+
+int prof_collect(pskv_table* t) {
+  PSKV_HIP(hipStreamSynchronize(t->stream));
+  for (int k = 0; k < PSKV_KERNEL_COUNT; ++k) {
+    for (const EventPair& ev : t->pending[k]) {
+      float ms = 0.f;
+      if (hipEventElapsedTime(&ms, ev.a, ev.b) == hipSuccess) {
+        t->total_ms[k] += ms;
+        t->launches[k] += 1;
+      }
+      t->free_events.push_back(ev);
+    }
+    t->pending[k].clear();
+  }
+  return PSKV_OK;
+}
+
+// ---- memory ----------------------------------------------------------------------
+int grow(pskv_table* t, GrowBuf* b, size_t bytes) {
+  if (bytes <= b->bytes) return PSKV_OK;
+  size_t want = std::max(bytes, b->bytes + b->bytes / 2);
+  want = (want + 255) & ~(size_t)255;
+  if (b->ptr) {
+    // earlier requests on the stream may still read the old buffer
+    PSKV_HIP(hipStreamSynchronize(t->stream));
+    PSKV_HIP(hipFree(b->ptr));
+    b->ptr = nullptr;
+    b->bytes = 0;
+  }
+  PSKV_HIP(hipMalloc(&b->ptr, want));
+  b->bytes = want;
+  return PSKV_OK;
+}
+
+// Carves aligned pieces out of a GrowBuf that was grown to the total beforehand.
+struct Carver {
+  char* base;
+  size_t at = 0;
+  explicit Carver(void* p) : base(static_cast<char*>(p)) {}
+  template <typename T>
+  T* take(size_t count) {
+    T* r = reinterpret_cast<T*>(base + at);
+    at += (count * sizeof(T) + 255) & ~(size_t)255;
+    return r;
+  }
+  static size_t need(size_t count, size_t elem) { return (count * elem + 255) & ~(size_t)255; }
+};
+
+int read_state(pskv_table* t) {
+  PSKV_HIP(hipMemcpyAsync(t->st_host, t->st, sizeof(DevState), hipMemcpyDeviceToHost, t->stream));
+  PSKV_HIP(hipStreamSynchronize(t->stream));
+  return PSKV_OK;
+}
+
+// Turns device error bits into a status, clearing them on the device.
+int report_device_errors(pskv_table* t) {
+  const unsigned bits = t->st_host->error | t->st_host->req_error;
+  if (!bits) return PSKV_OK;
+  PSKV_HIP(hipMemsetAsync(&t->st->error, 0, 2 * sizeof(unsigned), t->stream));
+  PSKV_HIP(hipStreamSynchronize(t->stream));
+  if (bits & kDevErrFull) return set_error(PSKV_ENOMEM, "slot array full (internal sizing error)");
+  if (bits & kDevErrBadLen)
+    return set_error(PSKV_EINVAL, "a length is negative or above PSKV_MAX_VARLEN_ROW");
+  if (bits & kDevErrSizeMismatch)
+    return set_error(PSKV_ESIZE_MISMATCH, "lens do not add up to the number of values");
+  return set_error(PSKV_ELEN_CHANGED, "a pushed row length differs from the stored length");
+}
+
+int alloc_slots(uint64_t cap, Slot** out, hipStream_t stream) {
+  PSKV_HIP(hipMalloc(reinterpret_cast<void**>(out), cap * sizeof(Slot)));
+  // all-ones bytes: key = empty marker
+  PSKV_HIP(hipMemsetAsync(*out, 0xFF, cap * sizeof(Slot), stream));
+  return PSKV_OK;
+}
+
+// Makes room for `n` more keys (every key of a request may be new).
+int ensure_slots(pskv_table* t, uint64_t n) {
+  if (t->no_growth) return PSKV_OK;
+  const double limit = (double)t->max_load * (double)t->cap;
+  if ((double)(t->count_ub + n) <= limit) {
+    t->count_ub += n;
+    return PSKV_OK;
+  }
+  int rc = read_state(t);
+  if (rc) return rc;
+  t->count_ub = t->st_host->count;
+  if (t->mode != PSKV_MODE_SCALAR) {
+    t->top_ub = t->st_host->arena_top;
+  }
+  if ((double)(t->count_ub + n) > limit) {
+    uint64_t want = next_pow2((uint64_t)((double)(t->count_ub + n) / t->max_load) + 1);
+    want = std::max(want, t->cap * 2);
+    Slot* fresh = nullptr;
+    rc = alloc_slots(want, &fresh, t->stream);
+    if (rc) return rc;
+    {
+      ProfScope ps(t, PSKV_KERNEL_REHASH);
+      k_rehash<<<dim3(grid_for(t->cap, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(
+          t->slots, t->cap, fresh, want - 1, t->st);
+    }
+    PSKV_HIP(hipGetLastError());
+    PSKV_HIP(hipStreamSynchronize(t->stream));
+    PSKV_HIP(hipFree(t->slots));
+    t->slots = fresh;
+    t->cap = want;
+  }
+  t->count_ub += n;
+  return PSKV_OK;
+}
+
+// Makes room in the arena. `units` is in the arena's allocation unit (rows for FIXED,
+// 16 bytes for VARLEN); `floats_per_unit` converts to floats.
+int ensure_arena(pskv_table* t, uint64_t units, uint64_t floats_per_unit) {
+  if (t->no_growth) return PSKV_OK;
+  if ((t->top_ub + units) * floats_per_unit <= t->arena_cap) {
+    t->top_ub += units;
+    return PSKV_OK;
+  }
+  int rc = read_state(t);
+  if (rc) return rc;
+  t->top_ub = t->st_host->arena_top;
+  const uint64_t need = (t->top_ub + units) * floats_per_unit;
+  if (need > t->arena_cap) {
+    uint64_t want = std::max(need, t->arena_cap + t->arena_cap / 2);
+    want = (want + 1023) & ~(uint64_t)1023;
+    float* fresh = nullptr;
+    PSKV_HIP(hipMalloc(reinterpret_cast<void**>(&fresh), want * sizeof(float)));
+    const uint64_t live = t->top_ub * floats_per_unit;
+    if (live && t->arena) {
+      PSKV_HIP(hipMemcpyAsync(fresh, t->arena, live * sizeof(float), hipMemcpyDeviceToDevice,
+                              t->stream));
+    }
+    PSKV_HIP(hipStreamSynchronize(t->stream));
+    if (t->arena) PSKV_HIP(hipFree(t->arena));
+    t->arena = fresh;
+    t->arena_cap = want;
+  }
+  t->top_ub += units;
+  return PSKV_OK;
+}
+
+// ---- request pipeline ------------------------------------------------------------
+struct Request {
+  bool push, pull;
+  const uint64_t* keys;  // device
+  uint64_t n;
+  const float* vals;     // device
+  uint64_t nvals;
+  const int32_t* lens;   // device
+  float* out;            // device
+  uint64_t out_cap;
+  int32_t* out_lens;     // device (VARLEN pull)
+  uint64_t out_nvals;    // result
+  bool lazy_out;         // VARLEN pull into host memory: `out` is allocated once the size is known
+};
+
+int run_scalar(pskv_table* t, Request& r) {
+  r.out_nvals = r.pull ? r.n : 0;
+  if (r.n == 0) return PSKV_OK;
+  int rc = ensure_slots(t, r.n);
+  if (rc) return rc;
+  const dim3 grid(grid_for(r.n, kBlock, kMaxGrid)), block(kBlock);
+  const uint64_t mask = t->cap - 1;
+  if (r.push && r.pull) {
+    ProfScope ps(t, PSKV_KERNEL_PUSH_SCALAR);
+    k_scalar<true, true><<<grid, block, 0, t->stream>>>(t->slots, mask, t->st, r.keys, r.vals,
+                                                        r.out, r.n);
+  } else if (r.push) {
+    ProfScope ps(t, PSKV_KERNEL_PUSH_SCALAR);
+    k_scalar<true, false><<<grid, block, 0, t->stream>>>(t->slots, mask, t->st, r.keys, r.vals,
+                                                         nullptr, r.n);
+  } else {
+    ProfScope ps(t, PSKV_KERNEL_PULL_SCALAR);
+    k_scalar<false, true><<<grid, block, 0, t->stream>>>(t->slots, mask, t->st, r.keys, nullptr,
+                                                         r.out, r.n);
+  }
+  PSKV_HIP(hipGetLastError());
+  return PSKV_OK;
+}
+
+template <bool VARLEN>
+int launch_rows(pskv_table* t, int op, const RowsParams& p) {
+  if (p.total == 0) return PSKV_OK;
+  const uint64_t ntiles = (p.total + kTileFloats - 1) / kTileFloats;
+  if (ntiles > 0x7fffffffull) return set_error(PSKV_EINVAL, "request too large");
+  ProfScope ps(t, op == kOpAcc ? PSKV_KERNEL_ROWS_ACC : PSKV_KERNEL_ROWS_GATHER);
+  if (op == kOpAcc) {
+    k_rows<kOpAcc, VARLEN><<<dim3((unsigned)ntiles), dim3(kBlock), 0, t->stream>>>(p);
+  } else {
+    k_rows<kOpGather, VARLEN><<<dim3((unsigned)ntiles), dim3(kBlock), 0, t->stream>>>(p);
+  }
+  PSKV_HIP(hipGetLastError());
+  return PSKV_OK;
+}
+
+int run_fixed(pskv_table* t, Request& r) {
+  const uint64_t k = t->row_len;
+  r.out_nvals = r.pull ? r.n * k : 0;
+  if (r.n == 0) return PSKV_OK;
+  int rc = ensure_slots(t, r.n);
+  if (rc) return rc;
+  rc = ensure_arena(t, r.n, k);
+  if (rc) return rc;
+  rc = grow(t, &t->ws, Carver::need(r.n, sizeof(uint64_t)));
+  if (rc) return rc;
+  Carver c(t->ws.ptr);
+  uint64_t* ref = c.take<uint64_t>(r.n);
+  {
+    ProfScope ps(t, PSKV_KERNEL_LOOKUP);
+    k_lookup_fixed<<<dim3(grid_for(r.n, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(
+        t->slots, t->cap - 1, t->st, r.keys, r.n, ref);
+  }
+  PSKV_HIP(hipGetLastError());
+  RowsParams p{};
+  p.arena = t->arena;
+  p.ref = ref;
+  p.st = t->st;
+  p.n = r.n;
+  p.total = r.n * k;
+  p.k = k;
+  if (r.push) {
+    p.req = const_cast<float*>(r.vals);
+    p.force_scalar = ((k & 3) || (reinterpret_cast<uintptr_t>(r.vals) & 15)) ? 1u : 0u;
+    p.ignore_new = 0;
+    rc = launch_rows<false>(t, kOpAcc, p);
+    if (rc) return rc;
+  }
+  if (r.pull) {
+    p.req = r.out;
+    p.force_scalar = ((k & 3) || (reinterpret_cast<uintptr_t>(r.out) & 15)) ? 1u : 0u;
+    p.ignore_new = r.push ? 1u : 0u;
+    rc = launch_rows<false>(t, kOpGather, p);
+    if (rc) return rc;
+  }
+  return PSKV_OK;
+}
+
+// Grows the tile table to `total` request-side floats and fills it.
+int make_tile_keys(pskv_table* t, const uint64_t* off, uint64_t n, uint64_t total,
+                   const uint32_t** tile_key) {
+  const uint64_t ntiles = (total + kTileFloats - 1) / kTileFloats;
+  int rc = grow(t, &t->tiles, (ntiles + 1) * sizeof(uint32_t));
+  if (rc) return rc;
+  uint32_t* tk = static_cast<uint32_t*>(t->tiles.ptr);
+  k_tile_keys<<<dim3(grid_for(n, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(off, n, tk, ntiles);
+  PSKV_HIP(hipGetLastError());
+  *tile_key = tk;
+  return PSKV_OK;
+}
+
+int run_varlen(pskv_table* t, Request& r) {
+  r.out_nvals = 0;
+  if (r.n == 0) return PSKV_OK;
+  if (r.n > 0xfffffffeull) return set_error(PSKV_EINVAL, "too many keys in one request");
+  const uint64_t nparts = scan_num_parts(r.n);
+  const size_t need = Carver::need(r.n, 8) + Carver::need(r.n + 1, 8) + Carver::need(nparts, 8) +
+                      Carver::need(r.n, 4);
+  int rc = grow(t, &t->ws, need);
+  if (rc) return rc;
+  Carver c(t->ws.ptr);
+  uint64_t* ref = c.take<uint64_t>(r.n);
+  uint64_t* off = c.take<uint64_t>(r.n + 1);
+  unsigned long long* part = c.take<unsigned long long>(nparts);
+  int32_t* tmp_lens = c.take<int32_t>(r.n);
+  const dim3 kgrid(grid_for(r.n, kBlock, kMaxGrid)), block(kBlock);
+
+  RowsParams p{};
+  p.ref = ref;
+  p.off = off;
+  p.st = t->st;
+  p.n = r.n;
+
+  if (r.push) {
+    rc = ensure_slots(t, r.n);
+    if (rc) return rc;
+    rc = ensure_arena(t, r.nvals / 4 + r.n, 4);
+    if (rc) return rc;
+    k_begin_request<<<dim3(1), dim3(1), 0, t->stream>>>(t->st);
+    PSKV_HIP(launch_lens_scan(r.lens, r.n, off, part, t->st, PSKV_MAX_VARLEN_ROW, t->stream));
+    {
+      ProfScope ps(t, PSKV_KERNEL_LOOKUP);
+      k_lookup_var_push<<<kgrid, block, 0, t->stream>>>(t->slots, t->cap - 1, t->st, r.keys,
+                                                       r.lens, r.n, r.nvals, ref);
+    }
+    PSKV_HIP(hipGetLastError());
+    if (r.nvals) {
+      rc = make_tile_keys(t, off, r.n, r.nvals, &p.tile_key);
+      if (rc) return rc;
+      p.req = const_cast<float*>(r.vals);
+      p.arena = t->arena;
+      p.total = r.nvals;
+      p.force_scalar = (reinterpret_cast<uintptr_t>(r.vals) & 15) ? 1u : 0u;
+      p.ignore_new = 0;
+      rc = launch_rows<true>(t, kOpAcc, p);
+      if (rc) return rc;
+    }
+  }
+  if (r.pull) {
+    int32_t* lens_out = r.out_lens ? r.out_lens : tmp_lens;
+    if (r.push) {
+      // a refused push must not be followed by its pull half
+      rc = read_state(t);
+      if (rc) return rc;
+      rc = report_device_errors(t);
+      if (rc) return rc;
+    }
+    {
+      ProfScope ps(t, PSKV_KERNEL_LOOKUP);
+      k_lookup_var_pull<<<kgrid, block, 0, t->stream>>>(t->slots, t->cap - 1, t->st, r.keys, r.n,
+                                                       ref, lens_out);
+    }
+    PSKV_HIP(hipGetLastError());
+    k_begin_request<<<dim3(1), dim3(1), 0, t->stream>>>(t->st);
+    PSKV_HIP(launch_lens_scan(lens_out, r.n, off, part, t->st, PSKV_MAX_VARLEN_ROW, t->stream));
+    rc = read_state(t);  // the response size is data dependent
+    if (rc) return rc;
+    const uint64_t total = t->st_host->scan_total;
+    r.out_nvals = total;
+    if (total > r.out_cap)
+      return set_error(PSKV_ESIZE_MISMATCH, "response needs %llu floats, buffer holds %llu",
+                       (unsigned long long)total, (unsigned long long)r.out_cap);
+    if (total) {
+      if (r.lazy_out) {
+        rc = grow(t, &t->stage_out, total * sizeof(float));
+        if (rc) return rc;
+        r.out = static_cast<float*>(t->stage_out.ptr);
+      }
+      if (!r.out) return set_error(PSKV_EINVAL, "null out");
+      rc = make_tile_keys(t, off, r.n, total, &p.tile_key);
+      if (rc) return rc;
+      p.req = r.out;
+      p.arena = t->arena;
+      p.total = total;
+      p.force_scalar = (reinterpret_cast<uintptr_t>(r.out) & 15) ? 1u : 0u;
+      p.ignore_new = 1;
+      rc = launch_rows<true>(t, kOpGather, p);
+      if (rc) return rc;
+    }
+  }
+  return PSKV_OK;
+}
+
+// Host-side checks that mirror the CHECKs of the reference and the frozen rules of
+// the row modes; nothing is enqueued when they fail.
+int validate(pskv_table* t, bool push, bool pull, uint64_t n, uint64_t nvals, const int32_t* lens,
+             uint64_t nlens, int memkind) {
+  switch (t->mode) {
+    case PSKV_MODE_SCALAR:
+      // kv_app.h:447 CHECK_EQ(n, req_data.vals.size()); with pull set the reference
+      // indexes vals[i] unchecked, which this library refuses when the sizes differ
+      if (push && n != nvals)
+        return set_error(PSKV_ESIZE_MISMATCH, "%llu keys but %llu values", (unsigned long long)n,
+                         (unsigned long long)nvals);
+      return PSKV_OK;
+    case PSKV_MODE_FIXED:
+      if (push) {
+        if (n == 0) {
+          if (nvals) return set_error(PSKV_ESIZE_MISMATCH, "values without keys");
+        } else {
+          const uint64_t k = nvals / n;  // kv_app.h:548-549
+          if (k * n != nvals || k == 0)
+            return set_error(PSKV_ESIZE_MISMATCH, "%llu values do not divide over %llu keys",
+                             (unsigned long long)nvals, (unsigned long long)n);
+          if (t->row_len == 0) t->row_len = k;
+          if (k != t->row_len)
+            return set_error(PSKV_ESIZE_MISMATCH, "row length %llu, table holds rows of %llu",
+                             (unsigned long long)k, (unsigned long long)t->row_len);
+        }
+      }
+      if (n && t->row_len == 0) return set_error(PSKV_EINVAL, "pull before the row length is known");
+      return PSKV_OK;
+    default:
+      if (push) {
+        if (nlens != n)  // kv_app.h:489,551
+          return set_error(PSKV_ESIZE_MISMATCH, "%llu keys but %llu lens", (unsigned long long)n,
+                           (unsigned long long)nlens);
+        if (n && !lens) return set_error(PSKV_EINVAL, "lens missing");
+        if (n == 0 && nvals) return set_error(PSKV_ESIZE_MISMATCH, "values without keys");
+        if (memkind == PSKV_MEM_HOST) {
+          uint64_t total = 0;
+          for (uint64_t i = 0; i < n; ++i) {
+            if (lens[i] < 0 || (uint32_t)lens[i] > PSKV_MAX_VARLEN_ROW)
+              return set_error(PSKV_EINVAL, "lens[%llu] = %d out of range", (unsigned long long)i,
+                               lens[i]);
+            total += (uint64_t)lens[i];
+          }
+          if (total != nvals)
+            return set_error(PSKV_ESIZE_MISMATCH, "lens add up to %llu, %llu values given",
+                             (unsigned long long)total, (unsigned long long)nvals);
+        }
+      }
+      return PSKV_OK;
+  }
+}
+
+int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n, const float* vals,
+            size_t nvals, const int32_t* lens, size_t nlens, float* out, size_t out_cap,
+            int32_t* out_lens, size_t* out_nvals, int memkind) {
+  clear_error();
+  if (!t) return set_error(PSKV_EINVAL, "null table");
+  if (memkind != PSKV_MEM_HOST && memkind != PSKV_MEM_DEVICE)
+    return set_error(PSKV_EINVAL, "bad memkind %d", memkind);
+  if (n && !keys) return set_error(PSKV_EINVAL, "null keys");
+  if (push && nvals && !vals) return set_error(PSKV_EINVAL, "null vals");
+  if (out_nvals) *out_nvals = 0;
+  DeviceGuard guard(t->device);
+  if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", t->device);
+  int rc = validate(t, push, pull, n, nvals, lens, nlens, memkind);
+  if (rc) return rc;
+  const bool host = memkind == PSKV_MEM_HOST;
+  const bool varlen = t->mode == PSKV_MODE_VARLEN;
+
+  // SCALAR and FIXED know the response size up front. A response that does not fit is
+  // still computed (into scratch) so that the store ends up as the reference's would:
+  // a pull creates absent keys (kv_app.h:457).
+  uint64_t fixed_out = 0;
+  if (pull && !varlen) fixed_out = t->mode == PSKV_MODE_SCALAR ? n : n * t->row_len;
+  const bool too_small = pull && !varlen && fixed_out > out_cap;
+  if (pull && !varlen && fixed_out && !too_small && !out) return set_error(PSKV_EINVAL, "null out");
+
+  Request r{};
+  r.push = push;
+  r.pull = pull;
+  r.n = n;
+  r.nvals = push ? nvals : 0;
+  r.out_cap = out_cap;
+  if (!host) {
+    r.keys = keys;
+    r.vals = vals;
+    r.lens = lens;
+    r.out = out;
+    r.out_lens = out_lens;
+  } else {
+    const bool want_lens = push && varlen;
+    const bool want_out_lens = pull && varlen;
+    const size_t need = Carver::need(n, 8) + Carver::need(r.nvals, 4) +
+                        Carver::need(want_lens ? n : 0, 4) + Carver::need(want_out_lens ? n : 0, 4);
+    rc = grow(t, &t->stage, need);
+    if (rc) return rc;
+    Carver c(t->stage.ptr);
+    uint64_t* dkeys = c.take<uint64_t>(n);
+    float* dvals = c.take<float>(r.nvals);
+    int32_t* dlens = c.take<int32_t>(want_lens ? n : 0);
+    int32_t* dout_lens = c.take<int32_t>(want_out_lens ? n : 0);
+    if (n) PSKV_HIP(hipMemcpyAsync(dkeys, keys, n * 8, hipMemcpyHostToDevice, t->stream));
+    if (r.nvals) PSKV_HIP(hipMemcpyAsync(dvals, vals, r.nvals * 4, hipMemcpyHostToDevice, t->stream));
+    if (want_lens && n) PSKV_HIP(hipMemcpyAsync(dlens, lens, n * 4, hipMemcpyHostToDevice, t->stream));
+    r.keys = dkeys;
+    r.vals = dvals;
+    r.lens = dlens;
+    r.out_lens = want_out_lens ? dout_lens : nullptr;
+    r.lazy_out = pull && varlen;
+  }
+  if (pull && !varlen && (host || too_small) && fixed_out) {
+    rc = grow(t, &t->stage_out, fixed_out * sizeof(float));
+    if (rc) return rc;
+    r.out = static_cast<float*>(t->stage_out.ptr);
+    r.out_cap = fixed_out;
+  }
+
+  switch (t->mode) {
+    case PSKV_MODE_SCALAR: rc = run_scalar(t, r); break;
+    case PSKV_MODE_FIXED: rc = run_fixed(t, r); break;
+    default: rc = run_varlen(t, r); break;
+  }
+  if (out_nvals) *out_nvals = r.out_nvals;
+  if (rc) return rc;
+  if (too_small)
+    return set_error(PSKV_ESIZE_MISMATCH, "response needs %llu floats, buffer holds %llu",
+                     (unsigned long long)fixed_out, (unsigned long long)out_cap);
+
+  if (host) {
+    if (pull && r.out_nvals)
+      PSKV_HIP(hipMemcpyAsync(out, r.out, r.out_nvals * 4, hipMemcpyDeviceToHost, t->stream));
+    if (pull && varlen && out_lens && n)
+      PSKV_HIP(hipMemcpyAsync(out_lens, r.out_lens, n * 4, hipMemcpyDeviceToHost, t->stream));
+    rc = read_state(t);  // also waits for the copies above
+    if (rc) return rc;
+    return report_device_errors(t);
+  }
+  return PSKV_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
+  clear_error();
+  if (!out || !opts) return set_error(PSKV_EINVAL, "null argument");
+  *out = nullptr;
+  if (opts->mode < PSKV_MODE_SCALAR || opts->mode > PSKV_MODE_VARLEN)
+    return set_error(PSKV_EINVAL, "bad mode %d", opts->mode);
+  if (opts->max_load < 0.f || opts->max_load > 0.9f)
+    return set_error(PSKV_EINVAL, "max_load must lie in (0, 0.9]");
+  int ndev = 0;
+  if (hipGetDeviceCount(&ndev) != hipSuccess || ndev <= 0)
+    return set_error(PSKV_EHIP, "no HIP device available");
+  if (opts->device < 0 || opts->device >= ndev)
+    return set_error(PSKV_EINVAL, "device %d out of range (%d present)", opts->device, ndev);
+  DeviceGuard guard(opts->device);
+  if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", opts->device);
+
+  pskv_table* t = new (std::nothrow) pskv_table();
+  if (!t) return set_error(PSKV_ENOMEM, "out of host memory");
+  t->device = opts->device;
+  t->mode = opts->mode;
+  t->max_load = opts->max_load > 0.f ? opts->max_load : 0.5f;
+  t->row_len = opts->mode == PSKV_MODE_FIXED ? opts->row_len : 0;
+  auto fail = [&](int rc) {
+    pskv_table_destroy(t);
+    return rc;
+  };
+  if (opts->stream) {
+    t->stream = static_cast<hipStream_t>(opts->stream);
+  } else {
+    if (hipStreamCreateWithFlags(&t->stream, hipStreamNonBlocking) != hipSuccess)
+      return fail(set_error(PSKV_EHIP, "hipStreamCreateWithFlags failed"));
+    t->own_stream = true;
+  }
+  const uint64_t keys = opts->initial_capacity ? opts->initial_capacity : kDefaultCapacity;
+  t->cap = std::max(kMinSlots, next_pow2((uint64_t)((double)keys / t->max_load) + 1));
+  int rc = alloc_slots(t->cap, &t->slots, t->stream);
+  if (rc) return fail(rc);
+  if (hipMalloc(reinterpret_cast<void**>(&t->st), sizeof(DevState)) != hipSuccess ||
+      hipMemsetAsync(t->st, 0, sizeof(DevState), t->stream) != hipSuccess ||
+      hipHostMalloc(reinterpret_cast<void**>(&t->st_host), sizeof(DevState), hipHostMallocDefault) !=
+          hipSuccess)
+    return fail(set_error(PSKV_ENOMEM, "cannot allocate table state"));
+  if (t->mode != PSKV_MODE_SCALAR && opts->arena_floats) {
+    t->arena_cap = (opts->arena_floats + 1023) & ~(uint64_t)1023;
+    if (hipMalloc(reinterpret_cast<void**>(&t->arena), t->arena_cap * sizeof(float)) != hipSuccess)
+      return fail(set_error(PSKV_ENOMEM, "cannot allocate %llu floats of row storage",
+                            (unsigned long long)t->arena_cap));
+  }
+  if (hipStreamSynchronize(t->stream) != hipSuccess)
+    return fail(set_error(PSKV_EHIP, "table initialisation failed"));
+  *out = t;
+  return PSKV_OK;
+}
+
+int pskv_table_destroy(pskv_table* t) {
+  if (!t) return PSKV_OK;
+  DeviceGuard guard(t->device);
+  if (t->stream) (void)hipStreamSynchronize(t->stream);
+  for (int k = 0; k < PSKV_KERNEL_COUNT; ++k)
+    for (const EventPair& ev : t->pending[k]) t->free_events.push_back(ev);
+  for (const EventPair& ev : t->free_events) {
+    (void)hipEventDestroy(ev.a);
+    (void)hipEventDestroy(ev.b);
+  }
+  if (t->slots) (void)hipFree(t->slots);
+  if (t->st) (void)hipFree(t->st);
+  if (t->st_host) (void)hipHostFree(t->st_host);
+  if (t->arena) (void)hipFree(t->arena);
+  if (t->ws.ptr) (void)hipFree(t->ws.ptr);
+  if (t->stage.ptr) (void)hipFree(t->stage.ptr);
+  if (t->tiles.ptr) (void)hipFree(t->tiles.ptr);
+  if (t->stage_out.ptr) (void)hipFree(t->stage_out.ptr);
+  if (t->own_stream && t->stream) (void)hipStreamDestroy(t->stream);
+  delete t;
+  return PSKV_OK;
+}
+
+int pskv_push(pskv_table* t, const uint64_t* keys, size_t n, const float* vals, size_t nvals,
+              const int32_t* lens, size_t nlens, int memkind) {
+  return request(t, true, false, keys, n, vals, nvals, lens, nlens, nullptr, 0, nullptr, nullptr,
+                 memkind);
+}
+
+int pskv_pull(pskv_table* t, const uint64_t* keys, size_t n, float* out, size_t out_cap,
+              int32_t* out_lens, size_t* out_nvals, int memkind) {
+  return request(t, false, true, keys, n, nullptr, 0, nullptr, 0, out, out_cap, out_lens,
+                 out_nvals, memkind);
+}
+
+int pskv_pushpull(pskv_table* t, const uint64_t* keys, size_t n, const float* vals, size_t nvals,
+                  const int32_t* lens, size_t nlens, float* out, size_t out_cap,
+                  int32_t* out_lens, size_t* out_nvals, int memkind) {
+  return request(t, true, true, keys, n, vals, nvals, lens, nlens, out, out_cap, out_lens,
+                 out_nvals, memkind);
+}
+
+int pskv_sync(pskv_table* t) {
+  clear_error();
+  if (!t) return set_error(PSKV_EINVAL, "null table");
+  DeviceGuard guard(t->device);
+  int rc = read_state(t);
+  if (rc) return rc;
+  t->count_ub = t->st_host->count;
+  if (t->mode != PSKV_MODE_SCALAR) t->top_ub = t->st_host->arena_top;
+  return report_device_errors(t);
+}
+
+int pskv_size(pskv_table* t, uint64_t* n_keys, uint64_t* n_vals) {
+  clear_error();
+  if (!t) return set_error(PSKV_EINVAL, "null table");
+  DeviceGuard guard(t->device);
+  int rc = read_state(t);
+  if (rc) return rc;
+  const uint64_t nk = t->st_host->count;  // includes key 2^64-1 when present
+  if (n_keys) *n_keys = nk;
+  if (n_vals) {
+    if (t->mode == PSKV_MODE_SCALAR) {
+      *n_vals = nk;
+    } else if (t->mode == PSKV_MODE_FIXED) {
+      *n_vals = nk * t->row_len;
+    } else {
+      unsigned long long* d_total = nullptr;
+      PSKV_HIP(hipMalloc(reinterpret_cast<void**>(&d_total), sizeof(unsigned long long)));
+      PSKV_HIP(hipMemsetAsync(d_total, 0, sizeof(unsigned long long), t->stream));
+      k_sum_lens<<<dim3(grid_for(t->cap, kBlock, 4096)), dim3(kBlock), 0, t->stream>>>(
+          t->slots, t->cap, t->st, d_total);
+      unsigned long long total = 0;
+      hipError_t e = hipMemcpyAsync(&total, d_total, sizeof(total), hipMemcpyDeviceToHost, t->stream);
+      if (e == hipSuccess) e = hipStreamSynchronize(t->stream);
+      (void)hipFree(d_total);
+      PSKV_HIP(e);
+      *n_vals = total;
+    }
+  }
+  return PSKV_OK;
+}
+
+int pskv_dump(pskv_table* t, uint64_t* keys, int32_t* lens, size_t cap_keys, float* vals,
+              size_t cap_vals, size_t* n_keys, size_t* n_vals) {
+  clear_error();
+  if (!t) return set_error(PSKV_EINVAL, "null table");
+  uint64_t nk = 0, nv = 0;
+  int rc = pskv_size(t, &nk, &nv);
+  if (rc) return rc;
+  if (n_keys) *n_keys = nk;
+  if (n_vals) *n_vals = nv;
+  if (nk > cap_keys || nv > cap_vals)
+    return set_error(PSKV_ESIZE_MISMATCH, "dump needs room for %llu keys and %llu values",
+                     (unsigned long long)nk, (unsigned long long)nv);
+  if (nk == 0) return PSKV_OK;
+  DeviceGuard guard(t->device);
+  const uint64_t in_slots = t->st_host->count - (t->st_host->special_present ? 1 : 0);
+  if (in_slots) {
+    uint64_t* d_keys = nullptr;
+    unsigned long long* d_counter = nullptr;
+    PSKV_HIP(hipMalloc(reinterpret_cast<void**>(&d_keys), in_slots * sizeof(uint64_t)));
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&d_counter), sizeof(unsigned long long));
+    if (e == hipSuccess) e = hipMemsetAsync(d_counter, 0, sizeof(unsigned long long), t->stream);
+    if (e == hipSuccess) {
+      k_collect_keys<<<dim3(grid_for(t->cap, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(
+          t->slots, t->cap, d_keys, in_slots, d_counter);
+      e = hipMemcpyAsync(keys, d_keys, in_slots * sizeof(uint64_t), hipMemcpyDeviceToHost, t->stream);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(t->stream);
+    (void)hipFree(d_keys);
+    if (d_counter) (void)hipFree(d_counter);
+    PSKV_HIP(e);
+  }
+  if (t->st_host->special_present) keys[in_slots] = kEmptyKey;
+  std::sort(keys, keys + nk);
+  // every key is present, so this pull changes nothing in the store
+  size_t got = 0;
+  std::vector<int32_t> tmp_lens;
+  int32_t* lens_out = lens;
+  if (t->mode == PSKV_MODE_VARLEN && !lens_out) {
+    tmp_lens.resize(nk);
+    lens_out = tmp_lens.data();
+  }
+  t->no_growth = true;
+  rc = pskv_pull(t, keys, nk, vals, cap_vals, t->mode == PSKV_MODE_VARLEN ? lens_out : nullptr, &got,
+                 PSKV_MEM_HOST);
+  t->no_growth = false;
+  if (rc) return rc;
+  if (lens && t->mode != PSKV_MODE_VARLEN) {
+    const int32_t l = t->mode == PSKV_MODE_SCALAR ? 1 : (int32_t)t->row_len;
+    for (uint64_t i = 0; i < nk; ++i) lens[i] = l;
+  }
+  return PSKV_OK;
+}
+
+int pskv_prof_enable(pskv_table* t, int on) {
+  if (!t) return set_error(PSKV_EINVAL, "null table");
+  t->prof = on != 0;
+  return PSKV_OK;
+}
+
+int pskv_prof_reset(pskv_table* t) {
+  if (!t) return set_error(PSKV_EINVAL, "null table");
+  DeviceGuard guard(t->device);
+  int rc = prof_collect(t);
+  for (int k = 0; k < PSKV_KERNEL_COUNT; ++k) {
+    t->launches[k] = 0;
+    t->total_ms[k] = 0.0;
+  }
+  return rc;
+}
+
+int pskv_prof_read(pskv_table* t, int kernel, uint64_t* launches, double* total_ms) {
+  if (!t) return set_error(PSKV_EINVAL, "null table");
+  if (kernel < 0 || kernel >= PSKV_KERNEL_COUNT) return set_error(PSKV_EINVAL, "bad kernel id");
+  DeviceGuard guard(t->device);
+  int rc = prof_collect(t);
+  if (launches) *launches = t->launches[kernel];
+  if (total_ms) *total_ms = t->total_ms[kernel];
+  return rc;
+}
+
+int pskv_copy_probe(pskv_table* t, void* dst, const void* src, size_t bytes) {
+  if (!t) return set_error(PSKV_EINVAL, "null table");
+  if ((bytes & 15) || (reinterpret_cast<uintptr_t>(dst) & 15) || (reinterpret_cast<uintptr_t>(src) & 15))
+    return set_error(PSKV_EINVAL, "copy probe needs 16-byte aligned buffers and size");
+  if (!bytes) return PSKV_OK;
+  DeviceGuard guard(t->device);
+  const uint64_t n16 = bytes / 16;
+  k_copy<<<dim3(grid_for(n16, kBlock * 4, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(
+      static_cast<float4*>(dst), static_cast<const float4*>(src), n16);
+  PSKV_HIP(hipGetLastError());
+  return PSKV_OK;
+}
+
+const char* pskv_last_error(void) { return g_last_error.c_str(); }
+const char* pskv_version(void) { return "pskv 0.1 gfx950"; }
+
+}  // extern "C"

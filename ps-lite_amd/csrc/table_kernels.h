@@ -1,0 +1,433 @@
+// Device kernels of the HBM-resident key-value store (gfx950).
+//
+// They replace the body of KVServerDefaultHandle::operator()
+// (include/ps/kv_app.h:442-461): `store[key] += val` becomes find-or-insert in an
+// open-addressing table followed by a float add, `res.vals[i] = store[key]`
+// becomes a gather. The row kernels extend the same two operations to the
+// multi-float layouts of KVPairs (kv_app.h:17-31).
+#ifndef PSKV_TABLE_KERNELS_H_
+#define PSKV_TABLE_KERNELS_H_
+#include "device_common.h"
+
+namespace pskv {
+
+// ---------------------------------------------------------------------------------
+// SCALAR mode: one float per key, kept in the low word of the slot payload so that a
+// probe reads key and value with one 128-bit load.
+// One lane per key. Keys are unique within a request, so the value word of a slot is
+// only ever touched by the lane that owns the key: no atomics on values, and the
+// per-key sum order is the request order (requests are serialised on one stream).
+// ---------------------------------------------------------------------------------
+template <bool PUSH, bool PULL>
+__global__ __launch_bounds__(kBlock) void k_scalar(Slot* __restrict__ slots, uint64_t mask,
+                                                  DevState* st,
+                                                  const uint64_t* __restrict__ keys,
+                                                  const float* __restrict__ vals,
+                                                  float* __restrict__ out, uint64_t n) {
+  unsigned created = 0;
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+    const uint64_t key = keys[i];
+    float v = 0.0f;
+    if (PUSH) v = vals[i];
+    bool is_new;
+    uint64_t seen;
+    uint64_t* p = find_or_insert(slots, mask, st, key, is_new, seen);
+    if (!p) continue;
+    // an absent key starts from Val() == 0, then `+=` (kv_app.h:454): 0.0f + v, not a copy
+    float cur = is_new ? 0.0f : __uint_as_float((unsigned)seen);
+    if (PUSH) cur = cur + v;
+    if (PUSH || is_new) *reinterpret_cast<float*>(p) = cur;
+    if (PULL) out[i] = cur;
+    created += is_new ? 1u : 0u;
+  }
+  created = wave_sum_u32(created);
+  if ((threadIdx.x & 63) == 0 && created) atomicAdd(&st->count, (unsigned long long)created);
+}
+
+// ---------------------------------------------------------------------------------
+// Row modes, step 1: key -> row reference.
+// ---------------------------------------------------------------------------------
+
+// Resets the per-request words; one thread, first launch of every row-mode request.
+__global__ void k_begin_request(DevState* st) {
+  st->error |= st->req_error;
+  st->req_error = 0;
+  st->misaligned = 0;
+}
+
+// FIXED: find or create the row of every key. Push and pull both create
+// (pull of an absent key inserts a zero value, kv_app.h:457).
+__global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slots, uint64_t mask,
+                                                        DevState* st,
+                                                        const uint64_t* __restrict__ keys,
+                                                        uint64_t n, uint64_t* __restrict__ ref) {
+  unsigned created = 0;
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  // uniform trip count per wavefront: the wave-wide scan below needs all 64 lanes
+  for (uint64_t base = (uint64_t)blockIdx.x * kBlock; base < n; base += stride) {
+    const uint64_t i = base + threadIdx.x;
+    const bool active = i < n;
+    bool is_new = false;
+    uint64_t seen = 0;
+    uint64_t* p = nullptr;
+    if (active) p = find_or_insert(slots, mask, st, keys[i], is_new, seen);
+    const unsigned long long need = (p && is_new) ? 1ull : 0ull;
+    const unsigned long long inc = wave_incl_scan_u64(need);
+    const unsigned long long tot = __shfl(inc, 63);
+    unsigned long long first = 0;
+    if ((threadIdx.x & 63) == 63 && tot) first = atomicAdd(&st->arena_top, tot);
+    first = __shfl(first, 63);
+    if (p) {
+      uint64_t row = seen;
+      if (is_new) {
+        row = first + inc - need;
+        *p = row;
+        ++created;
+      }
+      ref[i] = row | (is_new ? kRefNew : 0ull);
+    } else if (active) {
+      ref[i] = kRefAbsent;
+    }
+  }
+  created = wave_sum_u32(created);
+  if ((threadIdx.x & 63) == 0 && created) atomicAdd(&st->count, (unsigned long long)created);
+}
+
+// VARLEN push: find or create; a created row gets ceil(len/4) 16-byte units of the
+// arena, so every row starts 16-byte aligned. A present row must have the pushed length.
+__global__ __launch_bounds__(kBlock) void k_lookup_var_push(
+    Slot* __restrict__ slots, uint64_t mask, DevState* st, const uint64_t* __restrict__ keys,
+    const int32_t* __restrict__ lens, uint64_t n, uint64_t nvals, uint64_t* __restrict__ ref) {
+  // the request is refused as a whole when its lens are invalid or do not add up to vals.size()
+  if (st->req_error & (kDevErrBadLen | kDevErrSizeMismatch)) return;
+  if (st->scan_total != nvals) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) atomicOr(&st->req_error, kDevErrSizeMismatch);
+    return;
+  }
+  unsigned created = 0;
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t base = (uint64_t)blockIdx.x * kBlock; base < n; base += stride) {
+    const uint64_t i = base + threadIdx.x;
+    const bool active = i < n;
+    bool is_new = false;
+    uint64_t seen = 0;
+    uint64_t* p = nullptr;
+    uint64_t len = 0;
+    if (active) {
+      len = (uint64_t)(uint32_t)lens[i];
+      p = find_or_insert(slots, mask, st, keys[i], is_new, seen);
+    }
+    const unsigned long long need = (p && is_new) ? ((len + 3) >> 2) : 0ull;
+    const unsigned long long inc = wave_incl_scan_u64(need);
+    const unsigned long long tot = __shfl(inc, 63);
+    unsigned long long first = 0;
+    if ((threadIdx.x & 63) == 63 && tot) first = atomicAdd(&st->arena_top, tot);
+    first = __shfl(first, 63);
+    if (p) {
+      uint64_t payload = seen;
+      if (is_new) {
+        payload = ((first + inc - need) << kLenBits) | len;
+        *p = payload;
+        ++created;
+      } else if ((payload & kLenMask) != len) {
+        atomicOr(&st->req_error, kDevErrLenChanged);
+      }
+      ref[i] = payload | (is_new ? kRefNew : 0ull);
+    } else if (active) {
+      ref[i] = kRefAbsent;
+    }
+  }
+  created = wave_sum_u32(created);
+  if ((threadIdx.x & 63) == 0 && created) atomicAdd(&st->count, (unsigned long long)created);
+}
+
+// VARLEN pull: an absent key answers length 0 and is not created.
+__global__ __launch_bounds__(kBlock) void k_lookup_var_pull(const Slot* __restrict__ slots,
+                                                           uint64_t mask, const DevState* st,
+                                                           const uint64_t* __restrict__ keys,
+                                                           uint64_t n, uint64_t* __restrict__ ref,
+                                                           int32_t* __restrict__ out_lens) {
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+    uint64_t payload;
+    const bool hit = find_only(slots, mask, st, keys[i], payload);
+    ref[i] = hit ? payload : kRefAbsent;
+    out_lens[i] = hit ? (int32_t)(payload & kLenMask) : 0;
+  }
+}
+
+// VARLEN: first key of every request-side tile. Key j owns floats [off[j], off[j+1]);
+// it writes its index for each tile whose first float it owns, so every tile gets
+// exactly one writer and no search is needed later. Entry `ntiles` closes the table.
+__global__ __launch_bounds__(kBlock) void k_tile_keys(const uint64_t* __restrict__ off, uint64_t n,
+                                                     uint32_t* __restrict__ tile_key,
+                                                     uint64_t ntiles) {
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t j = (uint64_t)blockIdx.x * kBlock + threadIdx.x; j < n; j += stride) {
+    const uint64_t a = off[j], b = off[j + 1];
+    if (j == 0) tile_key[ntiles] = (uint32_t)(n - 1);
+    if (b <= a) continue;
+    uint64_t t = (a + kTileFloats - 1) / kTileFloats;
+    const uint64_t t_last = (b - 1) / kTileFloats;
+    for (; t <= t_last && t < ntiles; ++t) tile_key[t] = (uint32_t)j;
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Row modes, step 2: stream the values.
+// A workgroup owns one tile of kTileFloats consecutive floats of the request-side
+// buffer, whatever rows they belong to, so the load is balanced for any mix of row
+// lengths and the request side is read or written fully coalesced with 128-bit
+// accesses. FIXED locates the row of an element by division; VARLEN stages the
+// offsets and row references of the keys that overlap the tile in LDS and locates
+// rows by binary search there.
+// ---------------------------------------------------------------------------------
+struct RowsParams {
+  float* req;                // push: request values (read); pull: response values (written)
+  float* arena;              // row storage
+  const uint64_t* ref;       // n row references from the lookup kernel
+  const uint64_t* off;       // VARLEN: n+1 request-side row offsets in floats
+  const uint32_t* tile_key;  // VARLEN: ntiles+1 entries
+  DevState* st;
+  uint64_t n;
+  uint64_t total;         // floats in req
+  uint64_t k;             // FIXED: floats per row
+  uint32_t force_scalar;  // request buffer or k not 16-byte friendly
+  uint32_t ignore_new;    // pull half of a push+pull: rows created by the push half hold data
+};
+
+constexpr int kOpAcc = 0;
+constexpr int kOpGather = 1;
+
+template <int VEC>
+struct VecT;
+template <>
+struct VecT<4> {
+  using type = float4;
+  __device__ static float4 zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+  __device__ static float4 add(float4 a, float4 b) {
+    return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
+  }
+};
+template <>
+struct VecT<1> {
+  using type = float;
+  __device__ static float zero() { return 0.f; }
+  __device__ static float add(float a, float b) { return a + b; }
+};
+
+template <int OP, int VEC, bool VARLEN>
+__device__ __forceinline__ void rows_tile(const RowsParams& p, int32_t* s_off, uint64_t* s_ref,
+                                          bool rejected) {
+  using V = typename VecT<VEC>::type;
+  constexpr int kIter = kTileFloats / (VEC * kBlock);  // elements per thread
+  constexpr int kGroup = 4;                            // loads issued back to back
+  const uint64_t f0 = (uint64_t)blockIdx.x * kTileFloats;
+  const uint32_t tile_floats =
+      (uint32_t)((p.total - f0 < (uint64_t)kTileFloats) ? (p.total - f0) : (uint64_t)kTileFloats);
+  const uint32_t nelem = tile_floats / VEC;
+
+  // FIXED: row and offset of the tile's first float
+  uint64_t j0 = 0, rem0 = 0;
+  // VARLEN: keys that overlap the tile
+  uint64_t j_lo = 0;
+  uint32_t span = 0;
+  bool staged = false;
+  if (VARLEN) {
+    j_lo = p.tile_key[blockIdx.x];
+    span = (uint32_t)((uint64_t)p.tile_key[blockIdx.x + 1] - j_lo + 1);
+    staged = span <= kSpanMax;
+    if (staged) {
+      for (uint32_t s = threadIdx.x; s <= span; s += kBlock) {
+        s_off[s] = (int32_t)(int64_t)(p.off[j_lo + s] - f0);
+        if (s < span) s_ref[s] = p.ref[j_lo + s];
+      }
+      __syncthreads();
+    }
+  } else {
+    j0 = f0 / p.k;
+    rem0 = f0 - j0 * p.k;
+  }
+
+#pragma unroll
+  for (int g = 0; g < kIter; g += kGroup) {
+    V x[kGroup], y[kGroup];
+    V* dst[kGroup];
+    uint32_t lf[kGroup];
+    bool live[kGroup], fresh[kGroup];
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
+      const uint32_t le = (uint32_t)(g + u) * kBlock + threadIdx.x;
+      live[u] = le < nelem;
+      lf[u] = le * VEC;
+      dst[u] = nullptr;
+      fresh[u] = false;
+      if (!live[u]) continue;
+      uint64_t r, within;
+      if (VARLEN) {
+        if (staged) {
+          // last key whose first float is at or before lf (zero-length rows repeat an offset)
+          uint32_t lo = 0, hi = span;
+          while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (s_off[mid] <= (int32_t)lf[u]) lo = mid + 1; else hi = mid;
+          }
+          r = s_ref[lo - 1];
+          within = (uint64_t)((int32_t)lf[u] - s_off[lo - 1]);
+        } else {
+          const uint64_t f = f0 + lf[u];
+          uint64_t lo = j_lo, hi = j_lo + span;
+          while (lo < hi) {
+            const uint64_t mid = (lo + hi) >> 1;
+            if (p.off[mid] <= f) lo = mid + 1; else hi = mid;
+          }
+          r = p.ref[lo - 1];
+          within = f - p.off[lo - 1];
+        }
+        dst[u] = reinterpret_cast<V*>(p.arena + (((r & ~kRefNew) >> kLenBits) << 2) + within);
+      } else {
+        const uint64_t xoff = rem0 + lf[u];
+        uint64_t q;
+        if (p.k >= (uint64_t)kTileFloats) {
+          q = xoff >= p.k ? 1u : 0u;
+          within = q ? xoff - p.k : xoff;
+        } else {
+          const uint32_t q32 = (uint32_t)xoff / (uint32_t)p.k;
+          q = q32;
+          within = (uint32_t)xoff - q32 * (uint32_t)p.k;
+        }
+        r = p.ref[j0 + q];
+        dst[u] = reinterpret_cast<V*>(p.arena + (r & ~kRefNew) * p.k + within);
+      }
+      if (r == kRefAbsent) {  // only after a full table, which the host sizing rules out
+        live[u] = false;
+        continue;
+      }
+      fresh[u] = (r & kRefNew) != 0 && !p.ignore_new;
+    }
+    // all loads of the group first, so each lane has up to 2*kGroup requests in flight
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
+      x[u] = VecT<VEC>::zero();
+      y[u] = VecT<VEC>::zero();
+      if (!live[u]) continue;
+      if (OP == kOpAcc) x[u] = *reinterpret_cast<const V*>(p.req + f0 + lf[u]);
+      if (!fresh[u]) y[u] = *dst[u];
+    }
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
+      if (!live[u]) continue;
+      if (OP == kOpAcc) {
+        if (rejected) {
+          // a refused push changes no stored value; rows it created stay, as zero rows
+          if (fresh[u]) *dst[u] = VecT<VEC>::zero();
+        } else {
+          // a created row is a zero row first (0.0f + v), kv_app.h:454
+          *dst[u] = VecT<VEC>::add(y[u], x[u]);
+        }
+      } else {
+        *reinterpret_cast<V*>(p.req + f0 + lf[u]) = y[u];
+        if (fresh[u]) *dst[u] = VecT<VEC>::zero();  // pull created the row: it now exists as zeros
+      }
+    }
+  }
+}
+
+template <int OP, bool VARLEN>
+__global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
+  __shared__ int32_t s_off[VARLEN ? kSpanMax + 1 : 1];
+  __shared__ uint64_t s_ref[VARLEN ? kSpanMax : 1];
+  bool rejected = false;
+  bool scalar = p.force_scalar != 0;
+  if (VARLEN) {
+    const unsigned err = p.st->req_error;
+    if (err & (kDevErrBadLen | kDevErrSizeMismatch)) return;
+    rejected = (err & kDevErrLenChanged) != 0;
+    scalar = scalar || (p.st->misaligned != 0);
+  }
+  if (scalar) {
+    rows_tile<OP, 1, VARLEN>(p, s_off, s_ref, rejected);
+  } else {
+    rows_tile<OP, 4, VARLEN>(p, s_off, s_ref, rejected);
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Maintenance kernels.
+// ---------------------------------------------------------------------------------
+
+// Growth: every live slot of the old array is re-inserted into the new one; payloads
+// move bit for bit, so stored sums are unchanged.
+__global__ __launch_bounds__(kBlock) void k_rehash(const Slot* __restrict__ old_slots,
+                                                  uint64_t old_cap, Slot* __restrict__ slots,
+                                                  uint64_t mask, DevState* st) {
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < old_cap; i += stride) {
+    const ulonglong2 s = *reinterpret_cast<const ulonglong2*>(&old_slots[i]);
+    if (s.x == kEmptyKey) continue;
+    uint64_t h = mix64(s.x) & mask;
+    bool placed = false;
+    for (uint64_t probes = 0; probes <= mask; ++probes) {
+      if (slots[h].key == kEmptyKey) {
+        unsigned long long old =
+            atomicCAS(reinterpret_cast<unsigned long long*>(&slots[h].key),
+                      (unsigned long long)kEmptyKey, (unsigned long long)s.x);
+        if (old == kEmptyKey) {
+          slots[h].payload = s.y;
+          placed = true;
+          break;
+        }
+      }
+      h = (h + 1) & mask;
+    }
+    if (!placed) atomicOr(&st->error, kDevErrFull);
+  }
+}
+
+// Collects the keys of all live slots (unordered); *counter must start at 0.
+__global__ __launch_bounds__(kBlock) void k_collect_keys(const Slot* __restrict__ slots,
+                                                        uint64_t cap, uint64_t* __restrict__ out,
+                                                        uint64_t out_cap,
+                                                        unsigned long long* counter) {
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t base = (uint64_t)blockIdx.x * kBlock; base < cap; base += stride) {
+    const uint64_t i = base + threadIdx.x;
+    uint64_t key = kEmptyKey;
+    if (i < cap) key = slots[i].key;
+    const unsigned long long need = key != kEmptyKey ? 1ull : 0ull;
+    const unsigned long long inc = wave_incl_scan_u64(need);
+    const unsigned long long tot = __shfl(inc, 63);
+    unsigned long long first = 0;
+    if ((threadIdx.x & 63) == 63 && tot) first = atomicAdd(counter, tot);
+    first = __shfl(first, 63);
+    const unsigned long long at = first + inc - need;
+    if (need && at < out_cap) out[at] = key;
+  }
+}
+
+// VARLEN: total floats of all stored rows.
+__global__ __launch_bounds__(kBlock) void k_sum_lens(const Slot* __restrict__ slots, uint64_t cap,
+                                                    const DevState* st,
+                                                    unsigned long long* total) {
+  unsigned long long s = 0;
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < cap; i += stride) {
+    const ulonglong2 v = *reinterpret_cast<const ulonglong2*>(&slots[i]);
+    if (v.x != kEmptyKey) s += v.y & kLenMask;
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0 && st->special_present) s += st->special_payload & kLenMask;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+  if ((threadIdx.x & 63) == 0 && s) atomicAdd(total, s);
+}
+
+// Plain streaming copy, 16 bytes per lane per step.
+__global__ __launch_bounds__(kBlock) void k_copy(float4* __restrict__ dst,
+                                                const float4* __restrict__ src, uint64_t n16) {
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
+}  // namespace pskv
+#endif  // PSKV_TABLE_KERNELS_H_

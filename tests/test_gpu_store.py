@@ -1,0 +1,275 @@
+"""GPU parity of the store (request handle) against the CPU oracle, through the C ABI.
+Bar: bit-exact pulled values, identical stored key sets, identical sizes."""
+import numpy as np
+import pytest
+
+from conftest import announce
+from helpers import KMAX, assert_bits_equal, from_dev, to_dev, unique_keys
+
+pytestmark = pytest.mark.gpu
+
+
+def _check_dump(t, o, what):
+    gk, gl, gv = t.dump()
+    ok, ol, ov = o.dump()
+    assert np.array_equal(gk, ok), what + ": stored keys differ"
+    assert np.array_equal(gl, ol), what + ": stored lens differ"
+    assert_bits_equal(gv, ov, what + " dump")
+    assert t.size() == o.size()
+
+
+@pytest.mark.parametrize("memkind", ["device", "host"])
+@pytest.mark.parametrize("n,cap", [(1, 0), (1000, 16), (50000, 1024)])
+def test_scalar_push_pull(capi, orc, dev, memkind, n, cap):
+    import torch
+    announce("scalar_push_pull", memkind, n, cap)
+    rng = np.random.default_rng(100 + n)
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=cap)
+    o = orc.Store(orc.MODE_SCALAR)
+    universe = unique_keys(rng, 2 * n)
+    for rep in range(4):
+        keys = np.sort(rng.choice(universe, size=n, replace=False))
+        vals = rng.standard_normal(n).astype(np.float32)
+        if memkind == "device":
+            t.push(to_dev(keys, dev), to_dev(vals, dev))
+        else:
+            t.push(keys, vals)
+        o.push(keys, vals)
+    keys = np.sort(rng.choice(universe, size=n, replace=False))
+    want, _ = o.pull(keys)
+    if memkind == "device":
+        out = torch.full((n,), 7.0, dtype=torch.float32, device=dev)
+        assert t.pull(to_dev(keys, dev), out) == n
+        t.sync()
+        got = from_dev(out)
+    else:
+        got = np.full(n, 7.0, np.float32)
+        assert t.pull(keys, got) == n
+    assert_bits_equal(got, want, "pull")
+    _check_dump(t, o, "scalar")
+
+
+def test_scalar_closed_form_50_pushes(capi, dev):
+    """tests/test_kv_app.cc:27-60: keys kMaxKey/num*i, 50 pushes then pull == 50*v, 50 more
+    push+pulls == 100*v."""
+    import torch
+    announce("scalar_closed_form")
+    num = 1000
+    keys = (np.uint64(KMAX // num) * np.arange(num, dtype=np.uint64))
+    vals = np.random.default_rng(7).integers(0, 1000, size=num).astype(np.float32)
+    t = capi.Table(capi.MODE_SCALAR)
+    dk, dv = to_dev(keys, dev), to_dev(vals, dev)
+    for _ in range(50):
+        t.push(dk, dv)
+    out = torch.zeros(num, dtype=torch.float32, device=dev)
+    t.pull(dk, out)
+    t.sync()
+    assert np.array_equal(from_dev(out), vals * 50)
+    for _ in range(50):
+        t.pushpull(dk, dv, out)
+    t.sync()
+    assert np.array_equal(from_dev(out), vals * 100)
+    assert t.size() == (num, num)
+
+
+def test_scalar_special_values(capi, orc, dev):
+    """-0.0 on a fresh key stores +0.0 (0.0f + v), denormals are kept, a pull creates absent keys,
+    and key 2^64-1 is an ordinary key for the handle."""
+    announce("scalar_special_values")
+    keys = np.array([0, 1, 5, 77, KMAX - 1, KMAX], np.uint64)
+    v1 = np.array([-0.0, 1e-42, np.inf, 3.5, -2.25, 9.0], np.float32)
+    v2 = np.array([-0.0, 1e-42, -1.0, 1e-45, 2.25, 1.0], np.float32)
+    t = capi.Table(capi.MODE_SCALAR)
+    o = orc.Store(orc.MODE_SCALAR)
+    for v in (v1, v2):
+        t.push(keys, v)
+        o.push(keys, v)
+    probe = np.array([0, 1, 2, 5, 77, 1000, KMAX - 1, KMAX], np.uint64)
+    got = np.full(probe.size, 5.0, np.float32)
+    t.pull(probe, got)
+    want, _ = o.pull(probe)
+    assert_bits_equal(got, want, "special")
+    assert got.view(np.uint32)[0] == 0  # +0.0, not 0x80000000
+    assert t.size() == o.size() == (8, 8)
+    _check_dump(t, o, "special")
+
+
+def test_scalar_growth(capi, orc, dev):
+    """The slot array grows from its minimum to 300k keys; sums survive every rehash."""
+    announce("scalar_growth")
+    rng = np.random.default_rng(5)
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=1)
+    o = orc.Store(orc.MODE_SCALAR)
+    universe = unique_keys(rng, 300000)
+    for rep in range(6):
+        keys = np.sort(universe[rng.random(universe.size) < 0.5])
+        vals = rng.standard_normal(keys.size).astype(np.float32)
+        t.push(to_dev(keys, dev), to_dev(vals, dev))
+        o.push(keys, vals)
+    _check_dump(t, o, "growth")
+
+
+def test_scalar_size_checks(capi, dev):
+    announce("scalar_size_checks")
+    t = capi.Table(capi.MODE_SCALAR)
+    keys = np.array([1, 2, 3], np.uint64)
+    with pytest.raises(capi.PskvError) as e:  # kv_app.h:447
+        t.push(keys, np.zeros(2, np.float32))
+    assert e.value.code == capi.ESIZE_MISMATCH
+    out = np.zeros(2, np.float32)
+    with pytest.raises(capi.PskvError) as e:
+        t.pull(keys, out)
+    assert e.value.code == capi.ESIZE_MISMATCH and t.last_out_nvals == 3
+    assert t.size() == (3, 3)  # the pull still created the keys, as the reference would
+    t.push(np.zeros(0, np.uint64), np.zeros(0, np.float32))
+    assert t.pull(np.zeros(0, np.uint64), np.zeros(0, np.float32)) == 0
+
+
+@pytest.mark.parametrize("memkind", ["device", "host"])
+@pytest.mark.parametrize("n,k", [(64, 4096 * 3), (5, 1), (1000, 2), (300, 7), (257, 64), (3, 100000),
+                                 (2, 4096 + 8)])
+def test_fixed_rows(capi, orc, dev, memkind, n, k):
+    import torch
+    announce("fixed_rows", memkind, n, k)
+    rng = np.random.default_rng(n * 131 + k)
+    t = capi.Table(capi.MODE_FIXED, initial_capacity=16)
+    o = orc.Store(orc.MODE_FIXED)
+    universe = unique_keys(rng, 2 * n)
+    for rep in range(3):
+        keys = np.sort(rng.choice(universe, size=n, replace=False))
+        vals = rng.uniform(-1, 1, size=n * k).astype(np.float32)
+        if rep == 0:
+            vals[: min(8, vals.size)] = -0.0
+        if memkind == "device":
+            t.push(to_dev(keys, dev), to_dev(vals, dev))
+        else:
+            t.push(keys, vals)
+        o.push(keys, vals)
+    keys = np.sort(rng.choice(universe, size=n, replace=False))
+    want, _ = o.pull(keys)
+    if memkind == "device":
+        out = torch.full((n * k,), 7.0, dtype=torch.float32, device=dev)
+        assert t.pull(to_dev(keys, dev), out) == n * k
+        t.sync()
+        got = from_dev(out)
+    else:
+        got = np.full(n * k, 7.0, np.float32)
+        assert t.pull(keys, got) == n * k
+    assert_bits_equal(got, want, "fixed pull")
+    # push+pull in one request
+    vals = rng.uniform(-1, 1, size=n * k).astype(np.float32)
+    want, _ = o.pushpull(keys, vals)
+    got = np.zeros(n * k, np.float32)
+    t.pushpull(keys, vals, got)
+    assert_bits_equal(got, want, "fixed pushpull")
+    _check_dump(t, o, "fixed")
+
+
+def test_fixed_errors(capi, dev):
+    announce("fixed_errors")
+    t = capi.Table(capi.MODE_FIXED)
+    keys = np.array([1, 2, 3], np.uint64)
+    with pytest.raises(capi.PskvError) as e:  # row length still unknown
+        t.pull(keys, np.zeros(3, np.float32))
+    assert e.value.code == capi.EINVAL
+    with pytest.raises(capi.PskvError) as e:  # kv_app.h:549
+        t.push(keys, np.zeros(7, np.float32))
+    assert e.value.code == capi.ESIZE_MISMATCH
+    t.push(keys, np.ones(6, np.float32))
+    with pytest.raises(capi.PskvError) as e:
+        t.push(keys, np.ones(9, np.float32))
+    assert e.value.code == capi.ESIZE_MISMATCH
+    got = np.zeros(6, np.float32)
+    t.pull(keys, got)
+    assert np.array_equal(got, np.ones(6, np.float32))
+
+
+LENS_SETS = {
+    "emb": [8, 16, 32, 64, 128],
+    "ragged": [0, 1, 2, 3, 5, 7, 9, 31],
+    "mult4": [0, 4, 4, 4, 8],
+    "long": [4, 20000, 8, 4096, 12],
+}
+
+
+@pytest.mark.parametrize("memkind", ["device", "host"])
+@pytest.mark.parametrize("n,lens_set", [(2000, "emb"), (5000, "ragged"), (9000, "mult4"),
+                                        (40, "long"), (1, "emb")])
+def test_varlen_rows(capi, orc, dev, memkind, n, lens_set):
+    import torch
+    announce("varlen_rows", memkind, n, lens_set)
+    rng = np.random.default_rng(n + len(lens_set))
+    t = capi.Table(capi.MODE_VARLEN, initial_capacity=16)
+    o = orc.Store(orc.MODE_VARLEN)
+    universe = unique_keys(rng, 2 * n)
+    len_of = dict(zip(universe.tolist(),
+                      rng.choice(np.array(LENS_SETS[lens_set], np.int32), size=universe.size).tolist()))
+    for rep in range(3):
+        keys = np.sort(rng.choice(universe, size=n, replace=False))
+        lens = np.array([len_of[k] for k in keys.tolist()], np.int32)
+        vals = rng.normal(0, 0.1, size=int(lens.sum())).astype(np.float32)
+        if memkind == "device":
+            t.push(to_dev(keys, dev), to_dev(vals, dev), to_dev(lens, dev))
+        else:
+            t.push(keys, vals, lens)
+        o.push(keys, vals, lens)
+    keys = np.sort(rng.choice(universe, size=n, replace=False))  # some absent: len 0, not created
+    want, want_lens = o.pull(keys)
+    if memkind == "device":
+        out = torch.full((want.size + 5,), 7.0, dtype=torch.float32, device=dev)
+        out_lens = torch.full((n,), -1, dtype=torch.int32, device=dev)
+        got_n = t.pull(to_dev(keys, dev), out, out_lens)
+        t.sync()
+        got, got_lens = from_dev(out)[:got_n], from_dev(out_lens)
+    else:
+        got = np.full(want.size, 7.0, np.float32)
+        got_lens = np.full(n, -1, np.int32)
+        got_n = t.pull(keys, got, got_lens)
+    assert got_n == want.size
+    assert np.array_equal(got_lens, want_lens)
+    assert_bits_equal(got, want, "varlen pull")
+    _check_dump(t, o, "varlen")
+
+
+def test_varlen_errors(capi, orc, dev):
+    announce("varlen_errors")
+    t = capi.Table(capi.MODE_VARLEN)
+    o = orc.Store(orc.MODE_VARLEN)
+    keys = np.array([10, 20, 30], np.uint64)
+    lens = np.array([2, 0, 3], np.int32)
+    vals = np.arange(5, dtype=np.float32)
+    for s in (t, o):
+        s.push(keys, vals, lens)
+    # host-visible checks
+    with pytest.raises(capi.PskvError) as e:
+        t.push(keys, vals, lens[:2])
+    assert e.value.code == capi.ESIZE_MISMATCH
+    with pytest.raises(capi.PskvError) as e:
+        t.push(keys, vals[:4], lens)
+    assert e.value.code == capi.ESIZE_MISMATCH
+    with pytest.raises(capi.PskvError) as e:
+        t.push(keys, vals, np.array([2, -1, 4], np.int32))
+    assert e.value.code == capi.EINVAL
+    # a changed length is refused: nothing stored changes, absent keys become zero rows
+    keys2 = np.array([10, 25, 30], np.uint64)
+    lens2 = np.array([2, 4, 1], np.int32)
+    vals2 = np.ones(7, np.float32)
+    with pytest.raises(capi.PskvError) as e:
+        t.push(keys2, vals2, lens2)
+    assert e.value.code == capi.ELEN_CHANGED
+    assert o.handle(True, False, keys2, vals2, lens2)[0] == orc.ELEN_CHANGED
+    _check_dump(t, o, "after refused push")
+    # the same through device buffers: the error is reported by the next sync
+    keys3 = np.array([10, 26, 30], np.uint64)
+    t.push(to_dev(keys3, dev), to_dev(vals2, dev), to_dev(lens2, dev))
+    with pytest.raises(capi.PskvError) as e:
+        t.sync()
+    assert e.value.code == capi.ELEN_CHANGED
+    assert o.handle(True, False, keys3, vals2, lens2)[0] == orc.ELEN_CHANGED
+    t.sync()  # reported once
+    _check_dump(t, o, "after refused device push")
+    # response too small
+    out = np.zeros(2, np.float32)
+    with pytest.raises(capi.PskvError) as e:
+        t.pull(keys, out, np.zeros(3, np.int32))
+    assert e.value.code == capi.ESIZE_MISMATCH and t.last_out_nvals == 5
