@@ -1,0 +1,409 @@
+#!/usr/bin/env python3
+"""Benchmark of the pskv hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+
+Workloads (BASELINE.json `configs`):
+  sparse_lr (default, configs[1]): every step slices 1,000,000 fresh sorted unique uint64
+      keys over 4 server key ranges, pushes each slice into the table of its range
+      (find-or-insert + float add) and pulls the same keys back. 20 steps grow the
+      store to 20M keys. value = (pushed + pulled keys) / s.
+  dense (configs[2]): 64 keys x 4,194,304 float32; a step is one push-accumulate of
+      1 GiB followed by one full pull. value = algorithmic GB/s.
+  varlen (configs[4]): 2,000,000 keys with lens in {8,16,32,64,128} over 16 ranges; a
+      step is one push of all keys followed by a pull with lens. value = keys/s.
+
+Prints ONE JSON line. Inputs are resident in HBM before the clock starts. `roofline`
+is the dominant kernel of the workload timed with HIP events on the stream it runs
+on (inside the timed steps); `cpu_baseline` is the CPU oracle on the same inputs,
+one thread, on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, REPO)
+import __graft_entry__ as graft  # noqa: E402
+
+KMAX = (1 << 64) - 1
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def unique_sorted_keys(rng, n, limit):
+    keys = np.unique(rng.integers(0, limit, size=n + n // 64 + 16, dtype=np.uint64))
+    while keys.size < n:
+        keys = np.unique(np.concatenate([keys, rng.integers(0, limit, size=n, dtype=np.uint64)]))
+    if keys.size > n:
+        keys = np.sort(rng.choice(keys, size=n, replace=False))
+    return keys
+
+
+def to_dev(a, dev):
+    import torch
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint64:
+        a = a.view(np.int64)
+    return torch.from_numpy(a).to(dev)
+
+
+def kernel_stats(tables, kernel):
+    n, ms = 0, 0.0
+    for t in tables:
+        a, b = t.prof_read(kernel)
+        n += a
+        ms += b
+    return n, ms
+
+
+def roofline(alg_bytes_per_launch, launches, total_ms, traffic=None):
+    avg_s = total_ms / launches * 1e-3 if launches else float("nan")
+    achieved = alg_bytes_per_launch / avg_s / 1e9 if launches else 0.0
+    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+            "launches": launches, "avg_us": round(avg_s * 1e6, 2),
+            "alg_bytes_per_launch": int(alg_bytes_per_launch)}
+
+
+# ------------------------------------------------------------------------------------
+# sparse_lr: configs[1]
+# ------------------------------------------------------------------------------------
+def gen_sparse_lr(steps, n, S):
+    limit = (KMAX // S) * S  # keys the stock ranges cover (postoffice.cc:169-180)
+    batches = []
+    for p in range(steps):
+        rng = np.random.default_rng(0xC0FFEE + p)
+        keys = unique_sorted_keys(rng, n, limit)
+        vals = rng.normal(0.0, 0.01, size=n).astype(np.float32)
+        batches.append((keys, vals))
+    return batches
+
+
+def run_sparse_lr(args, capi, dev):
+    import torch
+    n, S = args.keys or 1000000, 4
+    # the timed steps are followed by as many instrumented steps of the same shape
+    total_steps = args.warmup + 2 * args.steps
+    log("generating %d batches of %d keys" % (total_steps, n))
+    batches = gen_sparse_lr(total_steps, n, S)
+    rb, re = capi.server_ranges(S)
+    d_batches = [(to_dev(k, dev), to_dev(v, dev)) for k, v in batches]
+    out = torch.empty(n, dtype=torch.float32, device=dev)
+    # One table per server key range, sized for the keys the run will add. The tables
+    # share one stream: their kernels run back to back, each with the whole GPU, so a
+    # kernel's duration is its own and not that of four overlapping launches.
+    stream = torch.cuda.Stream()
+    cap = int(n * total_steps / S * 1.1)
+    tables = [capi.Table(capi.MODE_SCALAR, initial_capacity=cap, stream=stream.cuda_stream)
+              for _ in range(S)]
+
+    def step(i):
+        dk, dv = d_batches[i]
+        kp, vp, op = dk.data_ptr(), dv.data_ptr(), out.data_ptr()
+        pos, _, used = capi.slice_keys(dk, rb, re, nvals=n)
+        pos = [int(x) for x in pos]
+        for s in range(S):
+            if used[s]:
+                c = pos[s + 1] - pos[s]
+                tables[s].push_raw(kp + 8 * pos[s], c, vp + 4 * pos[s], c)
+        for s in range(S):
+            if used[s]:
+                c = pos[s + 1] - pos[s]
+                tables[s].pull_raw(kp + 8 * pos[s], c, op + 4 * pos[s], c)
+
+    def drain():
+        for t in tables:
+            t.sync()
+        torch.cuda.synchronize()
+
+    for i in range(args.warmup):
+        step(i)
+    drain()
+    t0 = time.perf_counter()
+    for i in range(args.warmup, args.warmup + args.steps):
+        step(i)
+    drain()
+    dt = time.perf_counter() - t0
+
+    # last pull must hold exactly the pushed values: each key was pushed once (0.0f + v)
+    last = args.warmup + args.steps - 1
+    want = batches[last][1] + np.float32(0.0)
+    got = out.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "pulled values differ"
+    held = sum(t.size()[0] for t in tables)
+    assert held == n * (args.warmup + args.steps), (held, n * (args.warmup + args.steps))
+
+    # Instrumented pass: the same steps continue with fresh keys while every launch of the
+    # store kernels is bracketed by HIP events on the stream it runs on. It is kept out of
+    # the timed region because an event pair per launch adds about 60 us to a 140 us step.
+    for t in tables:
+        t.prof_enable(True)
+        t.prof_reset()
+    for i in range(args.warmup + args.steps, total_steps):
+        step(i)
+    drain()
+    push_n, push_ms = kernel_stats(tables, capi.KERNEL_PUSH_SCALAR)
+    pull_n, pull_ms = kernel_stats(tables, capi.KERNEL_PULL_SCALAR)
+    for t in tables:
+        t.prof_enable(False)
+    keys_per_launch = n / S
+    res = {
+        "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
+        "dtype": "u64 keys, f32 values",
+        "config": {"workload": "sparse_lr: 1M sorted unique uint64 keys/step over 4 key ranges, "
+                               "push then pull, store grows by 1M keys/step", "keys_per_step": n,
+                   "ranges": S, "value_len": 1, "store_keys_after_timed_steps": held},
+        # every pushed key is new: 8 key + 4 val in, 8 slot read, 8 key + 4 val written
+        "roofline": dict(roofline(32.0 * keys_per_launch, push_n, push_ms),
+                         kernel="k_scalar<push> (find-or-insert + add)", bytes_per_key=32),
+        "kernels": {"pull_scalar": dict(roofline(24.0 * keys_per_launch, pull_n, pull_ms),
+                                        bytes_per_key=24)},
+    }
+    return res, batches[args.warmup:args.warmup + args.steps], (n, S)
+
+
+def cpu_sparse_lr(orc, batches, n, S, budget_s=25.0):
+    rb, re = orc.server_ranges(S)
+    stores = [orc.Store(orc.MODE_SCALAR) for _ in range(S)]
+    done = 0
+    t0 = time.perf_counter()
+    for keys, vals in batches:
+        pos, _, used = orc.slice_keys(keys, rb, re, nvals=n)
+        pos = pos.astype(np.int64)
+        for s in range(S):
+            if used[s]:
+                stores[s].push(keys[pos[s]:pos[s + 1]], vals[pos[s]:pos[s + 1]])
+        for s in range(S):
+            if used[s]:
+                stores[s].handle(False, True, keys[pos[s]:pos[s + 1]], out_cap=int(pos[s + 1] - pos[s]))
+        done += 1
+        if time.perf_counter() - t0 > budget_s:
+            break
+    dt = time.perf_counter() - t0
+    return {"value": 2.0 * n * done / dt, "unit": "keys/s", "cores": 1, "kind": "port",
+            "sample": "first %d of the timed steps (slice + push + pull of %d keys each), "
+                      "std::unordered_map store per range, one thread" % (done, n)}
+
+
+# ------------------------------------------------------------------------------------
+# dense: configs[2]
+# ------------------------------------------------------------------------------------
+def measure_dense(capi, dev, steps, warmup, nk=64, k=4194304):
+    """Returns (seconds for `steps` push+pull steps, accumulate stats, gather stats)."""
+    import torch
+    keys = to_dev(np.uint64(KMAX // nk) * np.arange(nk, dtype=np.uint64), dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(0xD15E)
+    vals = torch.rand(nk * k, device=dev, generator=g) * 2 - 1
+    out = torch.empty(nk * k, dtype=torch.float32, device=dev)
+    t = capi.Table(capi.MODE_FIXED, initial_capacity=1024, row_len=k, arena_floats=nk * k)
+    t.prof_enable(True)
+    t.push(keys, vals)  # first touch creates the rows
+    for _ in range(warmup):
+        t.push(keys, vals)
+        t.pull(keys, out)
+    t.sync()
+    t.prof_reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        t.push(keys, vals)
+        t.pull(keys, out)
+    t.sync()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    acc = t.prof_read(capi.KERNEL_ROWS_ACC)
+    gat = t.prof_read(capi.KERNEL_ROWS_GATHER)
+    # closed form: every float holds (1 + warmup + steps) * v, accumulated one add at a time
+    idx = torch.randint(0, nk * k, (4096,), device=dev)
+    ref = torch.zeros(4096, device=dev)
+    for _ in range(1 + warmup + steps):
+        ref = ref + vals[idx]
+    assert torch.equal(out[idx], ref), "dense sums differ from sequential float adds"
+    t.close()
+    return dt, acc, gat, nk, k
+
+
+def run_dense(args, capi, dev):
+    dt, acc, gat, nk, k = measure_dense(capi, dev, args.steps, args.warmup)
+    floats = nk * k
+    res = {
+        "value": 20.0 * floats * args.steps / dt / 1e9, "unit": "GB/s",
+        "ms_per_step": dt / args.steps * 1e3, "dtype": "f32",
+        "config": {"workload": "dense: 64 keys x 4,194,304 f32 (1 GiB), push-accumulate then full pull",
+                   "keys_per_step": nk, "value_len": k},
+        # 4 B in + 4 B row read + 4 B row write per float
+        "roofline": dict(roofline(12.0 * floats, acc[0], acc[1]),
+                         kernel="k_rows<acc,fixed> (row += in)", bytes_per_float=12),
+        "kernels": {"rows_gather": dict(roofline(8.0 * floats, gat[0], gat[1]), bytes_per_float=8)},
+    }
+    return res
+
+
+def cpu_dense(orc, nk=64, k=4194304, sample_keys=16):
+    rng = np.random.default_rng(0xD15E)
+    keys = (np.uint64(KMAX // nk) * np.arange(sample_keys, dtype=np.uint64))
+    vals = rng.uniform(-1, 1, size=sample_keys * k).astype(np.float32)
+    st = orc.Store(orc.MODE_FIXED, k)
+    st.push(keys, vals)
+    t0 = time.perf_counter()
+    reps = 0
+    while reps < 3 or time.perf_counter() - t0 < 10.0:
+        st.push(keys, vals)
+        st.handle(False, True, keys, out_cap=vals.size)
+        reps += 1
+    dt = time.perf_counter() - t0
+    return {"value": 20.0 * vals.size * reps / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "%d of the 64 rows (%d MiB), %d push+pull steps, one thread" % (
+                sample_keys, vals.size * 4 >> 20, reps)}
+
+
+# ------------------------------------------------------------------------------------
+# varlen: configs[4]
+# ------------------------------------------------------------------------------------
+def gen_varlen(n, S):
+    limit = (KMAX // S) * S
+    keys = unique_sorted_keys(np.random.default_rng(0xE3B), n, limit)
+    lens = np.random.default_rng(0xE3C).choice(np.array([8, 16, 32, 64, 128], np.int32), size=n)
+    return keys, lens.astype(np.int32)
+
+
+def run_varlen(args, capi, dev):
+    import torch
+    n, S = args.keys or 2000000, 16
+    keys, lens = gen_varlen(n, S)
+    nvals = int(lens.sum())
+    rb, re = capi.server_ranges(S)
+    dk, dl = to_dev(keys, dev), to_dev(lens, dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(0xE3D)
+    dv = torch.randn(nvals, device=dev, generator=g) * 0.1
+    out = torch.empty(nvals, dtype=torch.float32, device=dev)
+    out_lens = torch.empty(n, dtype=torch.int32, device=dev)
+    tables = [capi.Table(capi.MODE_VARLEN, initial_capacity=int(n / S * 1.2) * 4,
+                         arena_floats=int(nvals / S * 1.2)) for _ in range(S)]
+    for t in tables:
+        t.prof_enable(True)
+
+    def step():
+        pos, vpos, used = capi.slice_keys(dk, rb, re, lens=dl, nvals=nvals)
+        pos, vpos = pos.astype(np.int64), vpos.astype(np.int64)
+        for s in range(S):
+            if used[s]:
+                tables[s].push(dk[pos[s]:pos[s + 1]], dv[vpos[s]:vpos[s + 1]], dl[pos[s]:pos[s + 1]])
+        for s in range(S):
+            if used[s]:
+                tables[s].pull(dk[pos[s]:pos[s + 1]], out[vpos[s]:vpos[s + 1]], out_lens[pos[s]:pos[s + 1]])
+
+    step()  # creates the rows
+    for _ in range(args.warmup):
+        step()
+    for t in tables:
+        t.sync()
+        t.prof_reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    for t in tables:
+        t.sync()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert torch.equal(out_lens, dl), "pulled lens differ"
+    idx = torch.randint(0, nvals, (4096,), device=dev)
+    ref = torch.zeros(4096, device=dev)
+    for _ in range(1 + args.warmup + args.steps):
+        ref = ref + dv[idx]
+    assert torch.equal(out[idx], ref), "var-len sums differ from sequential float adds"
+    acc = kernel_stats(tables, capi.KERNEL_ROWS_ACC)
+    gat = kernel_stats(tables, capi.KERNEL_ROWS_GATHER)
+    floats_per_launch = nvals / S
+    res = {
+        "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
+        "dtype": "f32",
+        "config": {"workload": "varlen: 2M keys, lens in {8,16,32,64,128}, 16 key ranges, push then "
+                               "pull with lens", "keys_per_step": n, "floats_per_step": nvals,
+                   "ranges": S},
+        "gbps": (20.0 * nvals + 56.0 * n) * args.steps / dt / 1e9,
+        "roofline": dict(roofline(12.0 * floats_per_launch, acc[0], acc[1]),
+                         kernel="k_rows<acc,varlen> (row += in)", bytes_per_float=12),
+        "kernels": {"rows_gather": dict(roofline(8.0 * floats_per_launch, gat[0], gat[1]),
+                                        bytes_per_float=8)},
+    }
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="sparse_lr", choices=["sparse_lr", "dense", "varlen"])
+    ap.add_argument("--keys", type=int, default=0, help="keys per step (default: the config's)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the dense-chunk side measurement")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures ONE GPU: a table lives on one device and nothing here uses a "
+              "second one; run it with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    dev = torch.device("cuda:0")
+    capi = graft.load_package().capi
+    capi.load()  # raises if libpskv.so is missing: there is no other path
+
+    if args.workload == "sparse_lr":
+        res, timed_batches, (n, S) = run_sparse_lr(args, capi, dev)
+    elif args.workload == "dense":
+        res = run_dense(args, capi, dev)
+    else:
+        res = run_varlen(args, capi, dev)
+
+    extra = {}
+    if args.workload == "sparse_lr" and not args.no_extra:
+        # the dense-chunk kernels carry the bandwidth target of this path; measure them
+        # beside the default workload (10 push+pull steps of 1 GiB, well under a second)
+        dt, acc, gat, nk, k = measure_dense(capi, dev, 10, 2)
+        extra["dense_chunk"] = {
+            "rows_acc": dict(roofline(12.0 * nk * k, acc[0], acc[1]), bytes_per_float=12),
+            "rows_gather": dict(roofline(8.0 * nk * k, gat[0], gat[1]), bytes_per_float=8),
+        }
+
+    cpu = None
+    if not args.no_cpu:
+        orc = graft.load_oracle()
+        log("timing the CPU oracle (bounded sample)")
+        if args.workload == "sparse_lr":
+            cpu = cpu_sparse_lr(orc, timed_batches, n, S)
+        elif args.workload == "dense":
+            cpu = cpu_dense(orc)
+        else:
+            cpu = None  # the sparse and dense legs bracket it; timed in tests only
+
+    line = {
+        "metric": "push+pull keys/sec and achieved GB/s (% of HBM peak) on 1 MI355X",
+        "value": res["value"], "unit": res["unit"], "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": res["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": res["dtype"], "data": "synthetic",
+        "config": res["config"], "roofline": res["roofline"], "cpu_baseline": cpu,
+        "kernels": res.get("kernels"),
+    }
+    if "gbps" in res:
+        line["gbps"] = res["gbps"]
+    if extra:
+        line["extra"] = extra
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

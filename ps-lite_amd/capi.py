@@ -180,6 +180,14 @@ class Table:
         _check(rc)
         return got.value
 
+    def push_raw(self, keys_ptr, n, vals_ptr, nvals, lens_ptr=None, nlens=0):
+        """pskv_push on raw device addresses (no per-call tensor bookkeeping)."""
+        _check(self._lib.pskv_push(self._h, keys_ptr, n, vals_ptr, nvals, lens_ptr, nlens, MEM_DEVICE))
+
+    def pull_raw(self, keys_ptr, n, out_ptr, out_cap, out_lens_ptr=None):
+        _check(self._lib.pskv_pull(self._h, keys_ptr, n, out_ptr, out_cap, out_lens_ptr, None,
+                                   MEM_DEVICE))
+
     def sync(self):
         _check(self._lib.pskv_sync(self._h))
 

@@ -35,8 +35,13 @@ struct __align__(16) Slot {
   uint64_t payload;  // SCALAR: float bits in the low word; row modes: see above (without bit 63)
 };
 
+// Counters that every workgroup bumps are spread over kCountShards cache lines:
+// atomics on one address are served one at a time, and a request can run thousands
+// of workgroups.
+constexpr int kCountShards = 32;
+constexpr int kShardStride = 16;  // in 8-byte words: one shard per 128-byte line
+
 struct DevState {
-  unsigned long long count;            // keys held (slot array plus the side slot)
   unsigned long long arena_top;        // FIXED: rows handed out; VARLEN: 16-byte units handed out
   unsigned long long special_payload;  // payload of key 2^64-1
   unsigned long long scan_total;       // grand total of the last lens scan
@@ -44,7 +49,56 @@ struct DevState {
   unsigned int error;                  // sticky error bits of finished requests
   unsigned int req_error;              // error bits of the request in flight
   unsigned int misaligned;             // OR of (len & 3) over the lens of the current request
+  // keys held (slot array plus the side slot) = sum of the shards
+  unsigned long long count_shard[kCountShards * kShardStride];
 };
+
+// Adds the workgroup's total of `x` to one shard of the key counter. Every thread of
+// the workgroup must call it. `red` holds kBlock/64 words of LDS.
+__device__ __forceinline__ void block_count_add(DevState* st, unsigned x, unsigned* red) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = x;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned t = 0;
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; ++w) t += red[w];
+    if (t) atomicAdd(&st->count_shard[(blockIdx.x % kCountShards) * kShardStride], (unsigned long long)t);
+  }
+}
+
+// Workgroup-wide exclusive prefix sum of `x` plus the workgroup total; every thread must
+// call it. `red` holds kBlock/64 + 1 words of LDS and may be reused after the next barrier.
+__device__ __forceinline__ unsigned long long block_excl_scan_u64(unsigned long long x,
+                                                                  unsigned long long* red,
+                                                                  unsigned long long& total) {
+  unsigned long long inc = x;
+  const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    unsigned long long y = __shfl_up(inc, d);
+    if (lane >= (unsigned)d) inc += y;
+  }
+  __syncthreads();
+  if (lane == 63) red[wave] = inc;
+  __syncthreads();
+  unsigned long long before = 0, t = 0;
+#pragma unroll
+  for (unsigned w = 0; w < kBlock / 64; ++w) {
+    if (w < wave) before += red[w];
+    t += red[w];
+  }
+  total = t;
+  return before + inc - x;
+}
+
+typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+
+// One 128-bit read of a slot (key and payload together).
+__device__ __forceinline__ u64x2 load_slot(const Slot* p) {
+  return *reinterpret_cast<const u64x2*>(p);
+}
 
 // murmur3 finaliser: full avalanche, so evenly spaced keys (kMaxKey/n*i) spread out
 __device__ __forceinline__ uint64_t mix64(uint64_t x) {
@@ -53,12 +107,6 @@ __device__ __forceinline__ uint64_t mix64(uint64_t x) {
   x ^= x >> 33;
   x *= 0xc4ceb9fe1a85ec53ull;
   x ^= x >> 33;
-  return x;
-}
-
-__device__ __forceinline__ unsigned wave_sum_u32(unsigned x) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
   return x;
 }
 
@@ -89,7 +137,7 @@ __device__ __forceinline__ uint64_t* find_or_insert(Slot* __restrict__ slots, ui
   }
   uint64_t h = mix64(key) & mask;
   for (uint64_t probes = 0; probes <= mask; ++probes) {
-    const ulonglong2 s = *reinterpret_cast<const ulonglong2*>(&slots[h]);
+    const u64x2 s = load_slot(&slots[h]);
     if (s.x == key) {
       seen = s.y;
       return &slots[h].payload;
@@ -121,7 +169,7 @@ __device__ __forceinline__ bool find_only(const Slot* __restrict__ slots, uint64
   }
   uint64_t h = mix64(key) & mask;
   for (uint64_t probes = 0; probes <= mask; ++probes) {
-    const ulonglong2 s = *reinterpret_cast<const ulonglong2*>(&slots[h]);
+    const u64x2 s = load_slot(&slots[h]);
     if (s.x == key) {
       payload = s.y;
       return true;

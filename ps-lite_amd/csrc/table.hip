@@ -7,6 +7,8 @@
 #include <string>
 #include <vector>
 
+#include <hip/hip_ext.h>
+
 #include "host_common.h"
 #include "scan.h"
 #include "table_kernels.h"
@@ -56,7 +58,8 @@ struct pskv_table {
 
   Slot* slots = nullptr;
   uint64_t cap = 0;        // slots, a power of two
-  uint64_t count_ub = 0;   // upper bound of DevState::count kept on the host
+  uint64_t count_ub = 0;   // upper bound of the key count kept on the host
+  uint64_t count = 0;      // key count at the last read_state()
   DevState* st = nullptr;  // device
   DevState* st_host = nullptr;  // pinned mirror for read-backs
 
@@ -82,28 +85,35 @@ struct pskv_table {
 namespace {
 
 // ---- profiling -------------------------------------------------------------------
-struct ProfScope {
-  pskv_table* t;
-  int kernel;
-  EventPair ev;
-  bool on;
-  ProfScope(pskv_table* t_, int kernel_) : t(t_), kernel(kernel_), on(t_->prof) {
-    if (!on) return;
+// Launches `kernel` on the table's stream. While profiling is on, the launch carries
+// a start and a stop event of its own (hipExtLaunchKernelGGL), which take the
+// begin/end timestamps of that very dispatch: the same clock a profiler reads,
+// without the idle time that events recorded around a launch would add.
+template <typename... KArgs, typename... Args>
+void launch(pskv_table* t, int prof_kernel, void (*kernel)(KArgs...), dim3 grid, dim3 block,
+            Args... args) {
+  if (t->prof && prof_kernel >= 0) {
+    EventPair ev;
+    bool have = false;
     if (!t->free_events.empty()) {
       ev = t->free_events.back();
       t->free_events.pop_back();
-    } else if (hipEventCreate(&ev.a) != hipSuccess || hipEventCreate(&ev.b) != hipSuccess) {
-      on = false;
+      have = true;
+    } else if (hipEventCreate(&ev.a) == hipSuccess) {
+      if (hipEventCreate(&ev.b) == hipSuccess) {
+        have = true;
+      } else {
+        (void)hipEventDestroy(ev.a);
+      }
+    }
+    if (have) {
+      hipExtLaunchKernelGGL(kernel, grid, block, 0, t->stream, ev.a, ev.b, 0, static_cast<KArgs>(args)...);
+      t->pending[prof_kernel].push_back(ev);
       return;
     }
-    (void)hipEventRecord(ev.a, t->stream);
   }
-  ~ProfScope() {
-    if (!on) return;
-    (void)hipEventRecord(ev.b, t->stream);
-    t->pending[kernel].push_back(ev);
-  }
-};
+  hipLaunchKernelGGL(kernel, grid, block, 0, t->stream, static_cast<KArgs>(args)...);
+}
 
 int prof_collect(pskv_table* t) {
   PSKV_HIP(hipStreamSynchronize(t->stream));
@@ -155,6 +165,9 @@ struct Carver {
 int read_state(pskv_table* t) {
   PSKV_HIP(hipMemcpyAsync(t->st_host, t->st, sizeof(DevState), hipMemcpyDeviceToHost, t->stream));
   PSKV_HIP(hipStreamSynchronize(t->stream));
+  uint64_t c = 0;
+  for (int i = 0; i < kCountShards; ++i) c += t->st_host->count_shard[i * kShardStride];
+  t->count = c;
   return PSKV_OK;
 }
 
@@ -189,7 +202,7 @@ int ensure_slots(pskv_table* t, uint64_t n) {
   }
   int rc = read_state(t);
   if (rc) return rc;
-  t->count_ub = t->st_host->count;
+  t->count_ub = t->count;
   if (t->mode != PSKV_MODE_SCALAR) {
     t->top_ub = t->st_host->arena_top;
   }
@@ -199,11 +212,8 @@ int ensure_slots(pskv_table* t, uint64_t n) {
     Slot* fresh = nullptr;
     rc = alloc_slots(want, &fresh, t->stream);
     if (rc) return rc;
-    {
-      ProfScope ps(t, PSKV_KERNEL_REHASH);
-      k_rehash<<<dim3(grid_for(t->cap, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(
-          t->slots, t->cap, fresh, want - 1, t->st);
-    }
+    launch(t, PSKV_KERNEL_REHASH, k_rehash, dim3(grid_for(t->cap, kBlock, kMaxGrid)), dim3(kBlock),
+           t->slots, t->cap, fresh, want - 1, t->st);
     PSKV_HIP(hipGetLastError());
     PSKV_HIP(hipStreamSynchronize(t->stream));
     PSKV_HIP(hipFree(t->slots));
@@ -268,17 +278,14 @@ int run_scalar(pskv_table* t, Request& r) {
   const dim3 grid(grid_for(r.n, kBlock, kMaxGrid)), block(kBlock);
   const uint64_t mask = t->cap - 1;
   if (r.push && r.pull) {
-    ProfScope ps(t, PSKV_KERNEL_PUSH_SCALAR);
-    k_scalar<true, true><<<grid, block, 0, t->stream>>>(t->slots, mask, t->st, r.keys, r.vals,
-                                                        r.out, r.n);
+    launch(t, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, true>, grid, block, t->slots, mask, t->st,
+           r.keys, r.vals, r.out, r.n);
   } else if (r.push) {
-    ProfScope ps(t, PSKV_KERNEL_PUSH_SCALAR);
-    k_scalar<true, false><<<grid, block, 0, t->stream>>>(t->slots, mask, t->st, r.keys, r.vals,
-                                                         nullptr, r.n);
+    launch(t, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, false>, grid, block, t->slots, mask, t->st,
+           r.keys, r.vals, (float*)nullptr, r.n);
   } else {
-    ProfScope ps(t, PSKV_KERNEL_PULL_SCALAR);
-    k_scalar<false, true><<<grid, block, 0, t->stream>>>(t->slots, mask, t->st, r.keys, nullptr,
-                                                         r.out, r.n);
+    launch(t, PSKV_KERNEL_PULL_SCALAR, k_scalar<false, true>, grid, block, t->slots, mask, t->st,
+           r.keys, (const float*)nullptr, r.out, r.n);
   }
   PSKV_HIP(hipGetLastError());
   return PSKV_OK;
@@ -289,11 +296,11 @@ int launch_rows(pskv_table* t, int op, const RowsParams& p) {
   if (p.total == 0) return PSKV_OK;
   const uint64_t ntiles = (p.total + kTileFloats - 1) / kTileFloats;
   if (ntiles > 0x7fffffffull) return set_error(PSKV_EINVAL, "request too large");
-  ProfScope ps(t, op == kOpAcc ? PSKV_KERNEL_ROWS_ACC : PSKV_KERNEL_ROWS_GATHER);
   if (op == kOpAcc) {
-    k_rows<kOpAcc, VARLEN><<<dim3((unsigned)ntiles), dim3(kBlock), 0, t->stream>>>(p);
+    launch(t, PSKV_KERNEL_ROWS_ACC, k_rows<kOpAcc, VARLEN>, dim3((unsigned)ntiles), dim3(kBlock), p);
   } else {
-    k_rows<kOpGather, VARLEN><<<dim3((unsigned)ntiles), dim3(kBlock), 0, t->stream>>>(p);
+    launch(t, PSKV_KERNEL_ROWS_GATHER, k_rows<kOpGather, VARLEN>, dim3((unsigned)ntiles),
+           dim3(kBlock), p);
   }
   PSKV_HIP(hipGetLastError());
   return PSKV_OK;
@@ -311,11 +318,8 @@ int run_fixed(pskv_table* t, Request& r) {
   if (rc) return rc;
   Carver c(t->ws.ptr);
   uint64_t* ref = c.take<uint64_t>(r.n);
-  {
-    ProfScope ps(t, PSKV_KERNEL_LOOKUP);
-    k_lookup_fixed<<<dim3(grid_for(r.n, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(
-        t->slots, t->cap - 1, t->st, r.keys, r.n, ref);
-  }
+  launch(t, PSKV_KERNEL_LOOKUP, k_lookup_fixed, dim3(grid_for(r.n, kBlock * kLookupItems, kMaxGrid)),
+         dim3(kBlock), t->slots, t->cap - 1, t->st, r.keys, r.n, ref);
   PSKV_HIP(hipGetLastError());
   RowsParams p{};
   p.arena = t->arena;
@@ -383,11 +387,9 @@ int run_varlen(pskv_table* t, Request& r) {
     if (rc) return rc;
     k_begin_request<<<dim3(1), dim3(1), 0, t->stream>>>(t->st);
     PSKV_HIP(launch_lens_scan(r.lens, r.n, off, part, t->st, PSKV_MAX_VARLEN_ROW, t->stream));
-    {
-      ProfScope ps(t, PSKV_KERNEL_LOOKUP);
-      k_lookup_var_push<<<kgrid, block, 0, t->stream>>>(t->slots, t->cap - 1, t->st, r.keys,
-                                                       r.lens, r.n, r.nvals, ref);
-    }
+    launch(t, PSKV_KERNEL_LOOKUP, k_lookup_var_push,
+           dim3(grid_for(r.n, kBlock * kLookupItems, kMaxGrid)), block, t->slots, t->cap - 1, t->st,
+           r.keys, r.lens, r.n, r.nvals, ref);
     PSKV_HIP(hipGetLastError());
     if (r.nvals) {
       rc = make_tile_keys(t, off, r.n, r.nvals, &p.tile_key);
@@ -410,11 +412,8 @@ int run_varlen(pskv_table* t, Request& r) {
       rc = report_device_errors(t);
       if (rc) return rc;
     }
-    {
-      ProfScope ps(t, PSKV_KERNEL_LOOKUP);
-      k_lookup_var_pull<<<kgrid, block, 0, t->stream>>>(t->slots, t->cap - 1, t->st, r.keys, r.n,
-                                                       ref, lens_out);
-    }
+    launch(t, PSKV_KERNEL_LOOKUP, k_lookup_var_pull, kgrid, block, (const Slot*)t->slots, t->cap - 1,
+           (const DevState*)t->st, r.keys, r.n, ref, lens_out);
     PSKV_HIP(hipGetLastError());
     k_begin_request<<<dim3(1), dim3(1), 0, t->stream>>>(t->st);
     PSKV_HIP(launch_lens_scan(lens_out, r.n, off, part, t->st, PSKV_MAX_VARLEN_ROW, t->stream));
@@ -693,7 +692,7 @@ int pskv_sync(pskv_table* t) {
   DeviceGuard guard(t->device);
   int rc = read_state(t);
   if (rc) return rc;
-  t->count_ub = t->st_host->count;
+  t->count_ub = t->count;
   if (t->mode != PSKV_MODE_SCALAR) t->top_ub = t->st_host->arena_top;
   return report_device_errors(t);
 }
@@ -704,7 +703,7 @@ int pskv_size(pskv_table* t, uint64_t* n_keys, uint64_t* n_vals) {
   DeviceGuard guard(t->device);
   int rc = read_state(t);
   if (rc) return rc;
-  const uint64_t nk = t->st_host->count;  // includes key 2^64-1 when present
+  const uint64_t nk = t->count;  // includes key 2^64-1 when present
   if (n_keys) *n_keys = nk;
   if (n_vals) {
     if (t->mode == PSKV_MODE_SCALAR) {
@@ -742,7 +741,7 @@ int pskv_dump(pskv_table* t, uint64_t* keys, int32_t* lens, size_t cap_keys, flo
                      (unsigned long long)nk, (unsigned long long)nv);
   if (nk == 0) return PSKV_OK;
   DeviceGuard guard(t->device);
-  const uint64_t in_slots = t->st_host->count - (t->st_host->special_present ? 1 : 0);
+  const uint64_t in_slots = t->count - (t->st_host->special_present ? 1 : 0);
   if (in_slots) {
     uint64_t* d_keys = nullptr;
     unsigned long long* d_counter = nullptr;

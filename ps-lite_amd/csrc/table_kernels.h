@@ -24,6 +24,7 @@ __global__ __launch_bounds__(kBlock) void k_scalar(Slot* __restrict__ slots, uin
                                                   const uint64_t* __restrict__ keys,
                                                   const float* __restrict__ vals,
                                                   float* __restrict__ out, uint64_t n) {
+  __shared__ unsigned red[kBlock / 64];
   unsigned created = 0;
   const uint64_t stride = (uint64_t)gridDim.x * kBlock;
   for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
@@ -41,8 +42,7 @@ __global__ __launch_bounds__(kBlock) void k_scalar(Slot* __restrict__ slots, uin
     if (PULL) out[i] = cur;
     created += is_new ? 1u : 0u;
   }
-  created = wave_sum_u32(created);
-  if ((threadIdx.x & 63) == 0 && created) atomicAdd(&st->count, (unsigned long long)created);
+  block_count_add(st, created, red);
 }
 
 // ---------------------------------------------------------------------------------
@@ -56,42 +56,61 @@ __global__ void k_begin_request(DevState* st) {
   st->misaligned = 0;
 }
 
+constexpr int kLookupItems = 4;  // keys per thread and round of the creating lookups
+
 // FIXED: find or create the row of every key. Push and pull both create
 // (pull of an absent key inserts a zero value, kv_app.h:457).
+// A round handles kBlock*kLookupItems keys, kLookupItems consecutive ones per thread:
+// every thread claims slots for its keys, then the workgroup takes the rows of all
+// created keys from the arena with ONE atomic add and a workgroup-wide scan hands them
+// out in request order, so rows of neighbouring keys are neighbours in the arena.
 __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slots, uint64_t mask,
                                                         DevState* st,
                                                         const uint64_t* __restrict__ keys,
                                                         uint64_t n, uint64_t* __restrict__ ref) {
+  __shared__ unsigned long long red[kBlock / 64];
+  __shared__ unsigned cred[kBlock / 64];
+  __shared__ unsigned long long s_first;
   unsigned created = 0;
-  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-  // uniform trip count per wavefront: the wave-wide scan below needs all 64 lanes
-  for (uint64_t base = (uint64_t)blockIdx.x * kBlock; base < n; base += stride) {
-    const uint64_t i = base + threadIdx.x;
-    const bool active = i < n;
-    bool is_new = false;
-    uint64_t seen = 0;
-    uint64_t* p = nullptr;
-    if (active) p = find_or_insert(slots, mask, st, keys[i], is_new, seen);
-    const unsigned long long need = (p && is_new) ? 1ull : 0ull;
-    const unsigned long long inc = wave_incl_scan_u64(need);
-    const unsigned long long tot = __shfl(inc, 63);
-    unsigned long long first = 0;
-    if ((threadIdx.x & 63) == 63 && tot) first = atomicAdd(&st->arena_top, tot);
-    first = __shfl(first, 63);
-    if (p) {
-      uint64_t row = seen;
-      if (is_new) {
-        row = first + inc - need;
-        *p = row;
-        ++created;
-      }
-      ref[i] = row | (is_new ? kRefNew : 0ull);
-    } else if (active) {
-      ref[i] = kRefAbsent;
+  constexpr uint64_t kRound = (uint64_t)kBlock * kLookupItems;
+  for (uint64_t base = (uint64_t)blockIdx.x * kRound; base < n; base += (uint64_t)gridDim.x * kRound) {
+    uint64_t* p[kLookupItems];
+    uint64_t seen[kLookupItems];
+    bool is_new[kLookupItems];
+    unsigned mine = 0;
+#pragma unroll
+    for (int j = 0; j < kLookupItems; ++j) {
+      const uint64_t i = base + (uint64_t)threadIdx.x * kLookupItems + j;
+      p[j] = nullptr;
+      is_new[j] = false;
+      seen[j] = 0;
+      if (i < n) p[j] = find_or_insert(slots, mask, st, keys[i], is_new[j], seen[j]);
+      mine += (p[j] && is_new[j]) ? 1u : 0u;
     }
+    unsigned long long total;
+    unsigned long long at = block_excl_scan_u64(mine, red, total);
+    if (threadIdx.x == 0 && total) s_first = atomicAdd(&st->arena_top, total);
+    __syncthreads();
+    at += total ? s_first : 0ull;
+#pragma unroll
+    for (int j = 0; j < kLookupItems; ++j) {
+      const uint64_t i = base + (uint64_t)threadIdx.x * kLookupItems + j;
+      if (i >= n) continue;
+      if (!p[j]) {
+        ref[i] = kRefAbsent;
+        continue;
+      }
+      uint64_t row = seen[j];
+      if (is_new[j]) {
+        row = at++;
+        *p[j] = row;
+      }
+      ref[i] = row | (is_new[j] ? kRefNew : 0ull);
+    }
+    created += mine;
+    __syncthreads();  // s_first and red are reused by the next round
   }
-  created = wave_sum_u32(created);
-  if ((threadIdx.x & 63) == 0 && created) atomicAdd(&st->count, (unsigned long long)created);
+  block_count_add(st, created, cred);
 }
 
 // VARLEN push: find or create; a created row gets ceil(len/4) 16-byte units of the
@@ -105,41 +124,61 @@ __global__ __launch_bounds__(kBlock) void k_lookup_var_push(
     if (blockIdx.x == 0 && threadIdx.x == 0) atomicOr(&st->req_error, kDevErrSizeMismatch);
     return;
   }
+  __shared__ unsigned long long red[kBlock / 64];
+  __shared__ unsigned cred[kBlock / 64];
+  __shared__ unsigned long long s_first;
   unsigned created = 0;
-  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-  for (uint64_t base = (uint64_t)blockIdx.x * kBlock; base < n; base += stride) {
-    const uint64_t i = base + threadIdx.x;
-    const bool active = i < n;
-    bool is_new = false;
-    uint64_t seen = 0;
-    uint64_t* p = nullptr;
-    uint64_t len = 0;
-    if (active) {
-      len = (uint64_t)(uint32_t)lens[i];
-      p = find_or_insert(slots, mask, st, keys[i], is_new, seen);
+  constexpr uint64_t kRound = (uint64_t)kBlock * kLookupItems;
+  for (uint64_t base = (uint64_t)blockIdx.x * kRound; base < n; base += (uint64_t)gridDim.x * kRound) {
+    uint64_t* p[kLookupItems];
+    uint64_t seen[kLookupItems];
+    uint64_t len[kLookupItems];
+    bool is_new[kLookupItems];
+    unsigned long long units = 0;
+    unsigned mine = 0;
+#pragma unroll
+    for (int j = 0; j < kLookupItems; ++j) {
+      const uint64_t i = base + (uint64_t)threadIdx.x * kLookupItems + j;
+      p[j] = nullptr;
+      is_new[j] = false;
+      seen[j] = 0;
+      len[j] = 0;
+      if (i < n) {
+        len[j] = (uint64_t)(uint32_t)lens[i];
+        p[j] = find_or_insert(slots, mask, st, keys[i], is_new[j], seen[j]);
+      }
+      if (p[j] && is_new[j]) {
+        units += (len[j] + 3) >> 2;
+        ++mine;
+      }
     }
-    const unsigned long long need = (p && is_new) ? ((len + 3) >> 2) : 0ull;
-    const unsigned long long inc = wave_incl_scan_u64(need);
-    const unsigned long long tot = __shfl(inc, 63);
-    unsigned long long first = 0;
-    if ((threadIdx.x & 63) == 63 && tot) first = atomicAdd(&st->arena_top, tot);
-    first = __shfl(first, 63);
-    if (p) {
-      uint64_t payload = seen;
-      if (is_new) {
-        payload = ((first + inc - need) << kLenBits) | len;
-        *p = payload;
-        ++created;
-      } else if ((payload & kLenMask) != len) {
+    unsigned long long total;
+    unsigned long long at = block_excl_scan_u64(units, red, total);
+    if (threadIdx.x == 0 && total) s_first = atomicAdd(&st->arena_top, total);
+    __syncthreads();
+    at += total ? s_first : 0ull;
+#pragma unroll
+    for (int j = 0; j < kLookupItems; ++j) {
+      const uint64_t i = base + (uint64_t)threadIdx.x * kLookupItems + j;
+      if (i >= n) continue;
+      if (!p[j]) {
+        ref[i] = kRefAbsent;
+        continue;
+      }
+      uint64_t payload = seen[j];
+      if (is_new[j]) {
+        payload = ((uint64_t)at << kLenBits) | len[j];
+        at += (len[j] + 3) >> 2;
+        *p[j] = payload;
+      } else if ((payload & kLenMask) != len[j]) {
         atomicOr(&st->req_error, kDevErrLenChanged);
       }
-      ref[i] = payload | (is_new ? kRefNew : 0ull);
-    } else if (active) {
-      ref[i] = kRefAbsent;
+      ref[i] = payload | (is_new[j] ? kRefNew : 0ull);
     }
+    created += mine;
+    __syncthreads();
   }
-  created = wave_sum_u32(created);
-  if ((threadIdx.x & 63) == 0 && created) atomicAdd(&st->count, (unsigned long long)created);
+  block_count_add(st, created, cred);
 }
 
 // VARLEN pull: an absent key answers length 0 and is not created.
