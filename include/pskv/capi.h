@@ -161,6 +161,16 @@ int pskv_prof_read(pskv_table* t, int kernel, uint64_t* launches, double* total_
  * copy ceiling next to the accumulate kernels. No counterpart in the reference. */
 int pskv_copy_probe(pskv_table* t, void* dst, const void* src, size_t bytes);
 
+/* Pinned host memory for request/response buffers handed to PSKV_MEM_HOST calls
+ * (copies to and from it run as DMA). pskv_host_free may be called from any thread
+ * and never blocks in the GPU runtime: it only returns the buffer to a free list, as
+ * a ps-lite response buffer is released on a transport thread
+ * (src/zmq_van.h:20-26,159-175; SArray::reset with a deleter, sarray.h:162-165).
+ * pskv_host_trim gives the free list back to the system. */
+void* pskv_host_alloc(size_t bytes);
+void pskv_host_free(void* ptr);
+int pskv_host_trim(void);
+
 /* Text of the last error on the calling thread ("" if none). */
 const char* pskv_last_error(void);
 /* "pskv <major>.<minor> gfx950" */

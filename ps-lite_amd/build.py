@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 REPO = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libpskv.so")
-SOURCES = ["table.hip", "slice.hip"]
+SOURCES = ["table.hip", "slice.hip", "hostmem.hip"]
 HEADERS = ["device_common.h", "host_common.h", "scan.h", "table_kernels.h"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -55,6 +55,20 @@ def build_lib(verbose=False):
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB]
     subprocess.run(cmd, check=True)
     return LIB
+
+
+HOST_TEST = os.path.join(HERE, "host", "test_kv_app_gpu")
+
+
+def build_host_test():
+    """Compiles the C++ program that drives the adapters of include/pskv/ps_adapters.h the
+    way tests/test_kv_app.cc of the reference drives ps-lite."""
+    cmd = ["g++", "-std=c++11", "-O2", "-Wall", "-I" + os.path.join(REPO, "include"),
+           os.path.join(HERE, "host", "test_kv_app_gpu.cc"), "-L" + HERE, "-lpskv",
+           "-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib", "-lamdhip64",
+           "-o", HOST_TEST]
+    subprocess.run(cmd, check=True)
+    return HOST_TEST
 
 
 def build_oracle():

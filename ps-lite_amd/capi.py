@@ -39,7 +39,8 @@ SYMBOLS = [
     "pskv_table_create", "pskv_table_destroy", "pskv_push", "pskv_pull", "pskv_pushpull",
     "pskv_sync", "pskv_size", "pskv_dump", "pskv_slice", "pskv_server_ranges",
     "pskv_assemble_pull", "pskv_prof_enable", "pskv_prof_reset", "pskv_prof_read",
-    "pskv_copy_probe", "pskv_last_error", "pskv_version",
+    "pskv_copy_probe", "pskv_host_alloc", "pskv_host_free", "pskv_host_trim", "pskv_last_error",
+    "pskv_version",
 ]
 
 
@@ -92,6 +93,10 @@ def load():
     lib.pskv_prof_reset.argtypes = [vp]
     lib.pskv_prof_read.argtypes = [vp, i32, ctypes.POINTER(u64), ctypes.POINTER(ctypes.c_double)]
     lib.pskv_copy_probe.argtypes = [vp, vp, vp, sz]
+    lib.pskv_host_alloc.argtypes = [sz]
+    lib.pskv_host_alloc.restype = vp
+    lib.pskv_host_free.argtypes = [vp]
+    lib.pskv_host_free.restype = None
     lib.pskv_last_error.restype = ctypes.c_char_p
     lib.pskv_version.restype = ctypes.c_char_p
     _lib = lib

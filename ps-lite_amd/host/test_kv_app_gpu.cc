@@ -1,0 +1,181 @@
+// The reference's key-value integration test (tests/test_kv_app.cc) run against the GPU
+// slicer and the GPU request handle through the in-process ps:: surface: the same
+// worker program, the same closed forms, plus the multi-float layouts and the failure
+// cases of the data path.
+//
+//   test_kv_app_gpu [num_servers]
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "pskv/ps_min.h"
+#include "pskv/ps_adapters.h"
+
+using namespace ps;
+
+static int g_failures = 0;
+#define EXPECT(cond)                                                        \
+  do {                                                                      \
+    if (!(cond)) {                                                          \
+      std::fprintf(stderr, "%s:%d: EXPECT failed: %s\n", __FILE__, __LINE__, #cond); \
+      ++g_failures;                                                         \
+    }                                                                       \
+  } while (0)
+
+static std::vector<std::unique_ptr<KVServer<float>>> StartServers(int app_id, int num, int mode) {
+  std::vector<std::unique_ptr<KVServer<float>>> servers;
+  for (int i = 0; i < num; ++i) {
+    servers.emplace_back(new KVServer<float>(app_id));
+    pskv_opts o = pskv_opts();
+    o.mode = mode;
+    o.initial_capacity = 1024;
+    servers.back()->set_request_handle(pskv::GpuKVHandle<float>(o));  // tests/test_kv_app.cc:10-11
+  }
+  return servers;
+}
+
+// tests/test_kv_app.cc:15-62
+static void RunWorker(int app_id, int num, bool ones) {
+  KVWorker<float> kv(app_id, 0);
+  kv.set_slicer(pskv::GpuSlicer<float>(0));
+  std::vector<Key> keys(num);
+  std::vector<float> vals(num);
+  const int rank = 0;
+  srand(rank + 7);
+  for (int i = 0; i < num; ++i) {
+    keys[i] = kMaxKey / num * i + rank;
+    vals[i] = ones ? 1.0f : static_cast<float>(rand() % 1000);
+  }
+  const int repeat = 50;
+  std::vector<int> ts;
+  for (int i = 0; i < repeat; ++i) {
+    ts.push_back(kv.Push(keys, vals));
+    if (i > 10) kv.Wait(ts[ts.size() - 10]);
+  }
+  for (int t : ts) kv.Wait(t);
+
+  std::vector<float> rets;
+  kv.Wait(kv.Pull(keys, &rets));
+
+  std::vector<float> outs;
+  for (int i = 0; i < repeat; ++i) kv.Wait(kv.PushPull(keys, vals, &outs));
+
+  float res = 0, res2 = 0;
+  for (int i = 0; i < num; ++i) {
+    res += std::fabs(rets[i] - vals[i] * repeat);
+    res2 += std::fabs(outs[i] - vals[i] * 2 * repeat);
+  }
+  EXPECT(rets.size() == static_cast<size_t>(num));
+  EXPECT(res / repeat < 1e-5);
+  EXPECT(res2 / (2 * repeat) < 1e-5);
+  // integer-valued floats below 2^24 add exactly, so the sums are not merely close
+  EXPECT(res == 0.0f && res2 == 0.0f);
+  std::printf("kv_app num=%d error: %g, %g\n", num, res / repeat, res2 / (2 * repeat));
+}
+
+// The example of kv_app.h:89-96: two keys with length-2 values.
+static void RunFixed() {
+  KVWorker<float> kv(1, 0);
+  kv.set_slicer(pskv::GpuSlicer<float>(0));
+  std::vector<Key> keys = {1, 3};
+  std::vector<float> vals = {1.1f, 1.2f, 3.1f, 3.2f};
+  kv.Wait(kv.Push(keys, vals));
+  kv.Wait(kv.Push(keys, vals));
+  std::vector<float> out;
+  kv.Wait(kv.Pull(keys, &out));
+  EXPECT(out.size() == 4);
+  for (size_t i = 0; i < out.size() && i < 4; ++i) EXPECT(out[i] == (0.0f + vals[i]) + vals[i]);
+  // keys spread over all servers, 3 floats each
+  const int num = 999;
+  std::vector<Key> k2(num);
+  std::vector<float> v2(num * 4);
+  for (int i = 0; i < num; ++i) k2[i] = kMaxKey / num * i + 5;
+  for (size_t i = 0; i < v2.size(); ++i) v2[i] = static_cast<float>(i % 17) - 8.0f;
+  KVWorker<float> kv2(2, 0);
+  kv2.set_slicer(pskv::GpuSlicer<float>(0));
+  for (int r = 0; r < 3; ++r) kv2.Wait(kv2.Push(k2, v2));
+  std::vector<float> o2;
+  kv2.Wait(kv2.Pull(k2, &o2));
+  EXPECT(o2.size() == v2.size());
+  for (size_t i = 0; i < o2.size() && i < v2.size(); ++i) EXPECT(o2[i] == 3 * v2[i]);
+}
+
+// Values of different lengths with lens (KVPairs layout, kv_app.h:24-31).
+static void RunVarLen() {
+  KVWorker<float> kv(3, 0);
+  kv.set_slicer(pskv::GpuSlicer<float>(0));
+  const int num = 2000;
+  const int choices[5] = {8, 16, 32, 64, 128};
+  std::vector<Key> keys(num);
+  std::vector<int> lens(num);
+  size_t total = 0;
+  for (int i = 0; i < num; ++i) {
+    keys[i] = kMaxKey / num * i + 11;
+    lens[i] = choices[(i * 7) % 5];
+    total += lens[i];
+  }
+  std::vector<float> vals(total);
+  for (size_t i = 0; i < total; ++i) vals[i] = static_cast<float>(i % 29) - 14.0f;
+  for (int r = 0; r < 4; ++r) kv.Wait(kv.Push(keys, vals, lens));
+  std::vector<float> out;
+  std::vector<int> out_lens;
+  kv.Wait(kv.Pull(keys, &out, &out_lens));
+  EXPECT(out.size() == total);
+  EXPECT(out_lens == lens);
+  for (size_t i = 0; i < out.size() && i < total; ++i) EXPECT(out[i] == 4 * vals[i]);
+}
+
+static void RunFailures(int num_servers) {
+  KVWorker<float> kv(0, 1);
+  kv.set_slicer(pskv::GpuSlicer<float>(0));
+  // the top keys are covered by no server range (src/postoffice.cc:169-180): kv_app.h:542 fails
+  std::vector<Key> keys = {5, kMaxKey - 1};
+  std::vector<float> vals = {1.0f, 2.0f};
+  if ((kMaxKey / num_servers) * num_servers <= kMaxKey - 1) {
+    bool thrown = false;
+    try {
+      kv.Push(keys, vals);
+    } catch (const dmlc::Error& e) {
+      thrown = true;
+      std::printf("expected failure: %s\n", e.what());
+    }
+    EXPECT(thrown);
+  }
+  // 3 values for 2 keys: kv_app.h:549
+  bool thrown = false;
+  try {
+    kv.Push({5, 6}, {1.0f, 2.0f, 3.0f});
+  } catch (const dmlc::Error&) {
+    thrown = true;
+  }
+  EXPECT(thrown);
+}
+
+int main(int argc, char** argv) {
+  const int num_servers = argc > 1 ? std::atoi(argv[1]) : 1;
+  try {
+    Postoffice::Get()->set_num_servers(num_servers);
+    auto s0 = StartServers(0, num_servers, PSKV_MODE_SCALAR);
+    auto s1 = StartServers(1, num_servers, PSKV_MODE_FIXED);
+    auto s2 = StartServers(2, num_servers, PSKV_MODE_FIXED);
+    auto s3 = StartServers(3, num_servers, PSKV_MODE_VARLEN);
+    auto s4 = StartServers(4, num_servers, PSKV_MODE_SCALAR);
+    RunWorker(0, 1000, true);     // 1,000 keys, all 1.0: pull == 50.0f
+    RunWorker(4, 10000, false);   // the reference's own sizes and values, on a fresh store
+    RunFixed();
+    RunVarLen();
+    RunFailures(num_servers);
+  } catch (const std::exception& e) {
+    std::fprintf(stderr, "unexpected exception: %s\n", e.what());
+    return 2;
+  }
+  if (g_failures) {
+    std::fprintf(stderr, "%d expectation(s) failed\n", g_failures);
+    return 1;
+  }
+  std::printf("test_kv_app_gpu: ok (%d server%s)\n", num_servers, num_servers == 1 ? "" : "s");
+  return 0;
+}

@@ -1,0 +1,23 @@
+"""Runs the C++ program that drives the GPU slicer and the GPU request handle through the
+ps::KVWorker / ps::KVServer interface the way tests/test_kv_app.cc of the reference does."""
+import os
+import subprocess
+
+import pytest
+
+from conftest import REPO, announce
+
+pytestmark = pytest.mark.gpu
+
+BIN = os.path.join(REPO, "ps-lite_amd", "host", "test_kv_app_gpu")
+
+
+@pytest.mark.parametrize("num_servers", [1, 2, 4])
+def test_kv_app_through_adapters(num_servers):
+    announce("kv_app_through_adapters", num_servers)
+    assert os.path.exists(BIN), "build() compiles ps-lite_amd/host/test_kv_app_gpu"
+    r = subprocess.run([BIN, str(num_servers)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                       text=True, timeout=100)
+    print(r.stdout)
+    assert r.returncode == 0, r.stdout
+    assert "test_kv_app_gpu: ok" in r.stdout
