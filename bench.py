@@ -228,6 +228,10 @@ def measure_dense(capi, dev, steps, warmup, nk=64, k=4194304):
     for _ in range(1 + warmup + steps):
         ref = ref + vals[idx]
     assert torch.equal(out[idx], ref), "dense sums differ from sequential float adds"
+    # one plain copy of the same 1 GiB: the known-size launch that memory-traffic counters are
+    # scaled by, and the copy ceiling next to the accumulate kernel
+    t.copy_probe(out, vals)
+    t.sync()
     t.close()
     return dt, acc, gat, nk, k
 
