@@ -1,0 +1,228 @@
+"""The five BASELINE configurations at their full sizes on the GPU, bit-exact against the CPU
+oracle on the same seeded inputs (each oracle leg finishes in seconds), plus size-independent
+properties: exact integer sums, stored-key sets, idempotent pulls, slice/reassembly round trips."""
+import numpy as np
+import pytest
+
+from conftest import announce
+from helpers import KMAX, assert_bits_equal, covered_limit, from_dev, to_dev, unique_keys
+
+pytestmark = pytest.mark.gpu
+
+
+def _slices(capi, dk, rb, re, dl=None, nvals=0):
+    pos, vpos, used = capi.slice_keys(dk, rb, re, lens=dl, nvals=nvals)
+    return [int(x) for x in pos], [int(x) for x in vpos], used
+
+
+def test_config1_plumbing_shape(capi, orc, dev):
+    """1,000 keys spread evenly over the key range, all 1.0, 50 pushes then a pull, one server."""
+    import torch
+    announce("config1")
+    n = 1000
+    keys = np.uint64(KMAX // n) * np.arange(n, dtype=np.uint64)
+    vals = np.ones(n, np.float32)
+    rb, re = capi.server_ranges(1)
+    dk, dv = to_dev(keys, dev), to_dev(vals, dev)
+    t = capi.Table(capi.MODE_SCALAR)
+    o = orc.Store(orc.MODE_SCALAR)
+    for _ in range(50):
+        pos, _, used = _slices(capi, dk, rb, re, nvals=n)
+        assert pos == [0, n] and used[0] == 1
+        t.push(dk, dv)
+        o.push(keys, vals)
+    out = torch.zeros(n, dtype=torch.float32, device=dev)
+    t.pull(dk, out)
+    t.sync()
+    assert np.all(from_dev(out) == np.float32(50.0))
+    assert_bits_equal(from_dev(out), o.pull(keys)[0], "config1")
+
+
+def test_config2_sparse_lr_full(capi, orc, dev):
+    """20 pushes of 1M fresh uniform keys over 4 ranges (store grows to 20M), then pulls."""
+    import torch
+    announce("config2 full size")
+    n, S, pushes = 1000000, 4, 20
+    rb, re = capi.server_ranges(S)
+    tables = [capi.Table(capi.MODE_SCALAR, initial_capacity=1 << 20) for _ in range(S)]  # grows 3 times
+    stores = [orc.Store(orc.MODE_SCALAR) for _ in range(S)]
+    all_keys = []
+    for p in range(pushes):
+        rng = np.random.default_rng(0xC0FFEE + p)
+        keys = unique_keys(rng, n, S)
+        vals = rng.normal(0, 0.01, size=n).astype(np.float32)
+        all_keys.append(keys)
+        dk, dv = to_dev(keys, dev), to_dev(vals, dev)
+        pos, _, used = _slices(capi, dk, rb, re, nvals=n)
+        o_pos, _, o_used = orc.slice_keys(keys, rb, re, nvals=n)
+        assert pos == [int(x) for x in o_pos] and np.array_equal(used, o_used)
+        for s in range(S):
+            tables[s].push(dk[pos[s]:pos[s + 1]], dv[pos[s]:pos[s + 1]])
+            stores[s].push(keys[pos[s]:pos[s + 1]], vals[pos[s]:pos[s + 1]])
+        for t in tables:
+            t.sync()  # dk/dv are released after this iteration
+    # pull of the last push's keys, then of a mix of old keys and absent keys (which get created)
+    rng = np.random.default_rng(5)
+    mix = np.unique(np.concatenate([rng.choice(np.concatenate(all_keys[:5]), size=500000, replace=False),
+                                    unique_keys(rng, 200000, S)]))
+    for probe in (all_keys[-1], mix):
+        dk = to_dev(probe, dev)
+        out = torch.empty(probe.size, dtype=torch.float32, device=dev)
+        pos, _, used = _slices(capi, dk, rb, re, nvals=0)
+        want = np.empty(probe.size, np.float32)
+        for s in range(S):
+            tables[s].pull(dk[pos[s]:pos[s + 1]], out[pos[s]:pos[s + 1]])
+            want[pos[s]:pos[s + 1]] = stores[s].pull(probe[pos[s]:pos[s + 1]])[0]
+        for t in tables:
+            t.sync()
+        assert_bits_equal(from_dev(out), want, "config2 pull")
+    for s in range(S):
+        assert tables[s].size() == stores[s].size()
+    gk, _, gv = tables[1].dump()
+    ok, _, ov = stores[1].dump()
+    assert np.array_equal(gk, ok)
+    assert_bits_equal(gv, ov, "config2 dump of range 1")
+
+
+def test_config3_dense_chunks_full(capi, orc, dev):
+    """64 keys x 4,194,304 f32 (1 GiB per push), 8 worker pushes in fixed order, one full pull."""
+    import torch
+    announce("config3 full size")
+    nk, k, workers = 64, 4194304, 8
+    keys = np.uint64(KMAX // nk) * np.arange(nk, dtype=np.uint64)
+    dk = to_dev(keys, dev)
+    t = capi.Table(capi.MODE_FIXED, row_len=k, arena_floats=nk * k)
+    o = orc.Store(orc.MODE_FIXED, k)
+    for w in range(workers):
+        vals = np.random.default_rng(0xD15E + w).uniform(-1, 1, size=nk * k).astype(np.float32)
+        dv = to_dev(vals, dev)
+        t.push(dk, dv)
+        o.push(keys, vals)
+        t.sync()
+        del dv
+    out = torch.empty(nk * k, dtype=torch.float32, device=dev)
+    assert t.pull(dk, out) == nk * k
+    t.sync()
+    want = np.empty(nk * k, np.float32)
+    rc, want, _, _ = o.handle(False, True, keys, out_cap=nk * k)
+    assert rc == 0
+    assert_bits_equal(from_dev(out), want, "config3")
+    assert t.size() == (nk, nk * k)
+
+
+def _zipf_unique(rng, n, universe, s=1.1):
+    """n distinct ranks in [0, universe) with Zipf(s) popularity, sorted."""
+    got = np.zeros(0, np.int64)
+    while got.size < n:
+        r = rng.zipf(s, size=2 * n).astype(np.int64) - 1
+        got = np.unique(np.concatenate([got, r[(r >= 0) & (r < universe)]]))
+    if got.size > n:
+        got = np.sort(rng.choice(got, size=n, replace=False))
+    return got
+
+
+def _rank_to_key(r):
+    """An injective scatter of ranks over the covered key space (odd multiplier mod 2^64, then >> 1)."""
+    return ((r.astype(np.uint64) * np.uint64(0x9E3779B97F4A7C15)) >> np.uint64(1)).astype(np.uint64)
+
+
+@pytest.mark.parametrize("scale", [8, 1])
+def test_config4_zipf(capi, orc, dev, scale):
+    """8 worker pushes of Zipf(1.1)-popular keys from a 100M-key universe, then a pull of Zipf keys
+    of which many are absent. scale=8 is compared with the oracle float for float; scale=1 (4M keys
+    per push, 16M pulled) uses small-integer values, whose sums are exact in any order, against numpy."""
+    import torch
+    announce("config4", scale)
+    universe, n_push, n_pull, workers = 100000000 // scale, 4000000 // scale, 16000000 // scale, 8
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=1 << 20)
+    o = orc.Store(orc.MODE_SCALAR) if scale > 1 else None
+    pushed_ranks, pushed_vals = [], []
+    for w in range(workers):
+        rng = np.random.default_rng(0x21F + w)
+        ranks = _zipf_unique(rng, n_push, universe)
+        keys = np.sort(_rank_to_key(ranks))
+        vals = rng.standard_normal(n_push).astype(np.float32) if scale > 1 else \
+            rng.integers(-500, 500, size=n_push).astype(np.float32)
+        assert np.all(np.diff(keys.astype(np.int64 if keys.max() < 2 ** 63 else np.uint64)) != 0)
+        t.push(to_dev(keys, dev), to_dev(vals, dev))
+        t.sync()
+        if o:
+            o.push(keys, vals)
+        else:
+            pushed_ranks.append(keys)
+            pushed_vals.append(vals)
+    rng = np.random.default_rng(0x9011)
+    probe = np.sort(_rank_to_key(_zipf_unique(rng, n_pull, universe)))
+    dk = to_dev(probe, dev)
+    out = torch.empty(probe.size, dtype=torch.float32, device=dev)
+    t.pull(dk, out)
+    t.sync()
+    got = from_dev(out)
+    if o:
+        assert_bits_equal(got, o.pull(probe)[0], "config4")
+        assert t.size() == o.size()
+        gk, _, gv = t.dump()
+        ok, _, ov = o.dump()
+        assert np.array_equal(gk, ok)
+        assert_bits_equal(gv, ov, "config4 dump")
+    else:
+        allk = np.concatenate(pushed_ranks)
+        allv = np.concatenate(pushed_vals).astype(np.int64)
+        order = np.argsort(allk, kind="stable")
+        allk, allv = allk[order], allv[order]
+        uk, start = np.unique(allk, return_index=True)
+        sums = np.add.reduceat(allv, start)
+        idx = np.searchsorted(uk, probe)
+        idx[idx == uk.size] = 0
+        hit = uk[idx] == probe
+        want = np.where(hit, sums[idx], 0).astype(np.float32)
+        assert np.array_equal(got, want)
+        # a pull creates the absent keys: the store now holds the union
+        assert t.size()[0] == np.union1d(uk, probe).size
+        # pulling again changes nothing
+        out2 = torch.empty_like(out)
+        t.pull(dk, out2)
+        t.sync()
+        assert torch.equal(out, out2)
+
+
+def test_config5_varlen_rows_full(capi, orc, dev):
+    """2M keys with lens in {8,16,32,64,128} over 16 ranges, 10 pushes, then a pull with lens."""
+    import torch
+    announce("config5 full size")
+    n, S, pushes = 2000000, 16, 10
+    rb, re = capi.server_ranges(S)
+    keys = unique_keys(np.random.default_rng(0xE3B), n, S)
+    lens = np.random.default_rng(0xE3C).choice(np.array([8, 16, 32, 64, 128], np.int32), size=n).astype(np.int32)
+    nvals = int(lens.sum())
+    dk, dl = to_dev(keys, dev), to_dev(lens, dev)
+    pos, vpos, used = _slices(capi, dk, rb, re, dl, nvals)
+    o_pos, o_vpos, o_used = orc.slice_keys(keys, rb, re, lens, nvals)
+    assert pos == [int(x) for x in o_pos] and vpos == [int(x) for x in o_vpos]
+    tables = [capi.Table(capi.MODE_VARLEN, initial_capacity=n // S) for _ in range(S)]
+    o = orc.Store(orc.MODE_VARLEN)  # one oracle store: the ranges are disjoint
+    for p in range(pushes):
+        vals = np.random.default_rng(0xE3D + p).normal(0, 0.1, size=nvals).astype(np.float32)
+        dv = to_dev(vals, dev)
+        for s in range(S):
+            tables[s].push(dk[pos[s]:pos[s + 1]], dv[vpos[s]:vpos[s + 1]], dl[pos[s]:pos[s + 1]])
+        o.push(keys, vals, lens)
+        for t in tables:
+            t.sync()
+    out = torch.empty(nvals, dtype=torch.float32, device=dev)
+    out_lens = torch.empty(n, dtype=torch.int32, device=dev)
+    responses = []
+    for s in range(S):
+        ks = dk[pos[s]:pos[s + 1]]
+        part = torch.empty(vpos[s + 1] - vpos[s], dtype=torch.float32, device=dev)
+        part_lens = torch.empty(ks.numel(), dtype=torch.int32, device=dev)
+        assert tables[s].pull(ks, part, part_lens) == part.numel()
+        responses.append((ks, part, part_lens))
+    for t in tables:
+        t.sync()
+    assert capi.assemble_pull(dk, responses[::-1], out, out_lens) == nvals
+    want, want_lens = o.pull(keys)
+    assert np.array_equal(from_dev(out_lens), want_lens)
+    assert_bits_equal(from_dev(out), want, "config5")
+    assert sum(t.size()[0] for t in tables) == n
+    assert sum(t.size()[1] for t in tables) == nvals
