@@ -4,6 +4,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#ifndef PSKV_TILE_VAR
+#define PSKV_TILE_VAR 2048
+#endif
+
 namespace pskv {
 
 // ps::kMaxKey (include/ps/base.h:18). The stock server ranges never cover it
@@ -27,7 +31,6 @@ constexpr unsigned kDevErrBadLen = 4u;      // negative or too long length
 constexpr unsigned kDevErrSizeMismatch = 8u;  // lens do not add up to the number of values
 
 constexpr int kBlock = 256;             // threads per workgroup of every kernel here (4 waves)
-constexpr unsigned kTileFloats = 4096;  // request-side floats handled by one workgroup of the row kernels
 constexpr unsigned kSpanMax = 1024;     // keys whose offsets a row-kernel workgroup stages in LDS
 
 struct __align__(16) Slot {

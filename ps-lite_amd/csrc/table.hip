@@ -291,16 +291,24 @@ int run_scalar(pskv_table* t, Request& r) {
   return PSKV_OK;
 }
 
+// Requests at least this large are streamed with non-temporal accesses: they cannot stay
+// in the 256 MB last-level cache between two requests anyway.
+constexpr uint64_t kStreamFloats = 16u << 20;
+
 template <bool VARLEN>
 int launch_rows(pskv_table* t, int op, const RowsParams& p) {
   if (p.total == 0) return PSKV_OK;
-  const uint64_t ntiles = (p.total + kTileFloats - 1) / kTileFloats;
+  const uint64_t tile = VARLEN ? kTileVar : kTileFixed;
+  const uint64_t ntiles = (p.total + tile - 1) / tile;
   if (ntiles > 0x7fffffffull) return set_error(PSKV_EINVAL, "request too large");
+  const dim3 grid((unsigned)ntiles), block(kBlock);
+  const bool stream = p.total >= kStreamFloats;
   if (op == kOpAcc) {
-    launch(t, PSKV_KERNEL_ROWS_ACC, k_rows<kOpAcc, VARLEN>, dim3((unsigned)ntiles), dim3(kBlock), p);
+    if (stream) launch(t, PSKV_KERNEL_ROWS_ACC, k_rows<kOpAcc, VARLEN, true>, grid, block, p);
+    else launch(t, PSKV_KERNEL_ROWS_ACC, k_rows<kOpAcc, VARLEN, false>, grid, block, p);
   } else {
-    launch(t, PSKV_KERNEL_ROWS_GATHER, k_rows<kOpGather, VARLEN>, dim3((unsigned)ntiles),
-           dim3(kBlock), p);
+    if (stream) launch(t, PSKV_KERNEL_ROWS_GATHER, k_rows<kOpGather, VARLEN, true>, grid, block, p);
+    else launch(t, PSKV_KERNEL_ROWS_GATHER, k_rows<kOpGather, VARLEN, false>, grid, block, p);
   }
   PSKV_HIP(hipGetLastError());
   return PSKV_OK;
@@ -348,11 +356,12 @@ int run_fixed(pskv_table* t, Request& r) {
 // Grows the tile table to `total` request-side floats and fills it.
 int make_tile_keys(pskv_table* t, const uint64_t* off, uint64_t n, uint64_t total,
                    const uint32_t** tile_key) {
-  const uint64_t ntiles = (total + kTileFloats - 1) / kTileFloats;
+  const uint64_t ntiles = (total + kTileVar - 1) / kTileVar;
   int rc = grow(t, &t->tiles, (ntiles + 1) * sizeof(uint32_t));
   if (rc) return rc;
   uint32_t* tk = static_cast<uint32_t*>(t->tiles.ptr);
-  k_tile_keys<<<dim3(grid_for(n, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(off, n, tk, ntiles);
+  k_tile_keys<<<dim3(grid_for(n, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(off, n, tk, ntiles,
+                                                                                  (uint64_t)kTileVar);
   PSKV_HIP(hipGetLastError());
   *tile_key = tk;
   return PSKV_OK;
@@ -814,8 +823,9 @@ int pskv_copy_probe(pskv_table* t, void* dst, const void* src, size_t bytes) {
   if (!bytes) return PSKV_OK;
   DeviceGuard guard(t->device);
   const uint64_t n16 = bytes / 16;
-  k_copy<<<dim3(grid_for(n16, kBlock * 4, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(
-      static_cast<float4*>(dst), static_cast<const float4*>(src), n16);
+  if ((n16 + kBlock - 1) / kBlock > 0x7fffffffull) return set_error(PSKV_EINVAL, "copy too large");
+  k_copy<<<dim3((unsigned)((n16 + kBlock - 1) / kBlock)), dim3(kBlock), 0, t->stream>>>(
+      static_cast<f32x4*>(dst), static_cast<const f32x4*>(src), n16);
   PSKV_HIP(hipGetLastError());
   return PSKV_OK;
 }
