@@ -3,6 +3,8 @@
 // table_kernels.h in request order on one stream. This is what a ps-lite server
 // calls in place of KVServerDefaultHandle (include/ps/kv_app.h:440-463).
 #include <algorithm>
+#include <atomic>
+#include <cstring>
 #include <new>
 #include <string>
 #include <vector>
@@ -44,6 +46,27 @@ struct EventPair {
   hipEvent_t a, b;
 };
 
+// Counters of the table as of the start of request `seq`, written by the device into
+// pinned host memory. seq_begin == seq_end marks a consistent record.
+struct Snapshot {
+  volatile uint64_t seq_begin;
+  volatile uint64_t count;
+  volatile uint64_t arena_top;
+  volatile uint64_t seq_end;
+};
+
+// One thread, launched in front of a request's kernels when the table is close to a limit.
+__global__ void k_publish(const DevState* st, Snapshot* out, uint64_t seq) {
+  unsigned long long c = 0;
+  for (int i = 0; i < kCountShards; ++i) c += st->count_shard[i * kShardStride];
+  out->seq_begin = seq;
+  __threadfence_system();
+  out->count = c;
+  out->arena_top = st->arena_top;
+  __threadfence_system();
+  out->seq_end = seq;
+}
+
 }  // namespace
 }  // namespace pskv
 
@@ -58,15 +81,25 @@ struct pskv_table {
 
   Slot* slots = nullptr;
   uint64_t cap = 0;        // slots, a power of two
-  uint64_t count_ub = 0;   // upper bound of the key count kept on the host
   uint64_t count = 0;      // key count at the last read_state()
+
+  // Host-side bounds of what the device counters can have reached. Requests are enqueued
+  // without waiting, so the host only knows exact counters (`base_*`) as of request
+  // `base_seq` and must assume that every key of a later request was new (`pend_*`).
+  // A published snapshot (below) moves the base forward without a stream wait.
+  uint64_t seq = 0;        // requests begun so far
+  uint64_t base_seq = 0;   // base_count / base_top hold after all requests < base_seq
+  uint64_t base_count = 0, base_top = 0;
+  uint64_t pend_keys = 0, pend_units = 0;  // sums of the log over [base_seq, seq)
+  static const int kLog = 64;
+  uint64_t log_keys[kLog] = {0}, log_units[kLog] = {0};
+  Snapshot* snap = nullptr;  // pinned host memory the device publishes into
   DevState* st = nullptr;  // device
   DevState* st_host = nullptr;  // pinned mirror for read-backs
 
   // row modes
   float* arena = nullptr;
   uint64_t arena_cap = 0;  // floats
-  uint64_t top_ub = 0;     // upper bound of DevState::arena_top (rows or 16-byte units)
   uint64_t row_len = 0;    // FIXED
 
   GrowBuf ws;         // per-request workspace (row references, offsets)
@@ -168,6 +201,11 @@ int read_state(pskv_table* t) {
   uint64_t c = 0;
   for (int i = 0; i < kCountShards; ++i) c += t->st_host->count_shard[i * kShardStride];
   t->count = c;
+  // everything enqueued so far is complete: the bounds become exact
+  t->base_seq = t->seq;
+  t->base_count = c;
+  t->base_top = t->st_host->arena_top;
+  t->pend_keys = t->pend_units = 0;
   return PSKV_OK;
 }
 
@@ -192,66 +230,98 @@ int alloc_slots(uint64_t cap, Slot** out, hipStream_t stream) {
   return PSKV_OK;
 }
 
-// Makes room for `n` more keys (every key of a request may be new).
-int ensure_slots(pskv_table* t, uint64_t n) {
-  if (t->no_growth) return PSKV_OK;
-  const double limit = (double)t->max_load * (double)t->cap;
-  if ((double)(t->count_ub + n) <= limit) {
-    t->count_ub += n;
-    return PSKV_OK;
+// Moves the base of the bounds forward to the newest record the device has published.
+void adopt_snapshot(pskv_table* t) {
+  const Snapshot* sn = t->snap;
+  const uint64_t s1 = sn->seq_end;
+  std::atomic_thread_fence(std::memory_order_acquire);
+  const uint64_t c = sn->count, top = sn->arena_top;
+  std::atomic_thread_fence(std::memory_order_acquire);
+  const uint64_t s0 = sn->seq_begin;
+  if (s0 != s1 || s1 <= t->base_seq || s1 > t->seq) return;
+  for (uint64_t r = t->base_seq; r < s1; ++r) {
+    t->pend_keys -= t->log_keys[r % pskv_table::kLog];
+    t->pend_units -= t->log_units[r % pskv_table::kLog];
   }
-  int rc = read_state(t);
+  t->base_seq = s1;
+  t->base_count = c;
+  t->base_top = top;
+}
+
+int grow_slots(pskv_table* t, uint64_t keys_needed) {
+  uint64_t want = next_pow2((uint64_t)((double)keys_needed / t->max_load) + 1);
+  want = std::max(want, t->cap * 2);
+  Slot* fresh = nullptr;
+  int rc = alloc_slots(want, &fresh, t->stream);
   if (rc) return rc;
-  t->count_ub = t->count;
-  if (t->mode != PSKV_MODE_SCALAR) {
-    t->top_ub = t->st_host->arena_top;
-  }
-  if ((double)(t->count_ub + n) > limit) {
-    uint64_t want = next_pow2((uint64_t)((double)(t->count_ub + n) / t->max_load) + 1);
-    want = std::max(want, t->cap * 2);
-    Slot* fresh = nullptr;
-    rc = alloc_slots(want, &fresh, t->stream);
-    if (rc) return rc;
-    launch(t, PSKV_KERNEL_REHASH, k_rehash, dim3(grid_for(t->cap, kBlock, kMaxGrid)), dim3(kBlock),
-           t->slots, t->cap, fresh, want - 1, t->st);
-    PSKV_HIP(hipGetLastError());
-    PSKV_HIP(hipStreamSynchronize(t->stream));
-    PSKV_HIP(hipFree(t->slots));
-    t->slots = fresh;
-    t->cap = want;
-  }
-  t->count_ub += n;
+  launch(t, PSKV_KERNEL_REHASH, k_rehash, dim3(grid_for(t->cap, kBlock, kMaxGrid)), dim3(kBlock),
+         (const Slot*)t->slots, t->cap, fresh, want - 1, t->st);
+  PSKV_HIP(hipGetLastError());
+  PSKV_HIP(hipStreamSynchronize(t->stream));
+  PSKV_HIP(hipFree(t->slots));
+  t->slots = fresh;
+  t->cap = want;
   return PSKV_OK;
 }
 
-// Makes room in the arena. `units` is in the arena's allocation unit (rows for FIXED,
-// 16 bytes for VARLEN); `floats_per_unit` converts to floats.
-int ensure_arena(pskv_table* t, uint64_t units, uint64_t floats_per_unit) {
+int grow_arena(pskv_table* t, uint64_t floats_needed, uint64_t live_floats) {
+  uint64_t want = std::max(floats_needed, t->arena_cap + t->arena_cap / 2);
+  want = (want + 1023) & ~(uint64_t)1023;
+  float* fresh = nullptr;
+  PSKV_HIP(hipMalloc(reinterpret_cast<void**>(&fresh), want * sizeof(float)));
+  if (live_floats && t->arena) {
+    PSKV_HIP(hipMemcpyAsync(fresh, t->arena, live_floats * sizeof(float), hipMemcpyDeviceToDevice,
+                            t->stream));
+  }
+  PSKV_HIP(hipStreamSynchronize(t->stream));
+  if (t->arena) PSKV_HIP(hipFree(t->arena));
+  t->arena = fresh;
+  t->arena_cap = want;
+  return PSKV_OK;
+}
+
+// Begins a request that may create up to `n` keys and take up to `units` allocation units
+// of the arena (rows for FIXED, 16 bytes for VARLEN; `floats_per_unit` converts to floats).
+// Grows the slot array / the arena first if the bounds say they could overflow. The fast
+// path touches no device state; the next best reads the snapshot the device published;
+// only then does it wait for the stream and read the counters.
+int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit) {
   if (t->no_growth) return PSKV_OK;
-  if ((t->top_ub + units) * floats_per_unit <= t->arena_cap) {
-    t->top_ub += units;
-    return PSKV_OK;
-  }
-  int rc = read_state(t);
-  if (rc) return rc;
-  t->top_ub = t->st_host->arena_top;
-  const uint64_t need = (t->top_ub + units) * floats_per_unit;
-  if (need > t->arena_cap) {
-    uint64_t want = std::max(need, t->arena_cap + t->arena_cap / 2);
-    want = (want + 1023) & ~(uint64_t)1023;
-    float* fresh = nullptr;
-    PSKV_HIP(hipMalloc(reinterpret_cast<void**>(&fresh), want * sizeof(float)));
-    const uint64_t live = t->top_ub * floats_per_unit;
-    if (live && t->arena) {
-      PSKV_HIP(hipMemcpyAsync(fresh, t->arena, live * sizeof(float), hipMemcpyDeviceToDevice,
-                              t->stream));
+  const double limit = (double)t->max_load * (double)t->cap;
+  auto slots_short = [&]() { return (double)(t->base_count + t->pend_keys + n) > limit; };
+  auto arena_short = [&]() {
+    return units && (t->base_top + t->pend_units + units) * floats_per_unit > t->arena_cap;
+  };
+  if (slots_short() || arena_short() || t->seq - t->base_seq >= (uint64_t)pskv_table::kLog - 1) {
+    adopt_snapshot(t);
+    if (slots_short() || arena_short() || t->seq - t->base_seq >= (uint64_t)pskv_table::kLog - 1) {
+      int rc = read_state(t);  // exact counters, stream idle
+      if (rc) return rc;
+      if (slots_short()) {
+        rc = grow_slots(t, t->base_count + n);
+        if (rc) return rc;
+      }
+      if (arena_short()) {
+        rc = grow_arena(t, (t->base_top + units) * floats_per_unit, t->base_top * floats_per_unit);
+        if (rc) return rc;
+      }
     }
-    PSKV_HIP(hipStreamSynchronize(t->stream));
-    if (t->arena) PSKV_HIP(hipFree(t->arena));
-    t->arena = fresh;
-    t->arena_cap = want;
   }
-  t->top_ub += units;
+  const uint64_t q = t->seq++;
+  t->log_keys[q % pskv_table::kLog] = n;
+  t->log_units[q % pskv_table::kLog] = units;
+  t->pend_keys += n;
+  t->pend_units += units;
+  // Close to a limit: let the device publish its counters in front of this request, so that
+  // a later request can move the base forward without waiting for the stream.
+  const double limit_now = (double)t->max_load * (double)t->cap;
+  const bool tight_slots = (double)(t->base_count + t->pend_keys + 2 * n) > limit_now;
+  const bool tight_arena =
+      units && (t->base_top + t->pend_units + 2 * units) * floats_per_unit > t->arena_cap;
+  if (tight_slots || tight_arena || t->seq - t->base_seq >= (uint64_t)pskv_table::kLog / 2) {
+    k_publish<<<dim3(1), dim3(1), 0, t->stream>>>(t->st, t->snap, q);
+    PSKV_HIP(hipGetLastError());
+  }
   return PSKV_OK;
 }
 
@@ -273,7 +343,7 @@ struct Request {
 int run_scalar(pskv_table* t, Request& r) {
   r.out_nvals = r.pull ? r.n : 0;
   if (r.n == 0) return PSKV_OK;
-  int rc = ensure_slots(t, r.n);
+  int rc = reserve(t, r.n, 0, 0);
   if (rc) return rc;
   const dim3 grid(grid_for(r.n, kBlock, kMaxGrid)), block(kBlock);
   const uint64_t mask = t->cap - 1;
@@ -318,9 +388,7 @@ int run_fixed(pskv_table* t, Request& r) {
   const uint64_t k = t->row_len;
   r.out_nvals = r.pull ? r.n * k : 0;
   if (r.n == 0) return PSKV_OK;
-  int rc = ensure_slots(t, r.n);
-  if (rc) return rc;
-  rc = ensure_arena(t, r.n, k);
+  int rc = reserve(t, r.n, r.n, k);
   if (rc) return rc;
   rc = grow(t, &t->ws, Carver::need(r.n, sizeof(uint64_t)));
   if (rc) return rc;
@@ -390,9 +458,7 @@ int run_varlen(pskv_table* t, Request& r) {
   p.n = r.n;
 
   if (r.push) {
-    rc = ensure_slots(t, r.n);
-    if (rc) return rc;
-    rc = ensure_arena(t, r.nvals / 4 + r.n, 4);
+    rc = reserve(t, r.n, r.nvals / 4 + r.n, 4);
     if (rc) return rc;
     k_begin_request<<<dim3(1), dim3(1), 0, t->stream>>>(t->st);
     PSKV_HIP(launch_lens_scan(r.lens, r.n, off, part, t->st, PSKV_MAX_VARLEN_ROW, t->stream));
@@ -639,8 +705,11 @@ int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
   if (hipMalloc(reinterpret_cast<void**>(&t->st), sizeof(DevState)) != hipSuccess ||
       hipMemsetAsync(t->st, 0, sizeof(DevState), t->stream) != hipSuccess ||
       hipHostMalloc(reinterpret_cast<void**>(&t->st_host), sizeof(DevState), hipHostMallocDefault) !=
+          hipSuccess ||
+      hipHostMalloc(reinterpret_cast<void**>(&t->snap), sizeof(Snapshot), hipHostMallocDefault) !=
           hipSuccess)
     return fail(set_error(PSKV_ENOMEM, "cannot allocate table state"));
+  std::memset(t->snap, 0, sizeof(Snapshot));
   if (t->mode != PSKV_MODE_SCALAR && opts->arena_floats) {
     t->arena_cap = (opts->arena_floats + 1023) & ~(uint64_t)1023;
     if (hipMalloc(reinterpret_cast<void**>(&t->arena), t->arena_cap * sizeof(float)) != hipSuccess)
@@ -666,6 +735,7 @@ int pskv_table_destroy(pskv_table* t) {
   if (t->slots) (void)hipFree(t->slots);
   if (t->st) (void)hipFree(t->st);
   if (t->st_host) (void)hipHostFree(t->st_host);
+  if (t->snap) (void)hipHostFree(t->snap);
   if (t->arena) (void)hipFree(t->arena);
   if (t->ws.ptr) (void)hipFree(t->ws.ptr);
   if (t->stage.ptr) (void)hipFree(t->stage.ptr);
@@ -701,8 +771,6 @@ int pskv_sync(pskv_table* t) {
   DeviceGuard guard(t->device);
   int rc = read_state(t);
   if (rc) return rc;
-  t->count_ub = t->count;
-  if (t->mode != PSKV_MODE_SCALAR) t->top_ub = t->st_host->arena_top;
   return report_device_errors(t);
 }
 

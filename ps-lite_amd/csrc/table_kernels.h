@@ -277,6 +277,18 @@ __device__ __forceinline__ void rows_tile(const RowsParams& p, int32_t* s_off, u
       (uint32_t)((p.total - f0 < (uint64_t)TILE) ? (p.total - f0) : (uint64_t)TILE);
   const uint32_t nelem = tile_floats / VEC;
 
+  // The request-side loads depend on nothing but the tile index: issue them first so that
+  // they are in flight while the row references are fetched and searched.
+  V x[kIter];
+  if (OP == kOpAcc) {
+#pragma unroll
+    for (int i = 0; i < kIter; ++i) {
+      const uint32_t le = (uint32_t)i * kBlock + threadIdx.x;
+      x[i] = VecT<VEC>::zero();
+      if (le < nelem) x[i] = vload<STREAM>(reinterpret_cast<const V*>(p.req + f0 + le * VEC));
+    }
+  }
+
   // FIXED: row and offset of the tile's first float
   uint64_t j0 = 0, rem0 = 0;
   // VARLEN: keys that overlap the tile
@@ -301,7 +313,7 @@ __device__ __forceinline__ void rows_tile(const RowsParams& p, int32_t* s_off, u
 
 #pragma unroll
   for (int g = 0; g < kIter; g += kGroup) {
-    V x[kGroup], y[kGroup];
+    V y[kGroup];
     V* dst[kGroup];
     uint32_t lf[kGroup];
     bool live[kGroup], fresh[kGroup];
@@ -355,14 +367,11 @@ __device__ __forceinline__ void rows_tile(const RowsParams& p, int32_t* s_off, u
       }
       fresh[u] = (r & kRefNew) != 0 && !p.ignore_new;
     }
-    // all loads of the group first, so each lane has up to 2*kGroup requests in flight
+    // all stored-row loads of the group before the first add
 #pragma unroll
     for (int u = 0; u < kGroup; ++u) {
-      x[u] = VecT<VEC>::zero();
       y[u] = VecT<VEC>::zero();
-      if (!live[u]) continue;
-      if (OP == kOpAcc) x[u] = vload<STREAM>(reinterpret_cast<const V*>(p.req + f0 + lf[u]));
-      if (!fresh[u]) y[u] = vload<STREAM>(dst[u]);
+      if (live[u] && !fresh[u]) y[u] = vload<STREAM>(dst[u]);
     }
 #pragma unroll
     for (int u = 0; u < kGroup; ++u) {
@@ -373,7 +382,7 @@ __device__ __forceinline__ void rows_tile(const RowsParams& p, int32_t* s_off, u
           if (fresh[u]) vstore<STREAM>(VecT<VEC>::zero(), dst[u]);
         } else {
           // a created row is a zero row first (0.0f + v), kv_app.h:454
-          vstore<STREAM>(y[u] + x[u], dst[u]);
+          vstore<STREAM>(y[u] + x[g + u], dst[u]);
         }
       } else {
         vstore<STREAM>(y[u], reinterpret_cast<V*>(p.req + f0 + lf[u]));
