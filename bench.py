@@ -13,10 +13,12 @@ Workloads (BASELINE.json `configs`):
   varlen (configs[4]): 2,000,000 keys with lens in {8,16,32,64,128} over 16 ranges; a
       step is one push of all keys followed by a pull with lens. value = keys/s.
 
-Prints ONE JSON line. Inputs are resident in HBM before the clock starts. `roofline`
-is the dominant kernel of the workload timed with HIP events on the stream it runs
-on (inside the timed steps); `cpu_baseline` is the CPU oracle on the same inputs,
-one thread, on a bounded sample.
+Prints ONE JSON line. Inputs are resident in HBM before the clock starts. `value` comes
+from exactly K timed steps. `roofline` is the dominant kernel of the workload: after the
+timed steps the same steps run again with every launch of the store kernels carrying its
+own start/stop HIP events on the stream it runs on (per-launch events cost about 15 us of
+host time each, which is why they stay out of the timed region). `cpu_baseline` is the CPU
+oracle on the same inputs, one thread, on a bounded sample.
 """
 import argparse
 import json
@@ -32,6 +34,21 @@ import __graft_entry__ as graft  # noqa: E402
 
 KMAX = (1 << 64) - 1
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+# HBM bytes per launch (read + written) of the dominant kernels at the shapes below, from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this very script, scaled by what the same
+# counters read for the 1 GiB copy kernel (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0). They are
+# measured offline (a counter run cannot be nested in a timing run) and only reported when
+# the launch shape is the default one.
+TRAFFIC = {
+    ("push_scalar", 250000): 60.9e6, ("pull_scalar", 250000): 36.2e6,
+    ("rows_acc_fixed", 268435456): 3.0 * 2**30, ("rows_gather_fixed", 268435456): 2.0 * 2**30,
+    ("rows_acc_varlen", 6192336): 78.5e6, ("rows_gather_varlen", 6192336): 53.0e6,
+}
+
+
+def traffic(kind, units):
+    return TRAFFIC.get((kind, int(units)))
 
 
 def log(*a):
@@ -162,9 +179,11 @@ def run_sparse_lr(args, capi, dev):
                                "push then pull, store grows by 1M keys/step", "keys_per_step": n,
                    "ranges": S, "value_len": 1, "store_keys_after_timed_steps": held},
         # every pushed key is new: 8 key + 4 val in, 8 slot read, 8 key + 4 val written
-        "roofline": dict(roofline(32.0 * keys_per_launch, push_n, push_ms),
+        "roofline": dict(roofline(32.0 * keys_per_launch, push_n, push_ms,
+                                  traffic("push_scalar", keys_per_launch)),
                          kernel="k_scalar<push> (find-or-insert + add)", bytes_per_key=32),
-        "kernels": {"pull_scalar": dict(roofline(24.0 * keys_per_launch, pull_n, pull_ms),
+        "kernels": {"pull_scalar": dict(roofline(24.0 * keys_per_launch, pull_n, pull_ms,
+                                                 traffic("pull_scalar", keys_per_launch)),
                                         bytes_per_key=24)},
     }
     return res, batches[args.warmup:args.warmup + args.steps], (n, S)
@@ -205,13 +224,11 @@ def measure_dense(capi, dev, steps, warmup, nk=64, k=4194304):
     vals = torch.rand(nk * k, device=dev, generator=g) * 2 - 1
     out = torch.empty(nk * k, dtype=torch.float32, device=dev)
     t = capi.Table(capi.MODE_FIXED, initial_capacity=1024, row_len=k, arena_floats=nk * k)
-    t.prof_enable(True)
     t.push(keys, vals)  # first touch creates the rows
     for _ in range(warmup):
         t.push(keys, vals)
         t.pull(keys, out)
     t.sync()
-    t.prof_reset()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
@@ -220,12 +237,20 @@ def measure_dense(capi, dev, steps, warmup, nk=64, k=4194304):
     t.sync()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    # instrumented pass: the same steps again, every launch carrying its own HIP events
+    t.prof_enable(True)
+    t.prof_reset()
+    for _ in range(steps):
+        t.push(keys, vals)
+        t.pull(keys, out)
+    t.sync()
     acc = t.prof_read(capi.KERNEL_ROWS_ACC)
     gat = t.prof_read(capi.KERNEL_ROWS_GATHER)
-    # closed form: every float holds (1 + warmup + steps) * v, accumulated one add at a time
+    t.prof_enable(False)
+    # closed form: every float holds (1 + warmup + 2*steps) * v, accumulated one add at a time
     idx = torch.randint(0, nk * k, (4096,), device=dev)
     ref = torch.zeros(4096, device=dev)
-    for _ in range(1 + warmup + steps):
+    for _ in range(1 + warmup + 2 * steps):
         ref = ref + vals[idx]
     assert torch.equal(out[idx], ref), "dense sums differ from sequential float adds"
     # one plain copy of the same 1 GiB: the known-size launch that memory-traffic counters are
@@ -245,9 +270,11 @@ def run_dense(args, capi, dev):
         "config": {"workload": "dense: 64 keys x 4,194,304 f32 (1 GiB), push-accumulate then full pull",
                    "keys_per_step": nk, "value_len": k},
         # 4 B in + 4 B row read + 4 B row write per float
-        "roofline": dict(roofline(12.0 * floats, acc[0], acc[1]),
+        "roofline": dict(roofline(12.0 * floats, acc[0], acc[1], traffic("rows_acc_fixed", floats)),
                          kernel="k_rows<acc,fixed> (row += in)", bytes_per_float=12),
-        "kernels": {"rows_gather": dict(roofline(8.0 * floats, gat[0], gat[1]), bytes_per_float=8)},
+        "kernels": {"rows_gather": dict(roofline(8.0 * floats, gat[0], gat[1],
+                                                 traffic("rows_gather_fixed", floats)),
+                                        bytes_per_float=8)},
     }
     return res
 
@@ -292,43 +319,52 @@ def run_varlen(args, capi, dev):
     dv = torch.randn(nvals, device=dev, generator=g) * 0.1
     out = torch.empty(nvals, dtype=torch.float32, device=dev)
     out_lens = torch.empty(n, dtype=torch.int32, device=dev)
+    stream = torch.cuda.Stream()  # one stream for all ranges: kernels run one at a time
     tables = [capi.Table(capi.MODE_VARLEN, initial_capacity=int(n / S * 1.2) * 4,
-                         arena_floats=int(nvals / S * 1.2)) for _ in range(S)]
-    for t in tables:
-        t.prof_enable(True)
+                         arena_floats=int(nvals / S * 1.5) + 8 * n // S, stream=stream.cuda_stream)
+              for _ in range(S)]
+    kp, vp, lp, op, olp = dk.data_ptr(), dv.data_ptr(), dl.data_ptr(), out.data_ptr(), out_lens.data_ptr()
 
     def step():
         pos, vpos, used = capi.slice_keys(dk, rb, re, lens=dl, nvals=nvals)
-        pos, vpos = pos.astype(np.int64), vpos.astype(np.int64)
+        pos, vpos = [int(x) for x in pos], [int(x) for x in vpos]
         for s in range(S):
             if used[s]:
-                tables[s].push(dk[pos[s]:pos[s + 1]], dv[vpos[s]:vpos[s + 1]], dl[pos[s]:pos[s + 1]])
+                c, f = pos[s + 1] - pos[s], vpos[s + 1] - vpos[s]
+                tables[s].push_raw(kp + 8 * pos[s], c, vp + 4 * vpos[s], f, lp + 4 * pos[s], c)
         for s in range(S):
             if used[s]:
-                tables[s].pull(dk[pos[s]:pos[s + 1]], out[vpos[s]:vpos[s + 1]], out_lens[pos[s]:pos[s + 1]])
+                c, f = pos[s + 1] - pos[s], vpos[s + 1] - vpos[s]
+                tables[s].pull_raw(kp + 8 * pos[s], c, op + 4 * vpos[s], f, olp + 4 * pos[s])
+
+    def drain():
+        for t in tables:
+            t.sync()
+        torch.cuda.synchronize()
 
     step()  # creates the rows
     for _ in range(args.warmup):
         step()
-    for t in tables:
-        t.sync()
-        t.prof_reset()
-    torch.cuda.synchronize()
+    drain()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
-    for t in tables:
-        t.sync()
-    torch.cuda.synchronize()
+    drain()
     dt = time.perf_counter() - t0
+    for t in tables:
+        t.prof_enable(True)
+        t.prof_reset()
+    for _ in range(args.steps):
+        step()
+    drain()
+    acc = kernel_stats(tables, capi.KERNEL_ROWS_ACC)
+    gat = kernel_stats(tables, capi.KERNEL_ROWS_GATHER)
     assert torch.equal(out_lens, dl), "pulled lens differ"
     idx = torch.randint(0, nvals, (4096,), device=dev)
     ref = torch.zeros(4096, device=dev)
-    for _ in range(1 + args.warmup + args.steps):
+    for _ in range(1 + args.warmup + 2 * args.steps):
         ref = ref + dv[idx]
     assert torch.equal(out[idx], ref), "var-len sums differ from sequential float adds"
-    acc = kernel_stats(tables, capi.KERNEL_ROWS_ACC)
-    gat = kernel_stats(tables, capi.KERNEL_ROWS_GATHER)
     floats_per_launch = nvals / S
     res = {
         "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
@@ -337,12 +373,33 @@ def run_varlen(args, capi, dev):
                                "pull with lens", "keys_per_step": n, "floats_per_step": nvals,
                    "ranges": S},
         "gbps": (20.0 * nvals + 56.0 * n) * args.steps / dt / 1e9,
-        "roofline": dict(roofline(12.0 * floats_per_launch, acc[0], acc[1]),
+        "roofline": dict(roofline(12.0 * floats_per_launch, acc[0], acc[1],
+                                  traffic("rows_acc_varlen", floats_per_launch)),
                          kernel="k_rows<acc,varlen> (row += in)", bytes_per_float=12),
-        "kernels": {"rows_gather": dict(roofline(8.0 * floats_per_launch, gat[0], gat[1]),
+        "kernels": {"rows_gather": dict(roofline(8.0 * floats_per_launch, gat[0], gat[1],
+                                                 traffic("rows_gather_varlen", floats_per_launch)),
                                         bytes_per_float=8)},
     }
-    return res
+    return res, (keys, lens, nvals, n, S)
+
+
+def cpu_varlen(orc, keys, lens, nvals, n, S, budget_s=15.0):
+    rng = np.random.default_rng(0xE3D)
+    vals = rng.normal(0, 0.1, size=nvals).astype(np.float32)
+    rb, re = orc.server_ranges(S)
+    st = orc.Store(orc.MODE_VARLEN)  # the ranges are disjoint: one store serves all of them
+    pos, vpos, used = orc.slice_keys(keys, rb, re, lens, nvals)
+    st.push(keys, vals, lens)
+    done = 0
+    t0 = time.perf_counter()
+    while done < 2 or time.perf_counter() - t0 < budget_s:
+        orc.slice_keys(keys, rb, re, lens, nvals)
+        st.push(keys, vals, lens)
+        st.handle(False, True, keys, out_cap=nvals)
+        done += 1
+    dt = time.perf_counter() - t0
+    return {"value": 2.0 * n * done / dt, "unit": "keys/s", "cores": 1, "kind": "port",
+            "sample": "%d full steps (slice + push + pull of %d keys, %d floats), one thread" % (done, n, nvals)}
 
 
 def main():
@@ -371,7 +428,7 @@ def main():
     elif args.workload == "dense":
         res = run_dense(args, capi, dev)
     else:
-        res = run_varlen(args, capi, dev)
+        res, varlen_inputs = run_varlen(args, capi, dev)
 
     extra = {}
     if args.workload == "sparse_lr" and not args.no_extra:
@@ -379,8 +436,10 @@ def main():
         # beside the default workload (10 push+pull steps of 1 GiB, well under a second)
         dt, acc, gat, nk, k = measure_dense(capi, dev, 10, 2)
         extra["dense_chunk"] = {
-            "rows_acc": dict(roofline(12.0 * nk * k, acc[0], acc[1]), bytes_per_float=12),
-            "rows_gather": dict(roofline(8.0 * nk * k, gat[0], gat[1]), bytes_per_float=8),
+            "rows_acc": dict(roofline(12.0 * nk * k, acc[0], acc[1], traffic("rows_acc_fixed", nk * k)),
+                             bytes_per_float=12),
+            "rows_gather": dict(roofline(8.0 * nk * k, gat[0], gat[1],
+                                         traffic("rows_gather_fixed", nk * k)), bytes_per_float=8),
         }
 
     cpu = None
@@ -392,7 +451,7 @@ def main():
         elif args.workload == "dense":
             cpu = cpu_dense(orc)
         else:
-            cpu = None  # the sparse and dense legs bracket it; timed in tests only
+            cpu = cpu_varlen(orc, *varlen_inputs)
 
     line = {
         "metric": "push+pull keys/sec and achieved GB/s (% of HBM peak) on 1 MI355X",

@@ -361,9 +361,9 @@ int run_scalar(pskv_table* t, Request& r) {
   return PSKV_OK;
 }
 
-// Requests at least this large are streamed with non-temporal accesses: they cannot stay
-// in the 256 MB last-level cache between two requests anyway.
-constexpr uint64_t kStreamFloats = 16u << 20;
+// Requests at least this large (4 MiB) are streamed with non-temporal accesses: between two
+// requests of a busy server they do not survive in the caches anyway.
+constexpr uint64_t kStreamFloats = 1u << 20;
 
 template <bool VARLEN>
 int launch_rows(pskv_table* t, int op, const RowsParams& p) {
