@@ -94,8 +94,11 @@ int pskv_push(pskv_table* t, const uint64_t* keys, size_t n, const float* vals, 
  * answers an absent key with length 0 without inserting it. If the response
  * does not fit out_cap floats the status is PSKV_ESIZE_MISMATCH and *out_nvals
  * (a host pointer, may be NULL) holds the needed size; out/out_lens are then
- * unspecified. In PSKV_MODE_VARLEN the call waits for the device even with
- * PSKV_MEM_DEVICE buffers because the response size is data dependent. */
+ * unspecified. In PSKV_MODE_VARLEN the response size is data dependent: with a non-NULL
+ * out_nvals the call waits for the device even with PSKV_MEM_DEVICE buffers; with
+ * out_nvals == NULL it stays asynchronous, out must have room for the whole response,
+ * and a response that does not fit writes nothing and is reported by the next
+ * pskv_sync as PSKV_ESIZE_MISMATCH. */
 int pskv_pull(pskv_table* t, const uint64_t* keys, size_t n, float* out, size_t out_cap,
               int32_t* out_lens, size_t* out_nvals, int memkind);
 

@@ -29,6 +29,12 @@ constexpr unsigned kDevErrLenChanged = 1u;  // var-len push: stored length diffe
 constexpr unsigned kDevErrFull = 2u;        // probe sequence found no free slot (host sizing bug)
 constexpr unsigned kDevErrBadLen = 4u;      // negative or too long length
 constexpr unsigned kDevErrSizeMismatch = 8u;  // lens do not add up to the number of values
+constexpr unsigned kDevErrNoRoom = 16u;       // asynchronous var-len pull: response larger than the buffer
+constexpr unsigned kDevErrDuplicate = 32u;    // the same key twice in one request (row modes)
+
+// Payload of a slot that has been claimed but not filled in yet (slots start as all ones).
+// No valid payload has bit 63 set.
+constexpr uint64_t kPayloadUnset = ~0ull;
 
 constexpr int kBlock = 256;             // threads per workgroup of every kernel here (4 waves)
 constexpr unsigned kSpanMax = 1024;     // keys whose offsets a row-kernel workgroup stages in LDS
@@ -52,6 +58,10 @@ struct DevState {
   unsigned int error;                  // sticky error bits of finished requests
   unsigned int req_error;              // error bits of the request in flight
   unsigned int misaligned;             // OR of (len & 3) over the lens of the current request
+  unsigned int scan_bits;              // the same, while the lens scan is still collecting it
+  unsigned int scan_bad;               // a length out of range seen by the lens scan in flight
+  unsigned int scan_ticket;            // workgroups of the lens scan that have finished
+  unsigned int pad0;
   // keys held (slot array plus the side slot) = sum of the shards
   unsigned long long count_shard[kCountShards * kShardStride];
 };

@@ -55,10 +55,13 @@ struct Snapshot {
   volatile uint64_t seq_end;
 };
 
-// One thread, launched in front of a request's kernels when the table is close to a limit.
+// One wavefront, launched in front of a request's kernels when the table is close to a limit.
 __global__ void k_publish(const DevState* st, Snapshot* out, uint64_t seq) {
-  unsigned long long c = 0;
-  for (int i = 0; i < kCountShards; ++i) c += st->count_shard[i * kShardStride];
+  static_assert(kCountShards <= 64, "one lane per shard");
+  unsigned long long c = threadIdx.x < kCountShards ? st->count_shard[threadIdx.x * kShardStride] : 0ull;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
+  if (threadIdx.x != 0) return;
   out->seq_begin = seq;
   __threadfence_system();
   out->count = c;
@@ -220,6 +223,10 @@ int report_device_errors(pskv_table* t) {
     return set_error(PSKV_EINVAL, "a length is negative or above PSKV_MAX_VARLEN_ROW");
   if (bits & kDevErrSizeMismatch)
     return set_error(PSKV_ESIZE_MISMATCH, "lens do not add up to the number of values");
+  if (bits & kDevErrDuplicate)
+    return set_error(PSKV_EINVAL, "a request held the same key twice (keys must be unique)");
+  if (bits & kDevErrNoRoom)
+    return set_error(PSKV_ESIZE_MISMATCH, "a var-len pull response did not fit the caller's buffer");
   return set_error(PSKV_ELEN_CHANGED, "a pushed row length differs from the stored length");
 }
 
@@ -319,7 +326,7 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit)
   const bool tight_arena =
       units && (t->base_top + t->pend_units + 2 * units) * floats_per_unit > t->arena_cap;
   if (tight_slots || tight_arena || t->seq - t->base_seq >= (uint64_t)pskv_table::kLog / 2) {
-    k_publish<<<dim3(1), dim3(1), 0, t->stream>>>(t->st, t->snap, q);
+    k_publish<<<dim3(1), dim3(64), 0, t->stream>>>(t->st, t->snap, q);
     PSKV_HIP(hipGetLastError());
   }
   return PSKV_OK;
@@ -338,6 +345,7 @@ struct Request {
   int32_t* out_lens;     // device (VARLEN pull)
   uint64_t out_nvals;    // result
   bool lazy_out;         // VARLEN pull into host memory: `out` is allocated once the size is known
+  bool need_total;       // VARLEN pull: the caller wants the response size back (forces a wait)
 };
 
 int run_scalar(pskv_table* t, Request& r) {
@@ -394,8 +402,14 @@ int run_fixed(pskv_table* t, Request& r) {
   if (rc) return rc;
   Carver c(t->ws.ptr);
   uint64_t* ref = c.take<uint64_t>(r.n);
-  launch(t, PSKV_KERNEL_LOOKUP, k_lookup_fixed, dim3(grid_for(r.n, kBlock * kLookupItems, kMaxGrid)),
-         dim3(kBlock), t->slots, t->cap - 1, t->st, r.keys, r.n, ref);
+  if (r.n >= kLookupLargeKeys) {
+    launch(t, PSKV_KERNEL_LOOKUP, k_lookup_fixed<kLookupItemsLarge>,
+           dim3(grid_for(r.n, kBlock * kLookupItemsLarge, kMaxGrid)), dim3(kBlock), t->slots,
+           t->cap - 1, t->st, r.keys, r.n, ref);
+  } else {
+    launch(t, PSKV_KERNEL_LOOKUP, k_lookup_fixed<1>, dim3(grid_for(r.n, kBlock, kMaxGrid)),
+           dim3(kBlock), t->slots, t->cap - 1, t->st, r.keys, r.n, ref);
+  }
   PSKV_HIP(hipGetLastError());
   RowsParams p{};
   p.arena = t->arena;
@@ -460,15 +474,25 @@ int run_varlen(pskv_table* t, Request& r) {
   if (r.push) {
     rc = reserve(t, r.n, r.nvals / 4 + r.n, 4);
     if (rc) return rc;
-    k_begin_request<<<dim3(1), dim3(1), 0, t->stream>>>(t->st);
-    PSKV_HIP(launch_lens_scan(r.lens, r.n, off, part, t->st, PSKV_MAX_VARLEN_ROW, t->stream));
-    launch(t, PSKV_KERNEL_LOOKUP, k_lookup_var_push,
-           dim3(grid_for(r.n, kBlock * kLookupItems, kMaxGrid)), block, t->slots, t->cap - 1, t->st,
-           r.keys, r.lens, r.n, r.nvals, ref);
+    // the scan also fills the tile table of the request side (tile sizes are those of nvals;
+    // a request whose lens do not add up to nvals is refused by the lookup kernel)
+    const uint64_t push_tiles = (r.nvals + kTileVar - 1) / kTileVar;
+    rc = grow(t, &t->tiles, (push_tiles + 1) * sizeof(uint32_t));
+    if (rc) return rc;
+    uint32_t* push_tile_key = static_cast<uint32_t*>(t->tiles.ptr);
+    PSKV_HIP(launch_lens_scan(r.lens, r.n, off, part, &t->st->scan_ticket, t->st, PSKV_MAX_VARLEN_ROW,
+                              r.nvals ? push_tile_key : nullptr, push_tiles, kTileVar, t->stream));
+    if (r.n >= kLookupLargeKeys) {
+      launch(t, PSKV_KERNEL_LOOKUP, k_lookup_var_push<kLookupItemsLarge>,
+             dim3(grid_for(r.n, kBlock * kLookupItemsLarge, kMaxGrid)), block, t->slots, t->cap - 1,
+             t->st, r.keys, r.lens, r.n, r.nvals, ref);
+    } else {
+      launch(t, PSKV_KERNEL_LOOKUP, k_lookup_var_push<1>, kgrid, block, t->slots, t->cap - 1, t->st,
+             r.keys, r.lens, r.n, r.nvals, ref);
+    }
     PSKV_HIP(hipGetLastError());
     if (r.nvals) {
-      rc = make_tile_keys(t, off, r.n, r.nvals, &p.tile_key);
-      if (rc) return rc;
+      p.tile_key = push_tile_key;
       p.req = const_cast<float*>(r.vals);
       p.arena = t->arena;
       p.total = r.nvals;
@@ -490,8 +514,26 @@ int run_varlen(pskv_table* t, Request& r) {
     launch(t, PSKV_KERNEL_LOOKUP, k_lookup_var_pull, kgrid, block, (const Slot*)t->slots, t->cap - 1,
            (const DevState*)t->st, r.keys, r.n, ref, lens_out);
     PSKV_HIP(hipGetLastError());
-    k_begin_request<<<dim3(1), dim3(1), 0, t->stream>>>(t->st);
-    PSKV_HIP(launch_lens_scan(lens_out, r.n, off, part, t->st, PSKV_MAX_VARLEN_ROW, t->stream));
+    PSKV_HIP(launch_lens_scan(lens_out, r.n, off, part, &t->st->scan_ticket, t->st,
+                              PSKV_MAX_VARLEN_ROW, nullptr, 0, kTileVar, t->stream));
+    if (!r.need_total) {
+      // No host round trip: the grid covers the caller's buffer, the kernels take the real
+      // size from the scan, and a response that does not fit is reported by the next sync.
+      if (r.out_cap) {
+        if (!r.out) return set_error(PSKV_EINVAL, "null out");
+        rc = make_tile_keys(t, off, r.n, r.out_cap, &p.tile_key);
+        if (rc) return rc;
+        p.req = r.out;
+        p.arena = t->arena;
+        p.total = r.out_cap;
+        p.total_on_device = 1;
+        p.force_scalar = (reinterpret_cast<uintptr_t>(r.out) & 15) ? 1u : 0u;
+        p.ignore_new = 1;
+        rc = launch_rows<true>(t, kOpGather, p);
+        if (rc) return rc;
+      }
+      return PSKV_OK;
+    }
     rc = read_state(t);  // the response size is data dependent
     if (rc) return rc;
     const uint64_t total = t->st_host->scan_total;
@@ -604,6 +646,7 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
   r.n = n;
   r.nvals = push ? nvals : 0;
   r.out_cap = out_cap;
+  r.need_total = host || out_nvals != nullptr || push;
   if (!host) {
     r.keys = keys;
     r.vals = vals;
@@ -716,7 +759,10 @@ int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
       return fail(set_error(PSKV_ENOMEM, "cannot allocate %llu floats of row storage",
                             (unsigned long long)t->arena_cap));
   }
-  if (hipStreamSynchronize(t->stream) != hipSuccess)
+  const uint64_t unset = kPayloadUnset;
+  if (hipMemcpyAsync(&t->st->special_payload, &unset, sizeof(unset), hipMemcpyHostToDevice, t->stream) !=
+          hipSuccess ||
+      hipStreamSynchronize(t->stream) != hipSuccess)
     return fail(set_error(PSKV_EHIP, "table initialisation failed"));
   *out = t;
   return PSKV_OK;

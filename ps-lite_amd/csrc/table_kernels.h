@@ -49,14 +49,10 @@ __global__ __launch_bounds__(kBlock) void k_scalar(Slot* __restrict__ slots, uin
 // Row modes, step 1: key -> row reference.
 // ---------------------------------------------------------------------------------
 
-// Resets the per-request words; one thread, first launch of every row-mode request.
-__global__ void k_begin_request(DevState* st) {
-  st->error |= st->req_error;
-  st->req_error = 0;
-  st->misaligned = 0;
-}
-
-constexpr int kLookupItems = 4;  // keys per thread and round of the creating lookups
+// Keys per thread and round of the creating lookups: 4 for large requests (fewer atomic adds on
+// the arena counter), 1 for small ones (enough workgroups to fill the GPU).
+constexpr int kLookupItemsLarge = 4;
+constexpr uint64_t kLookupLargeKeys = 1u << 20;
 
 // FIXED: find or create the row of every key. Push and pull both create
 // (pull of an absent key inserts a zero value, kv_app.h:457).
@@ -64,6 +60,7 @@ constexpr int kLookupItems = 4;  // keys per thread and round of the creating lo
 // every thread claims slots for its keys, then the workgroup takes the rows of all
 // created keys from the arena with ONE atomic add and a workgroup-wide scan hands them
 // out in request order, so rows of neighbouring keys are neighbours in the arena.
+template <int kLookupItems>
 __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slots, uint64_t mask,
                                                         DevState* st,
                                                         const uint64_t* __restrict__ keys,
@@ -85,6 +82,11 @@ __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slot
       is_new[j] = false;
       seen[j] = 0;
       if (i < n) p[j] = find_or_insert(slots, mask, st, keys[i], is_new[j], seen[j]);
+      if (p[j] && !is_new[j] && seen[j] == kPayloadUnset) {
+        // another lane of this request is creating the very same key: keys must be unique
+        atomicOr(&st->error, kDevErrDuplicate);
+        p[j] = nullptr;
+      }
       mine += (p[j] && is_new[j]) ? 1u : 0u;
     }
     unsigned long long total;
@@ -115,6 +117,7 @@ __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slot
 
 // VARLEN push: find or create; a created row gets ceil(len/4) 16-byte units of the
 // arena, so every row starts 16-byte aligned. A present row must have the pushed length.
+template <int kLookupItems>
 __global__ __launch_bounds__(kBlock) void k_lookup_var_push(
     Slot* __restrict__ slots, uint64_t mask, DevState* st, const uint64_t* __restrict__ keys,
     const int32_t* __restrict__ lens, uint64_t n, uint64_t nvals, uint64_t* __restrict__ ref) {
@@ -146,6 +149,10 @@ __global__ __launch_bounds__(kBlock) void k_lookup_var_push(
       if (i < n) {
         len[j] = (uint64_t)(uint32_t)lens[i];
         p[j] = find_or_insert(slots, mask, st, keys[i], is_new[j], seen[j]);
+        if (p[j] && !is_new[j] && seen[j] == kPayloadUnset) {
+          atomicOr(&st->error, kDevErrDuplicate);  // the same key twice in this request
+          p[j] = nullptr;
+        }
       }
       if (p[j] && is_new[j]) {
         units += (len[j] + 3) >> 2;
@@ -199,9 +206,12 @@ __global__ __launch_bounds__(kBlock) void k_lookup_var_pull(const Slot* __restri
 // VARLEN: first key of every request-side tile. Key j owns floats [off[j], off[j+1]);
 // it writes its index for each tile whose first float it owns, so every tile gets
 // exactly one writer and no search is needed later. Entry `ntiles` closes the table.
+// `ntiles_cap` is the room in the table; the tiles in use follow from the scanned total off[n].
 __global__ __launch_bounds__(kBlock) void k_tile_keys(const uint64_t* __restrict__ off, uint64_t n,
                                                      uint32_t* __restrict__ tile_key,
-                                                     uint64_t ntiles, uint64_t tile) {
+                                                     uint64_t ntiles_cap, uint64_t tile) {
+  uint64_t ntiles = (off[n] + tile - 1) / tile;
+  if (ntiles > ntiles_cap) ntiles = ntiles_cap;
   const uint64_t stride = (uint64_t)gridDim.x * kBlock;
   for (uint64_t j = (uint64_t)blockIdx.x * kBlock + threadIdx.x; j < n; j += stride) {
     const uint64_t a = off[j], b = off[j + 1];
@@ -234,6 +244,8 @@ struct RowsParams {
   uint64_t k;             // FIXED: floats per row
   uint32_t force_scalar;  // request buffer or k not 16-byte friendly
   uint32_t ignore_new;    // pull half of a push+pull: rows created by the push half hold data
+  uint32_t total_on_device;  // VARLEN pull without a host round trip: the floats to move are
+                             // DevState::scan_total and `total` is the room in req
 };
 
 constexpr int kOpAcc = 0;
@@ -266,15 +278,14 @@ __device__ __forceinline__ void vstore(V v, V* p) {
 }
 
 template <int OP, int VEC, bool VARLEN, bool STREAM, unsigned TILE>
-__device__ __forceinline__ void rows_tile(const RowsParams& p, int32_t* s_off, uint64_t* s_ref,
-                                          bool rejected) {
+__device__ __forceinline__ void rows_tile(const RowsParams& p, uint64_t total, int32_t* s_off,
+                                          uint64_t* s_ref, bool rejected) {
   using V = typename VecT<VEC>::type;
   constexpr int kIter = TILE / (VEC * kBlock);      // elements per thread
   constexpr int kGroup = kIter < 4 ? kIter : 4;     // loads issued back to back
   static_assert(kIter >= 1 && kIter % kGroup == 0, "tile does not divide over the workgroup");
   const uint64_t f0 = (uint64_t)blockIdx.x * TILE;
-  const uint32_t tile_floats =
-      (uint32_t)((p.total - f0 < (uint64_t)TILE) ? (p.total - f0) : (uint64_t)TILE);
+  const uint32_t tile_floats = (uint32_t)((total - f0 < (uint64_t)TILE) ? (total - f0) : (uint64_t)TILE);
   const uint32_t nelem = tile_floats / VEC;
 
   // The request-side loads depend on nothing but the tile index: issue them first so that
@@ -406,16 +417,25 @@ __global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
   __shared__ uint64_t s_ref[VARLEN ? kSpanMax : 1];
   bool rejected = false;
   bool scalar = p.force_scalar != 0;
+  uint64_t total = p.total;
   if (VARLEN) {
     const unsigned err = p.st->req_error;
     if (err & (kDevErrBadLen | kDevErrSizeMismatch)) return;
     rejected = (err & kDevErrLenChanged) != 0;
     scalar = scalar || (p.st->misaligned != 0);
+    if (p.total_on_device) {
+      total = p.st->scan_total;
+      if (total > p.total) {  // the response does not fit the caller's buffer: write nothing
+        if (blockIdx.x == 0 && threadIdx.x == 0) atomicOr(&p.st->error, kDevErrNoRoom);
+        return;
+      }
+    }
   }
+  if ((uint64_t)blockIdx.x * TILE >= total) return;  // the grid was sized for the room, not the data
   if (scalar) {
-    rows_tile<OP, 1, VARLEN, STREAM, TILE>(p, s_off, s_ref, rejected);
+    rows_tile<OP, 1, VARLEN, STREAM, TILE>(p, total, s_off, s_ref, rejected);
   } else {
-    rows_tile<OP, 4, VARLEN, STREAM, TILE>(p, s_off, s_ref, rejected);
+    rows_tile<OP, 4, VARLEN, STREAM, TILE>(p, total, s_off, s_ref, rejected);
   }
 }
 

@@ -273,3 +273,70 @@ def test_varlen_errors(capi, orc, dev):
     with pytest.raises(capi.PskvError) as e:
         t.pull(keys, out, np.zeros(3, np.int32))
     assert e.value.code == capi.ESIZE_MISMATCH and t.last_out_nvals == 5
+
+
+def test_varlen_pull_without_host_round_trip(capi, orc, dev):
+    """out_nvals == NULL keeps a var-len pull asynchronous: the kernels take the response size from
+    the device-side scan. Too small a buffer writes nothing and is reported by the next sync."""
+    import torch
+    announce("varlen_async_pull")
+    rng = np.random.default_rng(44)
+    n = 30000
+    keys = unique_keys(rng, n)
+    lens = rng.choice(np.array([0, 8, 16, 24, 200], np.int32), size=n).astype(np.int32)
+    vals = rng.normal(0, 1, size=int(lens.sum())).astype(np.float32)
+    t = capi.Table(capi.MODE_VARLEN, initial_capacity=1024)
+    o = orc.Store(orc.MODE_VARLEN)
+    dk, dl = to_dev(keys, dev), to_dev(lens, dev)
+    for _ in range(2):
+        t.push(dk, to_dev(vals, dev), dl)
+        o.push(keys, vals, lens)
+    probe = np.sort(np.concatenate([keys[::2], unique_keys(rng, 500)]))
+    probe = np.unique(probe)
+    want, want_lens = o.pull(probe)
+    dp = to_dev(probe, dev)
+    out = torch.full((want.size + 4096,), 7.0, dtype=torch.float32, device=dev)  # more room than needed
+    out_lens = torch.full((probe.size,), -1, dtype=torch.int32, device=dev)
+    t.pull_raw(dp.data_ptr(), probe.size, out.data_ptr(), out.numel(), out_lens.data_ptr())
+    t.sync()
+    assert np.array_equal(from_dev(out_lens), want_lens)
+    assert_bits_equal(from_dev(out)[:want.size], want, "async pull")
+    assert np.all(from_dev(out)[want.size:] == 7.0)  # nothing written past the response
+    small = torch.full((want.size - 8,), 7.0, dtype=torch.float32, device=dev)
+    t.pull_raw(dp.data_ptr(), probe.size, small.data_ptr(), small.numel(), out_lens.data_ptr())
+    with pytest.raises(capi.PskvError) as e:
+        t.sync()
+    assert e.value.code == capi.ESIZE_MISMATCH
+    assert np.all(from_dev(small) == 7.0)
+    t.sync()
+    _check_dump(t, o, "after async pulls")
+
+
+@pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
+def test_duplicate_keys_do_no_harm(capi, dev, mode):
+    """Keys of a request must be unique (kv_app.h:17). A request that repeats a key is a caller error:
+    the row modes report it, and in no mode does it touch memory it should not."""
+    announce("duplicate_keys", mode)
+    keys = np.array([5, 9, 9, 9, 12, 12, 40], np.uint64)
+    m = {"scalar": capi.MODE_SCALAR, "fixed": capi.MODE_FIXED, "varlen": capi.MODE_VARLEN}[mode]
+    t = capi.Table(m, initial_capacity=16)
+    if mode == "scalar":
+        t.push(keys, np.ones(keys.size, np.float32))
+        out = np.zeros(keys.size, np.float32)
+        t.pull(keys, out)
+        assert t.size()[0] == 4  # which of the racing adds survives is unspecified
+        return
+    lens = np.full(keys.size, 8, np.int32)
+    try:
+        t.push(keys, np.ones(keys.size * 8, np.float32), lens if mode == "varlen" else None)
+        reported = False
+    except capi.PskvError as e:
+        reported = e.code == capi.EINVAL
+    assert reported
+    assert t.size()[0] == 4
+    # the table is still usable
+    uniq = np.unique(keys)
+    t.push(uniq, np.ones(uniq.size * 8, np.float32), np.full(uniq.size, 8, np.int32) if mode == "varlen" else None)
+    out = np.zeros(uniq.size * 8, np.float32)
+    t.pull(uniq, out, np.zeros(uniq.size, np.int32) if mode == "varlen" else None)
+    assert np.all(out >= 1.0)
