@@ -171,20 +171,27 @@ def run_sparse_lr(args, capi, dev):
     pull_n, pull_ms = kernel_stats(tables, capi.KERNEL_PULL_SCALAR)
     for t in tables:
         t.prof_enable(False)
+    # the slicer alone on an idle GPU: two small launches and one read-back of S+1 positions
+    t_s = time.perf_counter()
+    for _ in range(50):
+        capi.slice_keys(d_batches[0][0], rb, re, nvals=n)
+    slice_us = (time.perf_counter() - t_s) / 50 * 1e6
     keys_per_launch = n / S
     res = {
         "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
-        "dtype": "u64 keys, f32 values",
+        "dtype": "f32",
         "config": {"workload": "sparse_lr: 1M sorted unique uint64 keys/step over 4 key ranges, "
                                "push then pull, store grows by 1M keys/step", "keys_per_step": n,
-                   "ranges": S, "value_len": 1, "store_keys_after_timed_steps": held},
+                   "ranges": S, "value_len": 1, "key_dtype": "u64",
+                   "store_keys_after_timed_steps": held},
         # every pushed key is new: 8 key + 4 val in, 8 slot read, 8 key + 4 val written
         "roofline": dict(roofline(32.0 * keys_per_launch, push_n, push_ms,
                                   traffic("push_scalar", keys_per_launch)),
                          kernel="k_scalar<push> (find-or-insert + add)", bytes_per_key=32),
         "kernels": {"pull_scalar": dict(roofline(24.0 * keys_per_launch, pull_n, pull_ms,
                                                  traffic("pull_scalar", keys_per_launch)),
-                                        bytes_per_key=24)},
+                                        bytes_per_key=24),
+                    "slicer": {"wall_us_per_call": round(slice_us, 1), "keys": n, "ranges": S}},
     }
     return res, batches[args.warmup:args.warmup + args.steps], (n, S)
 
