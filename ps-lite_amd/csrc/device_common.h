@@ -62,9 +62,41 @@ struct DevState {
   unsigned int scan_bad;               // a length out of range seen by the lens scan in flight
   unsigned int scan_ticket;            // workgroups of the lens scan that have finished
   unsigned int pad0;
+  // "Same keys as the request that last filled the workspace" fast path of the row modes.
+  // Every row-mode request has a number (epoch). cache_epoch is the request whose keys, lens,
+  // row references, offsets and tile table the workspace and the key cache hold; bad_epoch ==
+  // cache_epoch marks them unusable. same_epoch == e is the verdict, reached once by the
+  // compare kernel before anything else of request e runs, that e may reuse them.
+  unsigned long long cache_epoch;
+  unsigned long long bad_epoch;
+  unsigned long long same_epoch;
+  unsigned int same_diff;    // a workgroup of the compare kernel found a difference
+  unsigned int same_ticket;  // workgroups of the compare kernel that have finished
   // keys held (slot array plus the side slot) = sum of the shards
   unsigned long long count_shard[kCountShards * kShardStride];
 };
+
+// What a row-mode kernel needs to know about the request it belongs to.
+struct ReqTag {
+  unsigned long long epoch;  // number of the request
+  unsigned int try_cache;    // the host found the key cache structurally usable for this request
+  unsigned int pad;
+};
+
+// True when request `tag` carries exactly the keys (and lens) of the cached request, so that
+// the row references, offsets and tile table still in the workspace are this request's too.
+// The verdict is written once, by the compare kernel that runs before the other kernels of
+// the request, so every workgroup of every later kernel sees the same answer.
+__device__ __forceinline__ bool cache_same(const DevState* st, const ReqTag& tag) {
+  return st->same_epoch == tag.epoch;
+}
+
+// Records an error of request `epoch`; whatever that request left in the workspace is not
+// to be reused.
+__device__ __forceinline__ void raise_error(DevState* st, unsigned bit, unsigned long long epoch) {
+  atomicOr(&st->req_error, bit);
+  st->bad_epoch = epoch;
+}
 
 // Adds the workgroup's total of `x` to one shard of the key counter. Every thread of
 // the workgroup must call it. `red` holds kBlock/64 words of LDS.

@@ -62,7 +62,8 @@ __global__ __launch_bounds__(kBlock) void k_scan_partials(const int32_t* __restr
                                                          uint64_t n,
                                                          unsigned long long* __restrict__ part,
                                                          unsigned int* ticket, DevState* st,
-                                                         unsigned max_len) {
+                                                         unsigned max_len, ReqTag tag) {
+  if (st && cache_same(st, tag)) return;  // offsets and flags of the cached request still hold
   __shared__ unsigned long long red[kBlock / 64];
   __shared__ unsigned long long carry_s;
   __shared__ unsigned s_ticket;
@@ -103,7 +104,9 @@ __global__ __launch_bounds__(kBlock) void k_scan_partials(const int32_t* __restr
     *ticket = 0;  // ready for the next scan on this stream
     if (st) {
       st->error |= st->req_error;
-      st->req_error = atomicExch(&st->scan_bad, 0u) ? kDevErrBadLen : 0u;
+      const bool bad_len = atomicExch(&st->scan_bad, 0u) != 0u;
+      st->req_error = bad_len ? kDevErrBadLen : 0u;
+      if (bad_len) st->bad_epoch = tag.epoch;
       st->misaligned = atomicExch(&st->scan_bits, 0u);
     }
   }
@@ -119,7 +122,8 @@ __global__ __launch_bounds__(kBlock) void k_scan_final(const int32_t* __restrict
                                                       const unsigned long long* __restrict__ part,
                                                       uint64_t* __restrict__ off, DevState* st,
                                                       uint32_t* __restrict__ tile_key,
-                                                      uint64_t ntiles, uint64_t tile) {
+                                                      uint64_t ntiles, uint64_t tile, ReqTag tag) {
+  if (st && cache_same(st, tag)) return;
   __shared__ unsigned long long wsum[kBlock / 64];
   constexpr int kScanChunk = kBlock * kScanItems;
   const uint64_t base = (uint64_t)blockIdx.x * kScanChunk + (uint64_t)threadIdx.x * kScanItems;
@@ -168,17 +172,17 @@ inline uint64_t scan_num_parts(uint64_t n) {
 inline hipError_t launch_lens_scan(const int32_t* lens, uint64_t n, uint64_t* off,
                                    unsigned long long* part, unsigned int* ticket, DevState* st,
                                    unsigned max_len, uint32_t* tile_key, uint64_t ntiles,
-                                   uint64_t tile, hipStream_t stream) {
+                                   uint64_t tile, ReqTag tag, hipStream_t stream) {
   if (n == 0) return hipMemsetAsync(off, 0, sizeof(uint64_t), stream);
   const uint64_t nparts = scan_num_parts(n);
   const dim3 grid((unsigned)nparts), block(kBlock);
   if (scan_items(n) == kScanItemsLarge) {
-    k_scan_partials<kScanItemsLarge><<<grid, block, 0, stream>>>(lens, n, part, ticket, st, max_len);
+    k_scan_partials<kScanItemsLarge><<<grid, block, 0, stream>>>(lens, n, part, ticket, st, max_len, tag);
     k_scan_final<kScanItemsLarge><<<grid, block, 0, stream>>>(lens, n, part, off, st, tile_key, ntiles,
-                                                               tile);
+                                                               tile, tag);
   } else {
-    k_scan_partials<1><<<grid, block, 0, stream>>>(lens, n, part, ticket, st, max_len);
-    k_scan_final<1><<<grid, block, 0, stream>>>(lens, n, part, off, st, tile_key, ntiles, tile);
+    k_scan_partials<1><<<grid, block, 0, stream>>>(lens, n, part, ticket, st, max_len, tag);
+    k_scan_final<1><<<grid, block, 0, stream>>>(lens, n, part, off, st, tile_key, ntiles, tile, tag);
   }
   return hipGetLastError();
 }

@@ -111,6 +111,16 @@ struct pskv_table {
   GrowBuf stage_out;  // device-side response of a host-resident or undersized pull
   bool no_growth = false;  // set while dumping: every key is known to be present
 
+  // Row modes: the workspace keeps the row references, offsets and tile table of the last
+  // request that computed them, and the key cache keeps that request's keys and lens, so a
+  // request with the same keys (the usual case for a parameter server) can skip the lens
+  // scan and every hash probe. The device decides whether the keys match; these fields only
+  // say whether the buffers still have the shape the cached request gave them.
+  GrowBuf cache_keys, cache_lens;
+  bool cache_valid = false;
+  uint64_t cache_n = 0, cache_nvals = 0;
+  uint64_t epoch = 0;  // number of the last row-mode request
+
   bool prof = false;
   std::vector<EventPair> pending[PSKV_KERNEL_COUNT];
   std::vector<EventPair> free_events;
@@ -172,6 +182,8 @@ int grow(pskv_table* t, GrowBuf* b, size_t bytes) {
   if (bytes <= b->bytes) return PSKV_OK;
   size_t want = std::max(bytes, b->bytes + b->bytes / 2);
   want = (want + 255) & ~(size_t)255;
+  if (b == &t->ws || b == &t->tiles || b == &t->cache_keys || b == &t->cache_lens)
+    t->cache_valid = false;  // the contents do not survive a reallocation
   if (b->ptr) {
     // earlier requests on the stream may still read the old buffer
     PSKV_HIP(hipStreamSynchronize(t->stream));
@@ -392,6 +404,22 @@ int launch_rows(pskv_table* t, int op, const RowsParams& p) {
   return PSKV_OK;
 }
 
+// Starts a row-mode request: numbers it and, when the key cache has the right shape, lets the
+// device compare the request with the cached one. Call after every buffer the cache lives in
+// has been grown for this request.
+int begin_row_request(pskv_table* t, const Request& r, bool with_lens, ReqTag* tag) {
+  tag->epoch = ++t->epoch;
+  tag->pad = 0;
+  tag->try_cache = (t->cache_valid && t->cache_n == r.n) ? 1u : 0u;
+  if (tag->try_cache) {
+    k_same_keys<<<dim3(grid_for(r.n, kBlock * 4, 4096)), dim3(kBlock), 0, t->stream>>>(
+        r.keys, with_lens ? r.lens : nullptr, static_cast<const uint64_t*>(t->cache_keys.ptr),
+        with_lens ? static_cast<const int32_t*>(t->cache_lens.ptr) : nullptr, r.n, t->st, *tag);
+    PSKV_HIP(hipGetLastError());
+  }
+  return PSKV_OK;
+}
+
 int run_fixed(pskv_table* t, Request& r) {
   const uint64_t k = t->row_len;
   r.out_nvals = r.pull ? r.n * k : 0;
@@ -400,17 +428,27 @@ int run_fixed(pskv_table* t, Request& r) {
   if (rc) return rc;
   rc = grow(t, &t->ws, Carver::need(r.n, sizeof(uint64_t)));
   if (rc) return rc;
+  rc = grow(t, &t->cache_keys, r.n * sizeof(uint64_t));
+  if (rc) return rc;
   Carver c(t->ws.ptr);
   uint64_t* ref = c.take<uint64_t>(r.n);
+  uint64_t* cache_keys = static_cast<uint64_t*>(t->cache_keys.ptr);
+  ReqTag tag;
+  rc = begin_row_request(t, r, false, &tag);
+  if (rc) return rc;
   if (r.n >= kLookupLargeKeys) {
     launch(t, PSKV_KERNEL_LOOKUP, k_lookup_fixed<kLookupItemsLarge>,
            dim3(grid_for(r.n, kBlock * kLookupItemsLarge, kMaxGrid)), dim3(kBlock), t->slots,
-           t->cap - 1, t->st, r.keys, r.n, ref);
+           t->cap - 1, t->st, r.keys, r.n, ref, cache_keys, tag);
   } else {
     launch(t, PSKV_KERNEL_LOOKUP, k_lookup_fixed<1>, dim3(grid_for(r.n, kBlock, kMaxGrid)),
-           dim3(kBlock), t->slots, t->cap - 1, t->st, r.keys, r.n, ref);
+           dim3(kBlock), t->slots, t->cap - 1, t->st, r.keys, r.n, ref, cache_keys, tag);
   }
   PSKV_HIP(hipGetLastError());
+  // push and pull both create absent keys, so either leaves references for all n keys behind
+  t->cache_valid = true;
+  t->cache_n = r.n;
+  t->cache_nvals = r.n * k;
   RowsParams p{};
   p.arena = t->arena;
   p.ref = ref;
@@ -418,6 +456,7 @@ int run_fixed(pskv_table* t, Request& r) {
   p.n = r.n;
   p.total = r.n * k;
   p.k = k;
+  p.tag = tag;
   if (r.push) {
     p.req = const_cast<float*>(r.vals);
     p.force_scalar = ((k & 3) || (reinterpret_cast<uintptr_t>(r.vals) & 15)) ? 1u : 0u;
@@ -437,13 +476,13 @@ int run_fixed(pskv_table* t, Request& r) {
 
 // Grows the tile table to `total` request-side floats and fills it.
 int make_tile_keys(pskv_table* t, const uint64_t* off, uint64_t n, uint64_t total,
-                   const uint32_t** tile_key) {
+                   const uint32_t** tile_key, const ReqTag& tag) {
   const uint64_t ntiles = (total + kTileVar - 1) / kTileVar;
   int rc = grow(t, &t->tiles, (ntiles + 1) * sizeof(uint32_t));
   if (rc) return rc;
   uint32_t* tk = static_cast<uint32_t*>(t->tiles.ptr);
-  k_tile_keys<<<dim3(grid_for(n, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(off, n, tk, ntiles,
-                                                                                  (uint64_t)kTileVar);
+  k_tile_keys<<<dim3(grid_for(n, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(
+      off, n, tk, ntiles, (uint64_t)kTileVar, (const DevState*)t->st, tag);
   PSKV_HIP(hipGetLastError());
   *tile_key = tk;
   return PSKV_OK;
@@ -456,13 +495,27 @@ int run_varlen(pskv_table* t, Request& r) {
   const uint64_t nparts = scan_num_parts(r.n);
   const size_t need = Carver::need(r.n, 8) + Carver::need(r.n + 1, 8) + Carver::need(nparts, 8) +
                       Carver::need(r.n, 4);
+  // Every buffer the key cache lives in is grown BEFORE the request is compared with the
+  // cached one: a reallocation loses the cached contents and must rule the fast path out.
   int rc = grow(t, &t->ws, need);
   if (rc) return rc;
+  rc = grow(t, &t->cache_keys, r.n * sizeof(uint64_t));
+  if (rc) return rc;
+  rc = grow(t, &t->cache_lens, r.n * sizeof(int32_t));
+  if (rc) return rc;
+  const bool async_pull = r.pull && !r.push && !r.need_total;
+  const uint64_t tiles_for = r.push ? r.nvals : (async_pull ? r.out_cap : 0);
+  const uint64_t tiles_cap = (tiles_for + kTileVar - 1) / kTileVar;
+  rc = grow(t, &t->tiles, (tiles_cap + 1) * sizeof(uint32_t));
+  if (rc) return rc;
+
   Carver c(t->ws.ptr);
   uint64_t* ref = c.take<uint64_t>(r.n);
   uint64_t* off = c.take<uint64_t>(r.n + 1);
   unsigned long long* part = c.take<unsigned long long>(nparts);
   int32_t* tmp_lens = c.take<int32_t>(r.n);
+  uint64_t* cache_keys = static_cast<uint64_t*>(t->cache_keys.ptr);
+  int32_t* cache_lens = static_cast<int32_t*>(t->cache_lens.ptr);
   const dim3 kgrid(grid_for(r.n, kBlock, kMaxGrid)), block(kBlock);
 
   RowsParams p{};
@@ -474,23 +527,27 @@ int run_varlen(pskv_table* t, Request& r) {
   if (r.push) {
     rc = reserve(t, r.n, r.nvals / 4 + r.n, 4);
     if (rc) return rc;
+    if (t->cache_nvals != r.nvals) t->cache_valid = false;  // same lens would mean the same total
+    ReqTag tag;
+    rc = begin_row_request(t, r, true, &tag);
+    if (rc) return rc;
     // the scan also fills the tile table of the request side (tile sizes are those of nvals;
     // a request whose lens do not add up to nvals is refused by the lookup kernel)
-    const uint64_t push_tiles = (r.nvals + kTileVar - 1) / kTileVar;
-    rc = grow(t, &t->tiles, (push_tiles + 1) * sizeof(uint32_t));
-    if (rc) return rc;
     uint32_t* push_tile_key = static_cast<uint32_t*>(t->tiles.ptr);
     PSKV_HIP(launch_lens_scan(r.lens, r.n, off, part, &t->st->scan_ticket, t->st, PSKV_MAX_VARLEN_ROW,
-                              r.nvals ? push_tile_key : nullptr, push_tiles, kTileVar, t->stream));
+                              r.nvals ? push_tile_key : nullptr, tiles_cap, kTileVar, tag, t->stream));
     if (r.n >= kLookupLargeKeys) {
       launch(t, PSKV_KERNEL_LOOKUP, k_lookup_var_push<kLookupItemsLarge>,
              dim3(grid_for(r.n, kBlock * kLookupItemsLarge, kMaxGrid)), block, t->slots, t->cap - 1,
-             t->st, r.keys, r.lens, r.n, r.nvals, ref);
+             t->st, r.keys, r.lens, r.n, r.nvals, ref, cache_keys, cache_lens, tag);
     } else {
       launch(t, PSKV_KERNEL_LOOKUP, k_lookup_var_push<1>, kgrid, block, t->slots, t->cap - 1, t->st,
-             r.keys, r.lens, r.n, r.nvals, ref);
+             r.keys, r.lens, r.n, r.nvals, ref, cache_keys, cache_lens, tag);
     }
     PSKV_HIP(hipGetLastError());
+    t->cache_valid = true;  // whichever way the device decided, the cache now is this request
+    t->cache_n = r.n;
+    t->cache_nvals = r.nvals;
     if (r.nvals) {
       p.tile_key = push_tile_key;
       p.req = const_cast<float*>(r.vals);
@@ -498,6 +555,7 @@ int run_varlen(pskv_table* t, Request& r) {
       p.total = r.nvals;
       p.force_scalar = (reinterpret_cast<uintptr_t>(r.vals) & 15) ? 1u : 0u;
       p.ignore_new = 0;
+      p.tag = tag;
       rc = launch_rows<true>(t, kOpAcc, p);
       if (rc) return rc;
     }
@@ -511,17 +569,24 @@ int run_varlen(pskv_table* t, Request& r) {
       rc = report_device_errors(t);
       if (rc) return rc;
     }
+    // A pull with the keys of the cached push finds every key present with the cached length
+    // and reuses its references; any other pull recomputes them and so ends the cache.
+    ReqTag tag;
+    rc = begin_row_request(t, r, false, &tag);
+    if (rc) return rc;
+    if (!tag.try_cache) t->cache_valid = false;
     launch(t, PSKV_KERNEL_LOOKUP, k_lookup_var_pull, kgrid, block, (const Slot*)t->slots, t->cap - 1,
-           (const DevState*)t->st, r.keys, r.n, ref, lens_out);
+           t->st, r.keys, r.n, ref, lens_out, (const int32_t*)cache_lens, tag);
     PSKV_HIP(hipGetLastError());
     PSKV_HIP(launch_lens_scan(lens_out, r.n, off, part, &t->st->scan_ticket, t->st,
-                              PSKV_MAX_VARLEN_ROW, nullptr, 0, kTileVar, t->stream));
-    if (!r.need_total) {
+                              PSKV_MAX_VARLEN_ROW, nullptr, 0, kTileVar, tag, t->stream));
+    p.tag = tag;
+    if (async_pull) {
       // No host round trip: the grid covers the caller's buffer, the kernels take the real
       // size from the scan, and a response that does not fit is reported by the next sync.
       if (r.out_cap) {
         if (!r.out) return set_error(PSKV_EINVAL, "null out");
-        rc = make_tile_keys(t, off, r.n, r.out_cap, &p.tile_key);
+        rc = make_tile_keys(t, off, r.n, r.out_cap, &p.tile_key, tag);
         if (rc) return rc;
         p.req = r.out;
         p.arena = t->arena;
@@ -536,6 +601,7 @@ int run_varlen(pskv_table* t, Request& r) {
     }
     rc = read_state(t);  // the response size is data dependent
     if (rc) return rc;
+    if (t->st_host->same_epoch != tag.epoch) t->cache_valid = false;  // the pull recomputed the workspace
     const uint64_t total = t->st_host->scan_total;
     r.out_nvals = total;
     if (total > r.out_cap)
@@ -548,7 +614,7 @@ int run_varlen(pskv_table* t, Request& r) {
         r.out = static_cast<float*>(t->stage_out.ptr);
       }
       if (!r.out) return set_error(PSKV_EINVAL, "null out");
-      rc = make_tile_keys(t, off, r.n, total, &p.tile_key);
+      rc = make_tile_keys(t, off, r.n, total, &p.tile_key, tag);
       if (rc) return rc;
       p.req = r.out;
       p.arena = t->arena;
@@ -687,7 +753,10 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
     default: rc = run_varlen(t, r); break;
   }
   if (out_nvals) *out_nvals = r.out_nvals;
-  if (rc) return rc;
+  if (rc) {
+    t->cache_valid = false;
+    return rc;
+  }
   if (too_small)
     return set_error(PSKV_ESIZE_MISMATCH, "response needs %llu floats, buffer holds %llu",
                      (unsigned long long)fixed_out, (unsigned long long)out_cap);
@@ -699,7 +768,9 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
       PSKV_HIP(hipMemcpyAsync(out_lens, r.out_lens, n * 4, hipMemcpyDeviceToHost, t->stream));
     rc = read_state(t);  // also waits for the copies above
     if (rc) return rc;
-    return report_device_errors(t);
+    rc = report_device_errors(t);
+    if (rc) t->cache_valid = false;
+    return rc;
   }
   return PSKV_OK;
 }
@@ -786,6 +857,8 @@ int pskv_table_destroy(pskv_table* t) {
   if (t->ws.ptr) (void)hipFree(t->ws.ptr);
   if (t->stage.ptr) (void)hipFree(t->stage.ptr);
   if (t->tiles.ptr) (void)hipFree(t->tiles.ptr);
+  if (t->cache_keys.ptr) (void)hipFree(t->cache_keys.ptr);
+  if (t->cache_lens.ptr) (void)hipFree(t->cache_lens.ptr);
   if (t->stage_out.ptr) (void)hipFree(t->stage_out.ptr);
   if (t->own_stream && t->stream) (void)hipStreamDestroy(t->stream);
   delete t;

@@ -49,6 +49,42 @@ __global__ __launch_bounds__(kBlock) void k_scalar(Slot* __restrict__ slots, uin
 // Row modes, step 1: key -> row reference.
 // ---------------------------------------------------------------------------------
 
+// Compares a request with the cached one (keys, and lens when given) and reaches the verdict
+// for the whole request: the workgroup that finishes last (ticket counter) sees whether any
+// workgroup found a difference and whether the cache is usable at all, and writes same_epoch.
+// If the verdict is "different", the request is going to refill the cache, so it becomes the
+// cached request right here. Epochs start at 1.
+__global__ __launch_bounds__(kBlock) void k_same_keys(const uint64_t* __restrict__ keys,
+                                                     const int32_t* __restrict__ lens,
+                                                     const uint64_t* __restrict__ cache_keys,
+                                                     const int32_t* __restrict__ cache_lens,
+                                                     uint64_t n, DevState* st, ReqTag tag) {
+  __shared__ unsigned s_ticket;
+  bool differ = false;
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+    differ |= keys[i] != cache_keys[i];
+    if (lens) differ |= lens[i] != cache_lens[i];
+  }
+  const int any = __syncthreads_or(differ ? 1 : 0);
+  if (threadIdx.x == 0) {
+    if (any) atomicOr(&st->same_diff, 1u);
+    __threadfence();
+    s_ticket = atomicAdd(&st->same_ticket, 1u);
+  }
+  __syncthreads();
+  if (s_ticket != gridDim.x - 1 || threadIdx.x != 0) return;
+  __threadfence();
+  st->same_ticket = 0;
+  const bool different = atomicExch(&st->same_diff, 0u) != 0u;
+  const bool usable = st->cache_epoch != 0ull && st->bad_epoch != st->cache_epoch;
+  if (!different && usable) {
+    st->same_epoch = tag.epoch;
+  } else {
+    st->cache_epoch = tag.epoch;
+  }
+}
+
 // Keys per thread and round of the creating lookups: 4 for large requests (fewer atomic adds on
 // the arena counter), 1 for small ones (enough workgroups to fill the GPU).
 constexpr int kLookupItemsLarge = 4;
@@ -64,7 +100,11 @@ template <int kLookupItems>
 __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slots, uint64_t mask,
                                                         DevState* st,
                                                         const uint64_t* __restrict__ keys,
-                                                        uint64_t n, uint64_t* __restrict__ ref) {
+                                                        uint64_t n, uint64_t* __restrict__ ref,
+                                                        uint64_t* __restrict__ cache_keys,
+                                                        ReqTag tag) {
+  if (cache_same(st, tag)) return;  // the references of the cached request are this request's
+  if (blockIdx.x == 0 && threadIdx.x == 0) st->cache_epoch = cache_keys ? tag.epoch : 0ull;
   __shared__ unsigned long long red[kBlock / 64];
   __shared__ unsigned cred[kBlock / 64];
   __shared__ unsigned long long s_first;
@@ -81,10 +121,15 @@ __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slot
       p[j] = nullptr;
       is_new[j] = false;
       seen[j] = 0;
-      if (i < n) p[j] = find_or_insert(slots, mask, st, keys[i], is_new[j], seen[j]);
+      if (i < n) {
+        const uint64_t key = keys[i];
+        if (cache_keys) cache_keys[i] = key;
+        p[j] = find_or_insert(slots, mask, st, key, is_new[j], seen[j]);
+      }
       if (p[j] && !is_new[j] && seen[j] == kPayloadUnset) {
         // another lane of this request is creating the very same key: keys must be unique
         atomicOr(&st->error, kDevErrDuplicate);
+        st->bad_epoch = tag.epoch;
         p[j] = nullptr;
       }
       mine += (p[j] && is_new[j]) ? 1u : 0u;
@@ -120,11 +165,14 @@ __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slot
 template <int kLookupItems>
 __global__ __launch_bounds__(kBlock) void k_lookup_var_push(
     Slot* __restrict__ slots, uint64_t mask, DevState* st, const uint64_t* __restrict__ keys,
-    const int32_t* __restrict__ lens, uint64_t n, uint64_t nvals, uint64_t* __restrict__ ref) {
+    const int32_t* __restrict__ lens, uint64_t n, uint64_t nvals, uint64_t* __restrict__ ref,
+    uint64_t* __restrict__ cache_keys, int32_t* __restrict__ cache_lens, ReqTag tag) {
+  if (cache_same(st, tag)) return;  // the references of the cached request are this request's
+  if (blockIdx.x == 0 && threadIdx.x == 0) st->cache_epoch = cache_keys ? tag.epoch : 0ull;
   // the request is refused as a whole when its lens are invalid or do not add up to vals.size()
   if (st->req_error & (kDevErrBadLen | kDevErrSizeMismatch)) return;
   if (st->scan_total != nvals) {
-    if (blockIdx.x == 0 && threadIdx.x == 0) atomicOr(&st->req_error, kDevErrSizeMismatch);
+    if (blockIdx.x == 0 && threadIdx.x == 0) raise_error(st, kDevErrSizeMismatch, tag.epoch);
     return;
   }
   __shared__ unsigned long long red[kBlock / 64];
@@ -147,10 +195,16 @@ __global__ __launch_bounds__(kBlock) void k_lookup_var_push(
       seen[j] = 0;
       len[j] = 0;
       if (i < n) {
+        const uint64_t key = keys[i];
         len[j] = (uint64_t)(uint32_t)lens[i];
-        p[j] = find_or_insert(slots, mask, st, keys[i], is_new[j], seen[j]);
+        if (cache_keys) {
+          cache_keys[i] = key;
+          cache_lens[i] = (int32_t)len[j];
+        }
+        p[j] = find_or_insert(slots, mask, st, key, is_new[j], seen[j]);
         if (p[j] && !is_new[j] && seen[j] == kPayloadUnset) {
           atomicOr(&st->error, kDevErrDuplicate);  // the same key twice in this request
+          st->bad_epoch = tag.epoch;
           p[j] = nullptr;
         }
       }
@@ -178,7 +232,7 @@ __global__ __launch_bounds__(kBlock) void k_lookup_var_push(
         at += (len[j] + 3) >> 2;
         *p[j] = payload;
       } else if ((payload & kLenMask) != len[j]) {
-        atomicOr(&st->req_error, kDevErrLenChanged);
+        raise_error(st, kDevErrLenChanged, tag.epoch);
       }
       ref[i] = payload | (is_new[j] ? kRefNew : 0ull);
     }
@@ -189,12 +243,23 @@ __global__ __launch_bounds__(kBlock) void k_lookup_var_push(
 }
 
 // VARLEN pull: an absent key answers length 0 and is not created.
+// With the keys of the cached push the answer is known without a single probe: every key is
+// present with the cached length.
 __global__ __launch_bounds__(kBlock) void k_lookup_var_pull(const Slot* __restrict__ slots,
-                                                           uint64_t mask, const DevState* st,
+                                                           uint64_t mask, DevState* st,
                                                            const uint64_t* __restrict__ keys,
                                                            uint64_t n, uint64_t* __restrict__ ref,
-                                                           int32_t* __restrict__ out_lens) {
+                                                           int32_t* __restrict__ out_lens,
+                                                           const int32_t* __restrict__ cache_lens,
+                                                           ReqTag tag) {
   const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  if (cache_same(st, tag)) {
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride)
+      out_lens[i] = cache_lens[i];
+    return;
+  }
+  // this pull rewrites the references and offsets in the workspace: the cached push is gone
+  if (blockIdx.x == 0 && threadIdx.x == 0) st->bad_epoch = st->cache_epoch;
   for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
     uint64_t payload;
     const bool hit = find_only(slots, mask, st, keys[i], payload);
@@ -209,7 +274,9 @@ __global__ __launch_bounds__(kBlock) void k_lookup_var_pull(const Slot* __restri
 // `ntiles_cap` is the room in the table; the tiles in use follow from the scanned total off[n].
 __global__ __launch_bounds__(kBlock) void k_tile_keys(const uint64_t* __restrict__ off, uint64_t n,
                                                      uint32_t* __restrict__ tile_key,
-                                                     uint64_t ntiles_cap, uint64_t tile) {
+                                                     uint64_t ntiles_cap, uint64_t tile,
+                                                     const DevState* st, ReqTag tag) {
+  if (cache_same(st, tag)) return;  // the tile table of the cached request is this request's
   uint64_t ntiles = (off[n] + tile - 1) / tile;
   if (ntiles > ntiles_cap) ntiles = ntiles_cap;
   const uint64_t stride = (uint64_t)gridDim.x * kBlock;
@@ -246,6 +313,7 @@ struct RowsParams {
   uint32_t ignore_new;    // pull half of a push+pull: rows created by the push half hold data
   uint32_t total_on_device;  // VARLEN pull without a host round trip: the floats to move are
                              // DevState::scan_total and `total` is the room in req
+  ReqTag tag;
 };
 
 constexpr int kOpAcc = 0;
@@ -418,8 +486,11 @@ __global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
   bool rejected = false;
   bool scalar = p.force_scalar != 0;
   uint64_t total = p.total;
+  // a request served from the cached references creates nothing and cannot have been refused
+  const bool same = cache_same(p.st, p.tag);
+  if (same) p.ignore_new = 1;
   if (VARLEN) {
-    const unsigned err = p.st->req_error;
+    const unsigned err = same ? 0u : p.st->req_error;
     if (err & (kDevErrBadLen | kDevErrSizeMismatch)) return;
     rejected = (err & kDevErrLenChanged) != 0;
     scalar = scalar || (p.st->misaligned != 0);

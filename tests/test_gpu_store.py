@@ -340,3 +340,122 @@ def test_duplicate_keys_do_no_harm(capi, dev, mode):
     out = np.zeros(uniq.size * 8, np.float32)
     t.pull(uniq, out, np.zeros(uniq.size, np.int32) if mode == "varlen" else None)
     assert np.all(out >= 1.0)
+
+
+@pytest.mark.parametrize("mode", ["fixed", "varlen"])
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_repeated_and_alternating_key_sets(capi, orc, dev, mode, seed):
+    """Requests that repeat the previous request's keys take a path that skips the hash probes; requests
+    that do not must never see what that path left behind. Random sequences over a few key sets that
+    are equal, differ in one key, differ in one length or differ in size, through every entry point
+    and both memory kinds, checked against the oracle after every pull."""
+    import torch
+    announce("repeated_key_sets", mode, seed)
+    rng = np.random.default_rng(1000 + seed)
+    n = int(rng.integers(300, 3000))
+    k = 8
+    base = unique_keys(rng, n + 50)
+    sets = {}
+    sets["A"] = base[:n].copy()
+    b = base[:n].copy()
+    b[int(rng.integers(0, n))] = base[n + 1]  # one key differs
+    sets["B"] = np.sort(b)
+    sets["C"] = base[10:n + 10].copy()        # same size, shifted
+    sets["D"] = base[: n // 2].copy()         # a different size
+    lens_of = {int(key): int(l) for key, l in zip(base.tolist(), rng.choice([0, 4, 8, 12, 40], size=base.size))}
+    m = capi.MODE_FIXED if mode == "fixed" else capi.MODE_VARLEN
+    t = capi.Table(m, initial_capacity=64, row_len=k)  # small: the slot array grows during the sequence
+    o = orc.Store(orc.MODE_FIXED if mode == "fixed" else orc.MODE_VARLEN, k)
+
+    def lens_for(keys):
+        return np.array([lens_of[int(x)] for x in keys.tolist()], np.int32) if mode == "varlen" else None
+
+    names = ["A", "A", "A", "B", "C", "D", "A"]
+    for step in range(40):
+        name = names[int(rng.integers(0, len(names)))]
+        keys = sets[name]
+        lens = lens_for(keys)
+        nvals = int(lens.sum()) if mode == "varlen" else keys.size * k
+        op = ["push", "push", "pull", "pull_async", "pushpull"][int(rng.integers(0, 5))]
+        on_dev = bool(rng.integers(0, 2))
+        vals = rng.integers(-8, 8, size=nvals).astype(np.float32)
+        kk = to_dev(keys, dev) if on_dev else keys
+        vv = to_dev(vals, dev) if on_dev else vals
+        ll = None if lens is None else (to_dev(lens, dev) if on_dev else lens)
+        what = "step %d %s %s %s" % (step, op, name, "dev" if on_dev else "host")
+        if op == "push":
+            t.push(kk, vv, ll)
+            o.push(keys, vals, lens)
+        elif op == "pushpull":
+            want, want_lens = o.pushpull(keys, vals, lens)
+            if on_dev:
+                out = torch.full((nvals,), 7.0, dtype=torch.float32, device=dev)
+                out_lens = torch.full((keys.size,), -1, dtype=torch.int32, device=dev)
+                t.pushpull(kk, vv, out, ll, out_lens if mode == "varlen" else None)
+                t.sync()
+                got, got_lens = from_dev(out), from_dev(out_lens)
+            else:
+                got = np.full(nvals, 7.0, np.float32)
+                got_lens = np.full(keys.size, -1, np.int32)
+                t.pushpull(keys, vals, got, lens, got_lens if mode == "varlen" else None)
+            assert_bits_equal(got, want, what)
+            if mode == "varlen":
+                assert np.array_equal(got_lens, want_lens), what
+        else:
+            want, want_lens = o.pull(keys)
+            if op == "pull_async":
+                dk = to_dev(keys, dev)
+                out = torch.full((want.size + 64,), 7.0, dtype=torch.float32, device=dev)
+                out_lens = torch.full((keys.size,), -1, dtype=torch.int32, device=dev)
+                t.pull_raw(dk.data_ptr(), keys.size, out.data_ptr(), out.numel(),
+                           out_lens.data_ptr() if mode == "varlen" else None)
+                t.sync()
+                got, got_lens = from_dev(out)[:want.size], from_dev(out_lens)
+            elif on_dev:
+                out = torch.full((want.size,), 7.0, dtype=torch.float32, device=dev)
+                out_lens = torch.full((keys.size,), -1, dtype=torch.int32, device=dev)
+                assert t.pull(kk, out, out_lens if mode == "varlen" else None) == want.size
+                t.sync()
+                got, got_lens = from_dev(out), from_dev(out_lens)
+            else:
+                got = np.full(want.size, 7.0, np.float32)
+                got_lens = np.full(keys.size, -1, np.int32)
+                assert t.pull(keys, got, got_lens if mode == "varlen" else None) == want.size
+            assert_bits_equal(got, want, what)
+            if mode == "varlen":
+                assert np.array_equal(got_lens, want_lens), what
+    t.sync()
+    _check_dump(t, o, "after the sequence")
+
+
+def test_refused_push_does_not_poison_repeats(capi, orc, dev):
+    """A var-len push refused for a changed length must not leave anything behind that a repeat of the
+    same keys could pick up."""
+    announce("refused_push_then_repeat")
+    rng = np.random.default_rng(9)
+    keys = unique_keys(rng, 500)
+    lens = rng.choice(np.array([4, 8, 16], np.int32), size=500).astype(np.int32)
+    bad = lens.copy()
+    bad[123] += 4
+    t = capi.Table(capi.MODE_VARLEN, initial_capacity=64)
+    o = orc.Store(orc.MODE_VARLEN)
+    dk, dl, dbad = to_dev(keys, dev), to_dev(lens, dev), to_dev(bad, dev)
+    for which in ("good", "good", "bad", "bad", "good", "good"):
+        l, dlx = (lens, dl) if which == "good" else (bad, dbad)
+        vals = rng.integers(-4, 4, size=int(l.sum())).astype(np.float32)
+        t.push(dk, to_dev(vals, dev), dlx)
+        rc = o.handle(True, False, keys, vals, l)[0]
+        if which == "bad":
+            assert rc == orc.ELEN_CHANGED
+            with pytest.raises(capi.PskvError) as e:
+                t.sync()
+            assert e.value.code == capi.ELEN_CHANGED
+        else:
+            assert rc == 0
+            t.sync()
+        out = np.zeros(int(lens.sum()), np.float32)
+        out_lens = np.zeros(500, np.int32)
+        t.pull(keys, out, out_lens)
+        want, want_lens = o.pull(keys)
+        assert np.array_equal(out_lens, want_lens)
+        assert_bits_equal(out, want, "after a %s push" % which)
