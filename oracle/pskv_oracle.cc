@@ -202,7 +202,7 @@ static int handle_varlen(pskv_oracle_store* s, bool push, bool pull, const uint6
     }
     if (total != nvals) return PSKV_ORACLE_ESIZE_MISMATCH;
     // A row never changes its length. Absent keys are created (as zero rows)
-    // before the verdict, present rows are only touched when every length matches.
+    // before the decision, present rows are only touched when every length matches.
     bool changed = false;
     for (size_t i = 0; i < n; ++i) {
       auto it = s->rows.find(keys[i]);

@@ -65,7 +65,7 @@ struct DevState {
   // "Same keys as the request that last filled the workspace" fast path of the row modes.
   // Every row-mode request has a number (epoch). cache_epoch is the request whose keys, lens,
   // row references, offsets and tile table the workspace and the key cache hold; bad_epoch ==
-  // cache_epoch marks them unusable. same_epoch == e is the verdict, reached once by the
+  // cache_epoch marks them unusable. same_epoch == e is the decision, reached once by the
   // compare kernel before anything else of request e runs, that e may reuse them.
   unsigned long long cache_epoch;
   unsigned long long bad_epoch;
@@ -85,7 +85,7 @@ struct ReqTag {
 
 // True when request `tag` carries exactly the keys (and lens) of the cached request, so that
 // the row references, offsets and tile table still in the workspace are this request's too.
-// The verdict is written once, by the compare kernel that runs before the other kernels of
+// The decision is written once, by the compare kernel that runs before the other kernels of
 // the request, so every workgroup of every later kernel sees the same answer.
 __device__ __forceinline__ bool cache_same(const DevState* st, const ReqTag& tag) {
   return st->same_epoch == tag.epoch;

@@ -49,10 +49,10 @@ __global__ __launch_bounds__(kBlock) void k_scalar(Slot* __restrict__ slots, uin
 // Row modes, step 1: key -> row reference.
 // ---------------------------------------------------------------------------------
 
-// Compares a request with the cached one (keys, and lens when given) and reaches the verdict
+// Compares a request with the cached one (keys, and lens when given) and reaches the decision
 // for the whole request: the workgroup that finishes last (ticket counter) sees whether any
 // workgroup found a difference and whether the cache is usable at all, and writes same_epoch.
-// If the verdict is "different", the request is going to refill the cache, so it becomes the
+// If the decision is "different", the request is going to refill the cache, so it becomes the
 // cached request right here. Epochs start at 1.
 __global__ __launch_bounds__(kBlock) void k_same_keys(const uint64_t* __restrict__ keys,
                                                      const int32_t* __restrict__ lens,

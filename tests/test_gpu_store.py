@@ -459,3 +459,24 @@ def test_refused_push_does_not_poison_repeats(capi, orc, dev):
         want, want_lens = o.pull(keys)
         assert np.array_equal(out_lens, want_lens)
         assert_bits_equal(out, want, "after a %s push" % which)
+
+
+def test_scalar_long_probe_chains(capi, orc, dev):
+    """A nearly full slot array (fill 0.9) makes colliding keys walk long probe sequences; results and
+    the stored key set stay exact, and growth still happens before the array is full."""
+    announce("scalar_long_probes")
+    rng = np.random.default_rng(31)
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=900, max_load=0.9)
+    o = orc.Store(orc.MODE_SCALAR)
+    universe = unique_keys(rng, 20000)
+    for rep in range(30):
+        keys = np.sort(rng.choice(universe, size=int(rng.integers(1, 900)), replace=False))
+        vals = rng.integers(-100, 100, size=keys.size).astype(np.float32)
+        t.push(to_dev(keys, dev), to_dev(vals, dev))
+        o.push(keys, vals)
+        if rep % 5 == 4:
+            probe = np.sort(rng.choice(universe, size=700, replace=False))
+            got = np.zeros(700, np.float32)
+            t.pull(probe, got)
+            assert_bits_equal(got, o.pull(probe)[0], "rep %d" % rep)
+    _check_dump(t, o, "long probes")
