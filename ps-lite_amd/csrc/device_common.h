@@ -5,7 +5,7 @@
 #include <stdint.h>
 
 #ifndef PSKV_TILE_VAR
-#define PSKV_TILE_VAR 2048
+#define PSKV_TILE_VAR 256
 #endif
 
 namespace pskv {
@@ -24,6 +24,14 @@ constexpr uint64_t kRefAbsent = ~0ull;
 constexpr int kLenBits = 28;
 constexpr uint64_t kLenMask = (1ull << kLenBits) - 1;
 
+// Per-tile shortcut of the var-len row kernel. When the rows that overlap a request-side tile
+// lie in the arena back to back, in request order and without padding, the whole tile maps to
+// the arena with one offset: bits [0,62) = arena offset (in floats) of the tile's first float,
+// bit 62 = every row of the tile was created by this request. All ones = no shortcut.
+constexpr uint64_t kTileNotAffine = ~0ull;
+constexpr uint64_t kTileFresh = 1ull << 62;
+constexpr uint64_t kTileOffsetMask = kTileFresh - 1;
+
 // sticky device-side error bits (DevState::error)
 constexpr unsigned kDevErrLenChanged = 1u;  // var-len push: stored length differs
 constexpr unsigned kDevErrFull = 2u;        // probe sequence found no free slot (host sizing bug)
@@ -37,7 +45,6 @@ constexpr unsigned kDevErrDuplicate = 32u;    // the same key twice in one reque
 constexpr uint64_t kPayloadUnset = ~0ull;
 
 constexpr int kBlock = 256;             // threads per workgroup of every kernel here (4 waves)
-constexpr unsigned kSpanMax = 1024;     // keys whose offsets a row-kernel workgroup stages in LDS
 
 struct __align__(16) Slot {
   uint64_t key;

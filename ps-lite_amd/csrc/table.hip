@@ -107,6 +107,7 @@ struct pskv_table {
 
   GrowBuf ws;         // per-request workspace (row references, offsets)
   GrowBuf tiles;      // VARLEN: first key of every request-side tile
+  GrowBuf tiles_aff;  // VARLEN: arena offset of the tiles whose rows lie back to back
   GrowBuf stage;      // device copies of host-resident request buffers
   GrowBuf stage_out;  // device-side response of a host-resident or undersized pull
   bool no_growth = false;  // set while dumping: every key is known to be present
@@ -182,7 +183,8 @@ int grow(pskv_table* t, GrowBuf* b, size_t bytes) {
   if (bytes <= b->bytes) return PSKV_OK;
   size_t want = std::max(bytes, b->bytes + b->bytes / 2);
   want = (want + 255) & ~(size_t)255;
-  if (b == &t->ws || b == &t->tiles || b == &t->cache_keys || b == &t->cache_lens)
+  if (b == &t->ws || b == &t->tiles || b == &t->tiles_aff || b == &t->cache_keys ||
+      b == &t->cache_lens)
     t->cache_valid = false;  // the contents do not survive a reallocation
   if (b->ptr) {
     // earlier requests on the stream may still read the old buffer
@@ -388,7 +390,7 @@ constexpr uint64_t kStreamFloats = 1u << 20;
 template <bool VARLEN>
 int launch_rows(pskv_table* t, int op, const RowsParams& p) {
   if (p.total == 0) return PSKV_OK;
-  const uint64_t tile = VARLEN ? kTileVar : kTileFixed;
+  const uint64_t tile = VARLEN ? kRowsVarPerBlock : kTileFixed;  // request-side floats per workgroup
   const uint64_t ntiles = (p.total + tile - 1) / tile;
   if (ntiles > 0x7fffffffull) return set_error(PSKV_EINVAL, "request too large");
   const dim3 grid((unsigned)ntiles), block(kBlock);
@@ -474,17 +476,39 @@ int run_fixed(pskv_table* t, Request& r) {
   return PSKV_OK;
 }
 
-// Grows the tile table to `total` request-side floats and fills it.
-int make_tile_keys(pskv_table* t, const uint64_t* off, uint64_t n, uint64_t total,
-                   const uint32_t** tile_key, const ReqTag& tag) {
-  const uint64_t ntiles = (total + kTileVar - 1) / kTileVar;
-  int rc = grow(t, &t->tiles, (ntiles + 1) * sizeof(uint32_t));
+// Room in the two tile tables for `floats` request-side floats.
+int grow_tile_tables(pskv_table* t, uint64_t floats, uint64_t* ntiles_cap) {
+  *ntiles_cap = (floats + kTileVar - 1) / kTileVar;
+  int rc = grow(t, &t->tiles, (*ntiles_cap + 1) * sizeof(uint32_t));
+  if (rc) return rc;
+  return grow(t, &t->tiles_aff, (*ntiles_cap + 1) * sizeof(uint64_t));
+}
+
+// Marks the tiles whose rows lie back to back in the arena; needs the row references, so it
+// runs after the lookup kernel.
+int launch_tile_affine(pskv_table* t, const uint64_t* off, const uint64_t* ref, uint64_t n,
+                       uint64_t ntiles_cap, const ReqTag& tag) {
+  k_tile_affine<<<dim3(grid_for(ntiles_cap, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(
+      off, ref, n, static_cast<const uint32_t*>(t->tiles.ptr), static_cast<uint64_t*>(t->tiles_aff.ptr),
+      ntiles_cap, (uint64_t)kTileVar, (const DevState*)t->st, tag);
+  PSKV_HIP(hipGetLastError());
+  return PSKV_OK;
+}
+
+// Fills both tile tables of a pull whose offsets come from the stored lens.
+int make_tile_tables(pskv_table* t, const uint64_t* off, const uint64_t* ref, uint64_t n,
+                     uint64_t floats, RowsParams* p, const ReqTag& tag) {
+  uint64_t ntiles_cap = 0;
+  int rc = grow_tile_tables(t, floats, &ntiles_cap);
   if (rc) return rc;
   uint32_t* tk = static_cast<uint32_t*>(t->tiles.ptr);
   k_tile_keys<<<dim3(grid_for(n, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(
-      off, n, tk, ntiles, (uint64_t)kTileVar, (const DevState*)t->st, tag);
+      off, n, tk, ntiles_cap, (uint64_t)kTileVar, (const DevState*)t->st, tag);
   PSKV_HIP(hipGetLastError());
-  *tile_key = tk;
+  rc = launch_tile_affine(t, off, ref, n, ntiles_cap, tag);
+  if (rc) return rc;
+  p->tile_key = tk;
+  p->tile_aff = static_cast<const uint64_t*>(t->tiles_aff.ptr);
   return PSKV_OK;
 }
 
@@ -505,8 +529,8 @@ int run_varlen(pskv_table* t, Request& r) {
   if (rc) return rc;
   const bool async_pull = r.pull && !r.push && !r.need_total;
   const uint64_t tiles_for = r.push ? r.nvals : (async_pull ? r.out_cap : 0);
-  const uint64_t tiles_cap = (tiles_for + kTileVar - 1) / kTileVar;
-  rc = grow(t, &t->tiles, (tiles_cap + 1) * sizeof(uint32_t));
+  uint64_t tiles_cap = 0;
+  rc = grow_tile_tables(t, tiles_for, &tiles_cap);
   if (rc) return rc;
 
   Carver c(t->ws.ptr);
@@ -549,7 +573,10 @@ int run_varlen(pskv_table* t, Request& r) {
     t->cache_n = r.n;
     t->cache_nvals = r.nvals;
     if (r.nvals) {
+      rc = launch_tile_affine(t, off, ref, r.n, tiles_cap, tag);
+      if (rc) return rc;
       p.tile_key = push_tile_key;
+      p.tile_aff = static_cast<const uint64_t*>(t->tiles_aff.ptr);
       p.req = const_cast<float*>(r.vals);
       p.arena = t->arena;
       p.total = r.nvals;
@@ -586,7 +613,7 @@ int run_varlen(pskv_table* t, Request& r) {
       // size from the scan, and a response that does not fit is reported by the next sync.
       if (r.out_cap) {
         if (!r.out) return set_error(PSKV_EINVAL, "null out");
-        rc = make_tile_keys(t, off, r.n, r.out_cap, &p.tile_key, tag);
+        rc = make_tile_tables(t, off, ref, r.n, r.out_cap, &p, tag);
         if (rc) return rc;
         p.req = r.out;
         p.arena = t->arena;
@@ -614,7 +641,7 @@ int run_varlen(pskv_table* t, Request& r) {
         r.out = static_cast<float*>(t->stage_out.ptr);
       }
       if (!r.out) return set_error(PSKV_EINVAL, "null out");
-      rc = make_tile_keys(t, off, r.n, total, &p.tile_key, tag);
+      rc = make_tile_tables(t, off, ref, r.n, total, &p, tag);
       if (rc) return rc;
       p.req = r.out;
       p.arena = t->arena;
@@ -857,6 +884,7 @@ int pskv_table_destroy(pskv_table* t) {
   if (t->ws.ptr) (void)hipFree(t->ws.ptr);
   if (t->stage.ptr) (void)hipFree(t->stage.ptr);
   if (t->tiles.ptr) (void)hipFree(t->tiles.ptr);
+  if (t->tiles_aff.ptr) (void)hipFree(t->tiles_aff.ptr);
   if (t->cache_keys.ptr) (void)hipFree(t->cache_keys.ptr);
   if (t->cache_lens.ptr) (void)hipFree(t->cache_lens.ptr);
   if (t->stage_out.ptr) (void)hipFree(t->stage_out.ptr);

@@ -290,6 +290,55 @@ __global__ __launch_bounds__(kBlock) void k_tile_keys(const uint64_t* __restrict
   }
 }
 
+// VARLEN: finds the tiles whose rows lie back to back in the arena (see kTileNotAffine). One
+// thread per tile walks the rows that start inside its tile; tiles with more than
+// kAffineWalk rows, and tiles that mix created and existing rows, are left to the general path.
+constexpr unsigned kAffineWalk = 96;
+__global__ __launch_bounds__(kBlock) void k_tile_affine(const uint64_t* __restrict__ off,
+                                                       const uint64_t* __restrict__ ref,
+                                                       uint64_t n,
+                                                       const uint32_t* __restrict__ tile_key,
+                                                       uint64_t* __restrict__ tile_aff,
+                                                       uint64_t ntiles_cap, uint64_t tile,
+                                                       const DevState* st, ReqTag tag) {
+  if (cache_same(st, tag)) return;  // the table of the cached request is this request's
+  // a refused request has no usable offsets, tile table or references, and moves no data
+  if (st->req_error & (kDevErrBadLen | kDevErrSizeMismatch)) return;
+  const uint64_t total = off[n];
+  uint64_t ntiles = (total + tile - 1) / tile;
+  if (ntiles > ntiles_cap) ntiles = ntiles_cap;
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t wt = (uint64_t)blockIdx.x * kBlock + threadIdx.x; wt < ntiles; wt += stride) {
+    const uint64_t f0 = wt * tile;
+    const uint64_t f1 = f0 + tile < total ? f0 + tile : total;
+    uint64_t j = tile_key[wt];  // the row that owns float f0: it has floats
+    uint64_t r = j < n ? ref[j] : kRefAbsent;
+    uint64_t result = kTileNotAffine;
+    if (r != kRefAbsent) {
+      uint64_t begin = off[j], end = off[j + 1];
+      const uint64_t base = (((r & ~kRefNew) >> kLenBits) << 2) + (f0 - begin);
+      uint64_t expected = ((r & ~kRefNew) >> kLenBits) + ((end - begin + 3) >> 2);
+      unsigned fresh = (r & kRefNew) ? 1u : 0u, old = (r & kRefNew) ? 0u : 1u, walked = 0;
+      bool ok = true;
+      while (ok && end < f1 && j + 1 < n) {  // row j+1 starts inside the tile
+        if ((end - begin) & 3) ok = false;   // padding after the row breaks the 1:1 mapping
+        ++j;
+        begin = end;
+        end = off[j + 1];
+        if (++walked > kAffineWalk) ok = false;
+        if (end == begin) continue;          // a row without floats takes no part
+        r = ref[j];
+        if (r == kRefAbsent || ((r & ~kRefNew) >> kLenBits) != expected) ok = false;
+        expected += (end - begin + 3) >> 2;
+        if (r & kRefNew) ++fresh; else ++old;
+      }
+      if (ok && old == 0) result = base | kTileFresh;
+      if (ok && fresh == 0) result = base;
+    }
+    tile_aff[wt] = result;
+  }
+}
+
 // ---------------------------------------------------------------------------------
 // Row modes, step 2: stream the values.
 // A workgroup owns one tile of consecutive floats of the request-side
@@ -305,6 +354,7 @@ struct RowsParams {
   const uint64_t* ref;       // n row references from the lookup kernel
   const uint64_t* off;       // VARLEN: n+1 request-side row offsets in floats
   const uint32_t* tile_key;  // VARLEN: ntiles+1 entries
+  const uint64_t* tile_aff;  // VARLEN: ntiles entries (kTileNotAffine or the tile's arena offset)
   DevState* st;
   uint64_t n;
   uint64_t total;         // floats in req
@@ -345,19 +395,21 @@ __device__ __forceinline__ void vstore(V v, V* p) {
   if (STREAM) __builtin_nontemporal_store(v, p); else *p = v;
 }
 
-template <int OP, int VEC, bool VARLEN, bool STREAM, unsigned TILE>
-__device__ __forceinline__ void rows_tile(const RowsParams& p, uint64_t total, int32_t* s_off,
-                                          uint64_t* s_ref, bool rejected) {
+// FIXED rows: a workgroup owns TILE consecutive request-side floats; the row of an element
+// follows from a division (one compare when a row is at least a tile long).
+template <int OP, int VEC, bool STREAM, unsigned TILE>
+__device__ __forceinline__ void rows_tile_fixed(const RowsParams& p, uint64_t total) {
   using V = typename VecT<VEC>::type;
   constexpr int kIter = TILE / (VEC * kBlock);      // elements per thread
   constexpr int kGroup = kIter < 4 ? kIter : 4;     // loads issued back to back
   static_assert(kIter >= 1 && kIter % kGroup == 0, "tile does not divide over the workgroup");
   const uint64_t f0 = (uint64_t)blockIdx.x * TILE;
+  if (f0 >= total) return;
   const uint32_t tile_floats = (uint32_t)((total - f0 < (uint64_t)TILE) ? (total - f0) : (uint64_t)TILE);
   const uint32_t nelem = tile_floats / VEC;
 
   // The request-side loads depend on nothing but the tile index: issue them first so that
-  // they are in flight while the row references are fetched and searched.
+  // they are in flight while the row references are fetched.
   V x[kIter];
   if (OP == kOpAcc) {
 #pragma unroll
@@ -367,28 +419,8 @@ __device__ __forceinline__ void rows_tile(const RowsParams& p, uint64_t total, i
       if (le < nelem) x[i] = vload<STREAM>(reinterpret_cast<const V*>(p.req + f0 + le * VEC));
     }
   }
-
-  // FIXED: row and offset of the tile's first float
-  uint64_t j0 = 0, rem0 = 0;
-  // VARLEN: keys that overlap the tile
-  uint64_t j_lo = 0;
-  uint32_t span = 0;
-  bool staged = false;
-  if (VARLEN) {
-    j_lo = p.tile_key[blockIdx.x];
-    span = (uint32_t)((uint64_t)p.tile_key[blockIdx.x + 1] - j_lo + 1);
-    staged = span <= kSpanMax;
-    if (staged) {
-      for (uint32_t s = threadIdx.x; s <= span; s += kBlock) {
-        s_off[s] = (int32_t)(int64_t)(p.off[j_lo + s] - f0);
-        if (s < span) s_ref[s] = p.ref[j_lo + s];
-      }
-      __syncthreads();
-    }
-  } else {
-    j0 = f0 / p.k;
-    rem0 = f0 - j0 * p.k;
-  }
+  const uint64_t j0 = f0 / p.k;           // row of the tile's first float
+  const uint64_t rem0 = f0 - j0 * p.k;    // and its offset in that row
 
 #pragma unroll
   for (int g = 0; g < kIter; g += kGroup) {
@@ -404,43 +436,19 @@ __device__ __forceinline__ void rows_tile(const RowsParams& p, uint64_t total, i
       dst[u] = nullptr;
       fresh[u] = false;
       if (!live[u]) continue;
-      uint64_t r, within;
-      if (VARLEN) {
-        if (staged) {
-          // last key whose first float is at or before lf (zero-length rows repeat an offset)
-          uint32_t lo = 0, hi = span;
-          while (lo < hi) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (s_off[mid] <= (int32_t)lf[u]) lo = mid + 1; else hi = mid;
-          }
-          r = s_ref[lo - 1];
-          within = (uint64_t)((int32_t)lf[u] - s_off[lo - 1]);
-        } else {
-          const uint64_t f = f0 + lf[u];
-          uint64_t lo = j_lo, hi = j_lo + span;
-          while (lo < hi) {
-            const uint64_t mid = (lo + hi) >> 1;
-            if (p.off[mid] <= f) lo = mid + 1; else hi = mid;
-          }
-          r = p.ref[lo - 1];
-          within = f - p.off[lo - 1];
-        }
-        dst[u] = reinterpret_cast<V*>(p.arena + (((r & ~kRefNew) >> kLenBits) << 2) + within);
+      const uint64_t xoff = rem0 + lf[u];
+      uint64_t q, within;
+      if (p.k >= (uint64_t)TILE) {
+        q = xoff >= p.k ? 1u : 0u;
+        within = q ? xoff - p.k : xoff;
       } else {
-        const uint64_t xoff = rem0 + lf[u];
-        uint64_t q;
-        if (p.k >= (uint64_t)TILE) {
-          q = xoff >= p.k ? 1u : 0u;
-          within = q ? xoff - p.k : xoff;
-        } else {
-          const uint32_t q32 = (uint32_t)xoff / (uint32_t)p.k;
-          q = q32;
-          within = (uint32_t)xoff - q32 * (uint32_t)p.k;
-        }
-        r = p.ref[j0 + q];
-        dst[u] = reinterpret_cast<V*>(p.arena + (r & ~kRefNew) * p.k + within);
+        const uint32_t q32 = (uint32_t)xoff / (uint32_t)p.k;
+        q = q32;
+        within = (uint32_t)xoff - q32 * (uint32_t)p.k;
       }
-      if (r == kRefAbsent) {  // only after a full table, which the host sizing rules out
+      const uint64_t r = p.ref[j0 + q];
+      dst[u] = reinterpret_cast<V*>(p.arena + (r & ~kRefNew) * p.k + within);
+      if (r == kRefAbsent) {  // a key the lookup refused (duplicate in the request, full table)
         live[u] = false;
         continue;
       }
@@ -456,13 +464,8 @@ __device__ __forceinline__ void rows_tile(const RowsParams& p, uint64_t total, i
     for (int u = 0; u < kGroup; ++u) {
       if (!live[u]) continue;
       if (OP == kOpAcc) {
-        if (rejected) {
-          // a refused push changes no stored value; rows it created stay, as zero rows
-          if (fresh[u]) vstore<STREAM>(VecT<VEC>::zero(), dst[u]);
-        } else {
-          // a created row is a zero row first (0.0f + v), kv_app.h:454
-          vstore<STREAM>(y[u] + x[g + u], dst[u]);
-        }
+        // a created row is a zero row first (0.0f + v), kv_app.h:454
+        vstore<STREAM>(y[u] + x[g + u], dst[u]);
       } else {
         vstore<STREAM>(y[u], reinterpret_cast<V*>(p.req + f0 + lf[u]));
         if (fresh[u]) vstore<STREAM>(VecT<VEC>::zero(), dst[u]);  // pull created the row: zeros
@@ -471,18 +474,157 @@ __device__ __forceinline__ void rows_tile(const RowsParams& p, uint64_t total, i
   }
 }
 
-// Request-side floats one workgroup handles. One 128-bit access per lane and many small
-// workgroups stream fastest on this GPU (6.5 TB/s for `row += in` against 5.5 TB/s with
-// four accesses per lane), so the fixed-length kernel uses 1024. The var-len kernel pays
-// an LDS staging step per tile; 2048 measured best for it (1024 and 4096 are 3-10 % slower).
+// VARLEN rows: a WAVEFRONT owns WTILE consecutive request-side floats. The tile table names
+// the first key that overlaps them; the wavefront stages the offsets and row references of
+// the keys that overlap its tile in its own piece of LDS (no workgroup barrier: the four
+// wavefronts of a workgroup never wait for each other) and finds the row of each element by
+// binary search there. Tiles that overlap more than kWaveSpan keys (rows of a float or two)
+// search the global arrays instead.
+constexpr unsigned kWaveSpan = 128;
+
+template <int OP, int VEC, bool STREAM, unsigned WTILE>
+__device__ __forceinline__ void rows_wave_varlen(const RowsParams& p, uint64_t total,
+                                                 int32_t* s_off_all, uint64_t* s_ref_all,
+                                                 bool rejected) {
+  using V = typename VecT<VEC>::type;
+  constexpr int kIter = WTILE / (VEC * 64);  // elements per lane
+  static_assert(kIter >= 1 && kIter <= 8, "wave tile out of range");
+  const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint64_t wt = (uint64_t)blockIdx.x * (kBlock / 64) + wave;
+  const uint64_t f0 = wt * WTILE;
+  if (f0 >= total) return;  // the whole wavefront leaves; nothing below synchronises workgroups
+  const uint32_t tile_floats = (uint32_t)((total - f0 < (uint64_t)WTILE) ? (total - f0) : (uint64_t)WTILE);
+  const uint32_t nelem = tile_floats / VEC;
+
+  V x[kIter];
+  if (OP == kOpAcc) {
+#pragma unroll
+    for (int i = 0; i < kIter; ++i) {
+      const uint32_t le = (uint32_t)i * 64 + lane;
+      x[i] = VecT<VEC>::zero();
+      if (le < nelem) x[i] = vload<STREAM>(reinterpret_cast<const V*>(p.req + f0 + le * VEC));
+    }
+  }
+
+  // Shortcut: the rows of this tile lie back to back in the arena, so the tile maps to it with
+  // one offset and neither the row table nor a search is needed (wavefront-uniform branch).
+  if (VEC == 4) {
+    const uint64_t aff = p.tile_aff[wt];
+    if (aff != kTileNotAffine) {
+      const bool tile_fresh = (aff & kTileFresh) != 0 && !p.ignore_new;
+      V* base = reinterpret_cast<V*>(p.arena + (aff & kTileOffsetMask));
+      V y[kIter];
+#pragma unroll
+      for (int i = 0; i < kIter; ++i) {
+        const uint32_t le = (uint32_t)i * 64 + lane;
+        y[i] = VecT<VEC>::zero();
+        if (le < nelem && !tile_fresh) y[i] = vload<STREAM>(base + le);
+      }
+#pragma unroll
+      for (int i = 0; i < kIter; ++i) {
+        const uint32_t le = (uint32_t)i * 64 + lane;
+        if (le >= nelem) continue;
+        if (OP == kOpAcc) {
+          if (rejected) {
+            if (tile_fresh) vstore<STREAM>(VecT<VEC>::zero(), base + le);
+          } else {
+            vstore<STREAM>(y[i] + x[i], base + le);
+          }
+        } else {
+          vstore<STREAM>(y[i], reinterpret_cast<V*>(p.req + f0 + le * VEC));
+        }
+      }
+      return;
+    }
+  }
+
+  const uint64_t j_lo = p.tile_key[wt];
+  const uint32_t span = (uint32_t)((uint64_t)p.tile_key[wt + 1] - j_lo + 1);
+  const bool staged = span <= kWaveSpan;
+  int32_t* s_off = s_off_all + wave * kWaveSpan;
+  uint64_t* s_ref = s_ref_all + wave * kWaveSpan;
+  if (staged) {
+    for (uint32_t s = lane; s < span; s += 64) {
+      s_off[s] = (int32_t)(int64_t)(p.off[j_lo + s] - f0);
+      s_ref[s] = p.ref[j_lo + s];
+    }
+    // the wavefront's own LDS writes, visible to all of its lanes before the reads below
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+
+  V y[kIter];
+  V* dst[kIter];
+  bool live[kIter], fresh[kIter];
+#pragma unroll
+  for (int i = 0; i < kIter; ++i) {
+    const uint32_t le = (uint32_t)i * 64 + lane;
+    const uint32_t lf = le * VEC;
+    live[i] = le < nelem;
+    dst[i] = nullptr;
+    fresh[i] = false;
+    if (!live[i]) continue;
+    uint64_t r, within;
+    if (staged) {
+      // last key whose first float is at or before lf (zero-length rows repeat an offset)
+      uint32_t lo = 0, hi = span;
+      while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (s_off[mid] <= (int32_t)lf) lo = mid + 1; else hi = mid;
+      }
+      r = s_ref[lo - 1];
+      within = (uint64_t)((int32_t)lf - s_off[lo - 1]);
+    } else {
+      const uint64_t f = f0 + lf;
+      uint64_t lo = j_lo, hi = j_lo + span;
+      while (lo < hi) {
+        const uint64_t mid = (lo + hi) >> 1;
+        if (p.off[mid] <= f) lo = mid + 1; else hi = mid;
+      }
+      r = p.ref[lo - 1];
+      within = f - p.off[lo - 1];
+    }
+    dst[i] = reinterpret_cast<V*>(p.arena + (((r & ~kRefNew) >> kLenBits) << 2) + within);
+    if (r == kRefAbsent) {  // a key the lookup refused (duplicate in the request, full table)
+      live[i] = false;
+      continue;
+    }
+    fresh[i] = (r & kRefNew) != 0 && !p.ignore_new;
+  }
+#pragma unroll
+  for (int i = 0; i < kIter; ++i) {
+    y[i] = VecT<VEC>::zero();
+    if (live[i] && !fresh[i]) y[i] = vload<STREAM>(dst[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < kIter; ++i) {
+    if (!live[i]) continue;
+    const uint32_t lf = ((uint32_t)i * 64 + lane) * VEC;
+    if (OP == kOpAcc) {
+      if (rejected) {
+        // a refused push changes no stored value; rows it created stay, as zero rows
+        if (fresh[i]) vstore<STREAM>(VecT<VEC>::zero(), dst[i]);
+      } else {
+        vstore<STREAM>(y[i] + x[i], dst[i]);  // a created row is a zero row first (0.0f + v)
+      }
+    } else {
+      vstore<STREAM>(y[i], reinterpret_cast<V*>(p.req + f0 + lf));
+    }
+  }
+}
+
+// Request-side floats per workgroup (fixed rows) and per wavefront (var-len rows). One
+// 128-bit access per lane and many small workgroups stream fastest on this GPU (6.5 TB/s for
+// `row += in` against 5.5 TB/s with four accesses per lane).
 constexpr unsigned kTileFixed = 1024;
-constexpr unsigned kTileVar = PSKV_TILE_VAR;
+constexpr unsigned kTileVar = PSKV_TILE_VAR;        // per wavefront; the tile table's granularity
+constexpr unsigned kRowsVarPerBlock = kTileVar * (kBlock / 64);
 
 template <int OP, bool VARLEN, bool STREAM>
 __global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
-  constexpr unsigned TILE = VARLEN ? kTileVar : kTileFixed;
-  __shared__ int32_t s_off[VARLEN ? kSpanMax + 1 : 1];
-  __shared__ uint64_t s_ref[VARLEN ? kSpanMax : 1];
+  __shared__ int32_t s_off[VARLEN ? kWaveSpan * (kBlock / 64) : 1];
+  __shared__ uint64_t s_ref[VARLEN ? kWaveSpan * (kBlock / 64) : 1];
   bool rejected = false;
   bool scalar = p.force_scalar != 0;
   uint64_t total = p.total;
@@ -501,12 +643,18 @@ __global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
         return;
       }
     }
-  }
-  if ((uint64_t)blockIdx.x * TILE >= total) return;  // the grid was sized for the room, not the data
-  if (scalar) {
-    rows_tile<OP, 1, VARLEN, STREAM, TILE>(p, total, s_off, s_ref, rejected);
+    // the grid may have been sized for the room in the caller's buffer, not for the data
+    if (scalar) {
+      rows_wave_varlen<OP, 1, STREAM, kTileVar>(p, total, s_off, s_ref, rejected);
+    } else {
+      rows_wave_varlen<OP, 4, STREAM, kTileVar>(p, total, s_off, s_ref, rejected);
+    }
   } else {
-    rows_tile<OP, 4, VARLEN, STREAM, TILE>(p, total, s_off, s_ref, rejected);
+    if (scalar) {
+      rows_tile_fixed<OP, 1, STREAM, kTileFixed>(p, total);
+    } else {
+      rows_tile_fixed<OP, 4, STREAM, kTileFixed>(p, total);
+    }
   }
 }
 
