@@ -26,11 +26,8 @@ constexpr uint64_t kLenMask = (1ull << kLenBits) - 1;
 
 // Per-tile shortcut of the var-len row kernel. When the rows that overlap a request-side tile
 // lie in the arena back to back, in request order and without padding, the whole tile maps to
-// the arena with one offset: bits [0,62) = arena offset (in floats) of the tile's first float,
-// bit 62 = every row of the tile was created by this request. All ones = no shortcut.
+// the arena with one offset: the arena position (in floats) of the tile's first float.
 constexpr uint64_t kTileNotAffine = ~0ull;
-constexpr uint64_t kTileFresh = 1ull << 62;
-constexpr uint64_t kTileOffsetMask = kTileFresh - 1;
 
 // sticky device-side error bits (DevState::error)
 constexpr unsigned kDevErrLenChanged = 1u;  // var-len push: stored length differs

@@ -484,20 +484,10 @@ int grow_tile_tables(pskv_table* t, uint64_t floats, uint64_t* ntiles_cap) {
   return grow(t, &t->tiles_aff, (*ntiles_cap + 1) * sizeof(uint64_t));
 }
 
-// Marks the tiles whose rows lie back to back in the arena; needs the row references, so it
-// runs after the lookup kernel.
-int launch_tile_affine(pskv_table* t, const uint64_t* off, const uint64_t* ref, uint64_t n,
-                       uint64_t ntiles_cap, const ReqTag& tag) {
-  k_tile_affine<<<dim3(grid_for(ntiles_cap, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(
-      off, ref, n, static_cast<const uint32_t*>(t->tiles.ptr), static_cast<uint64_t*>(t->tiles_aff.ptr),
-      ntiles_cap, (uint64_t)kTileVar, (const DevState*)t->st, tag);
-  PSKV_HIP(hipGetLastError());
-  return PSKV_OK;
-}
-
-// Fills both tile tables of a pull whose offsets come from the stored lens.
-int make_tile_tables(pskv_table* t, const uint64_t* off, const uint64_t* ref, uint64_t n,
-                     uint64_t floats, RowsParams* p, const ReqTag& tag) {
+// Fills the tile table of a pull whose offsets come from the stored lens (the row kernel
+// fills the other one).
+int make_tile_tables(pskv_table* t, const uint64_t* off, uint64_t n, uint64_t floats,
+                     RowsParams* p, const ReqTag& tag) {
   uint64_t ntiles_cap = 0;
   int rc = grow_tile_tables(t, floats, &ntiles_cap);
   if (rc) return rc;
@@ -505,10 +495,8 @@ int make_tile_tables(pskv_table* t, const uint64_t* off, const uint64_t* ref, ui
   k_tile_keys<<<dim3(grid_for(n, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(
       off, n, tk, ntiles_cap, (uint64_t)kTileVar, (const DevState*)t->st, tag);
   PSKV_HIP(hipGetLastError());
-  rc = launch_tile_affine(t, off, ref, n, ntiles_cap, tag);
-  if (rc) return rc;
   p->tile_key = tk;
-  p->tile_aff = static_cast<const uint64_t*>(t->tiles_aff.ptr);
+  p->tile_aff = static_cast<uint64_t*>(t->tiles_aff.ptr);
   return PSKV_OK;
 }
 
@@ -573,10 +561,8 @@ int run_varlen(pskv_table* t, Request& r) {
     t->cache_n = r.n;
     t->cache_nvals = r.nvals;
     if (r.nvals) {
-      rc = launch_tile_affine(t, off, ref, r.n, tiles_cap, tag);
-      if (rc) return rc;
       p.tile_key = push_tile_key;
-      p.tile_aff = static_cast<const uint64_t*>(t->tiles_aff.ptr);
+      p.tile_aff = static_cast<uint64_t*>(t->tiles_aff.ptr);
       p.req = const_cast<float*>(r.vals);
       p.arena = t->arena;
       p.total = r.nvals;
@@ -613,7 +599,7 @@ int run_varlen(pskv_table* t, Request& r) {
       // size from the scan, and a response that does not fit is reported by the next sync.
       if (r.out_cap) {
         if (!r.out) return set_error(PSKV_EINVAL, "null out");
-        rc = make_tile_tables(t, off, ref, r.n, r.out_cap, &p, tag);
+        rc = make_tile_tables(t, off, r.n, r.out_cap, &p, tag);
         if (rc) return rc;
         p.req = r.out;
         p.arena = t->arena;
@@ -641,7 +627,7 @@ int run_varlen(pskv_table* t, Request& r) {
         r.out = static_cast<float*>(t->stage_out.ptr);
       }
       if (!r.out) return set_error(PSKV_EINVAL, "null out");
-      rc = make_tile_tables(t, off, ref, r.n, total, &p, tag);
+      rc = make_tile_tables(t, off, r.n, total, &p, tag);
       if (rc) return rc;
       p.req = r.out;
       p.arena = t->arena;

@@ -290,55 +290,6 @@ __global__ __launch_bounds__(kBlock) void k_tile_keys(const uint64_t* __restrict
   }
 }
 
-// VARLEN: finds the tiles whose rows lie back to back in the arena (see kTileNotAffine). One
-// thread per tile walks the rows that start inside its tile; tiles with more than
-// kAffineWalk rows, and tiles that mix created and existing rows, are left to the general path.
-constexpr unsigned kAffineWalk = 96;
-__global__ __launch_bounds__(kBlock) void k_tile_affine(const uint64_t* __restrict__ off,
-                                                       const uint64_t* __restrict__ ref,
-                                                       uint64_t n,
-                                                       const uint32_t* __restrict__ tile_key,
-                                                       uint64_t* __restrict__ tile_aff,
-                                                       uint64_t ntiles_cap, uint64_t tile,
-                                                       const DevState* st, ReqTag tag) {
-  if (cache_same(st, tag)) return;  // the table of the cached request is this request's
-  // a refused request has no usable offsets, tile table or references, and moves no data
-  if (st->req_error & (kDevErrBadLen | kDevErrSizeMismatch)) return;
-  const uint64_t total = off[n];
-  uint64_t ntiles = (total + tile - 1) / tile;
-  if (ntiles > ntiles_cap) ntiles = ntiles_cap;
-  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-  for (uint64_t wt = (uint64_t)blockIdx.x * kBlock + threadIdx.x; wt < ntiles; wt += stride) {
-    const uint64_t f0 = wt * tile;
-    const uint64_t f1 = f0 + tile < total ? f0 + tile : total;
-    uint64_t j = tile_key[wt];  // the row that owns float f0: it has floats
-    uint64_t r = j < n ? ref[j] : kRefAbsent;
-    uint64_t result = kTileNotAffine;
-    if (r != kRefAbsent) {
-      uint64_t begin = off[j], end = off[j + 1];
-      const uint64_t base = (((r & ~kRefNew) >> kLenBits) << 2) + (f0 - begin);
-      uint64_t expected = ((r & ~kRefNew) >> kLenBits) + ((end - begin + 3) >> 2);
-      unsigned fresh = (r & kRefNew) ? 1u : 0u, old = (r & kRefNew) ? 0u : 1u, walked = 0;
-      bool ok = true;
-      while (ok && end < f1 && j + 1 < n) {  // row j+1 starts inside the tile
-        if ((end - begin) & 3) ok = false;   // padding after the row breaks the 1:1 mapping
-        ++j;
-        begin = end;
-        end = off[j + 1];
-        if (++walked > kAffineWalk) ok = false;
-        if (end == begin) continue;          // a row without floats takes no part
-        r = ref[j];
-        if (r == kRefAbsent || ((r & ~kRefNew) >> kLenBits) != expected) ok = false;
-        expected += (end - begin + 3) >> 2;
-        if (r & kRefNew) ++fresh; else ++old;
-      }
-      if (ok && old == 0) result = base | kTileFresh;
-      if (ok && fresh == 0) result = base;
-    }
-    tile_aff[wt] = result;
-  }
-}
-
 // ---------------------------------------------------------------------------------
 // Row modes, step 2: stream the values.
 // A workgroup owns one tile of consecutive floats of the request-side
@@ -354,7 +305,7 @@ struct RowsParams {
   const uint64_t* ref;       // n row references from the lookup kernel
   const uint64_t* off;       // VARLEN: n+1 request-side row offsets in floats
   const uint32_t* tile_key;  // VARLEN: ntiles+1 entries
-  const uint64_t* tile_aff;  // VARLEN: ntiles entries (kTileNotAffine or the tile's arena offset)
+  uint64_t* tile_aff;        // VARLEN: ntiles entries (kTileNotAffine or the tile's arena offset)
   DevState* st;
   uint64_t n;
   uint64_t total;         // floats in req
@@ -485,7 +436,7 @@ constexpr unsigned kWaveSpan = 128;
 template <int OP, int VEC, bool STREAM, unsigned WTILE>
 __device__ __forceinline__ void rows_wave_varlen(const RowsParams& p, uint64_t total,
                                                  int32_t* s_off_all, uint64_t* s_ref_all,
-                                                 bool rejected) {
+                                                 bool rejected, bool same) {
   using V = typename VecT<VEC>::type;
   constexpr int kIter = WTILE / (VEC * 64);  // elements per lane
   static_assert(kIter >= 1 && kIter <= 8, "wave tile out of range");
@@ -506,30 +457,27 @@ __device__ __forceinline__ void rows_wave_varlen(const RowsParams& p, uint64_t t
     }
   }
 
-  // Shortcut: the rows of this tile lie back to back in the arena, so the tile maps to it with
-  // one offset and neither the row table nor a search is needed (wavefront-uniform branch).
-  if (VEC == 4) {
+  // Shortcut of a request that repeats the cached one: if the rows of this tile lie back to
+  // back in the arena, the tile maps to it with one offset and neither the row table nor a
+  // search is needed (wavefront-uniform branch). The table was written by the row kernel of
+  // the cached request, below.
+  if (VEC == 4 && same) {
     const uint64_t aff = p.tile_aff[wt];
     if (aff != kTileNotAffine) {
-      const bool tile_fresh = (aff & kTileFresh) != 0 && !p.ignore_new;
-      V* base = reinterpret_cast<V*>(p.arena + (aff & kTileOffsetMask));
+      V* base = reinterpret_cast<V*>(p.arena + aff);
       V y[kIter];
 #pragma unroll
       for (int i = 0; i < kIter; ++i) {
         const uint32_t le = (uint32_t)i * 64 + lane;
         y[i] = VecT<VEC>::zero();
-        if (le < nelem && !tile_fresh) y[i] = vload<STREAM>(base + le);
+        if (le < nelem) y[i] = vload<STREAM>(base + le);
       }
 #pragma unroll
       for (int i = 0; i < kIter; ++i) {
         const uint32_t le = (uint32_t)i * 64 + lane;
         if (le >= nelem) continue;
         if (OP == kOpAcc) {
-          if (rejected) {
-            if (tile_fresh) vstore<STREAM>(VecT<VEC>::zero(), base + le);
-          } else {
-            vstore<STREAM>(y[i] + x[i], base + le);
-          }
+          vstore<STREAM>(y[i] + x[i], base + le);
         } else {
           vstore<STREAM>(y[i], reinterpret_cast<V*>(p.req + f0 + le * VEC));
         }
@@ -541,17 +489,38 @@ __device__ __forceinline__ void rows_wave_varlen(const RowsParams& p, uint64_t t
   const uint64_t j_lo = p.tile_key[wt];
   const uint32_t span = (uint32_t)((uint64_t)p.tile_key[wt + 1] - j_lo + 1);
   const bool staged = span <= kWaveSpan;
-  int32_t* s_off = s_off_all + wave * kWaveSpan;
+  int32_t* s_off = s_off_all + wave * (kWaveSpan + 1);
   uint64_t* s_ref = s_ref_all + wave * kWaveSpan;
   if (staged) {
-    for (uint32_t s = lane; s < span; s += 64) {
+    for (uint32_t s = lane; s <= span; s += 64) {
       s_off[s] = (int32_t)(int64_t)(p.off[j_lo + s] - f0);
-      s_ref[s] = p.ref[j_lo + s];
+      if (s < span) s_ref[s] = p.ref[j_lo + s];
     }
     // the wavefront's own LDS writes, visible to all of its lanes before the reads below
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+  if (!same) {
+    // Leave a note for requests that repeat this one: the tile is "affine" when every row
+    // with floats in it sits at the same distance from its place in the request, i.e. the
+    // rows lie back to back, in request order, without padding between them.
+    uint64_t note = kTileNotAffine;
+    if (VEC == 4 && staged) {
+      const uint64_t r0 = s_ref[0];
+      const int64_t d0 = (int64_t)(((r0 & ~kRefNew) >> kLenBits) << 2) - (int64_t)s_off[0];
+      bool bad = r0 == kRefAbsent;
+      for (uint32_t s = lane; s < span; s += 64) {
+        const bool has_floats = s_off[s + 1] > s_off[s] && s_off[s] < (int32_t)tile_floats;
+        if (has_floats) {
+          const uint64_t r = s_ref[s];
+          const int64_t d = (int64_t)(((r & ~kRefNew) >> kLenBits) << 2) - (int64_t)s_off[s];
+          bad |= r == kRefAbsent || d != d0;
+        }
+      }
+      if (__ballot(bad) == 0ull) note = (uint64_t)d0;
+    }
+    if (lane == 0) p.tile_aff[wt] = note;
   }
 
   V y[kIter];
@@ -623,7 +592,7 @@ constexpr unsigned kRowsVarPerBlock = kTileVar * (kBlock / 64);
 
 template <int OP, bool VARLEN, bool STREAM>
 __global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
-  __shared__ int32_t s_off[VARLEN ? kWaveSpan * (kBlock / 64) : 1];
+  __shared__ int32_t s_off[VARLEN ? (kWaveSpan + 1) * (kBlock / 64) : 1];
   __shared__ uint64_t s_ref[VARLEN ? kWaveSpan * (kBlock / 64) : 1];
   bool rejected = false;
   bool scalar = p.force_scalar != 0;
@@ -645,9 +614,9 @@ __global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
     }
     // the grid may have been sized for the room in the caller's buffer, not for the data
     if (scalar) {
-      rows_wave_varlen<OP, 1, STREAM, kTileVar>(p, total, s_off, s_ref, rejected);
+      rows_wave_varlen<OP, 1, STREAM, kTileVar>(p, total, s_off, s_ref, rejected, same);
     } else {
-      rows_wave_varlen<OP, 4, STREAM, kTileVar>(p, total, s_off, s_ref, rejected);
+      rows_wave_varlen<OP, 4, STREAM, kTileVar>(p, total, s_off, s_ref, rejected, same);
     }
   } else {
     if (scalar) {
