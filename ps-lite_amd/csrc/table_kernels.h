@@ -447,6 +447,14 @@ __device__ __forceinline__ void rows_wave_varlen(const RowsParams& p, uint64_t t
   const uint32_t tile_floats = (uint32_t)((total - f0 < (uint64_t)WTILE) ? (total - f0) : (uint64_t)WTILE);
   const uint32_t nelem = tile_floats / VEC;
 
+  // Loads whose addresses depend on nothing but the tile index go first: the tile's shortcut
+  // note (read even when it turns out not to be needed, so that it is not a second round
+  // trip after the decision) and the request-side values.
+  uint64_t aff = kTileNotAffine;
+  if (VEC == 4) {
+    aff = p.tile_aff[wt];
+    asm volatile("" ::"v"((unsigned)aff), "v"((unsigned)(aff >> 32)));  // keep the load up here
+  }
   V x[kIter];
   if (OP == kOpAcc) {
 #pragma unroll
@@ -462,7 +470,6 @@ __device__ __forceinline__ void rows_wave_varlen(const RowsParams& p, uint64_t t
   // search is needed (wavefront-uniform branch). The table was written by the row kernel of
   // the cached request, below.
   if (VEC == 4 && same) {
-    const uint64_t aff = p.tile_aff[wt];
     if (aff != kTileNotAffine) {
       V* base = reinterpret_cast<V*>(p.arena + aff);
       V y[kIter];
