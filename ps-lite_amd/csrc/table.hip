@@ -35,6 +35,9 @@ namespace {
 constexpr uint64_t kDefaultCapacity = 1u << 20;
 constexpr uint64_t kMinSlots = 1024;
 constexpr unsigned kMaxGrid = 1u << 20;
+// Host-resident requests up to this size (per direction) skip the copy commands: the kernels
+// read the request from, and write the response to, pinned host memory mapped into the GPU.
+constexpr size_t kSmallBytes = 1024u << 10;
 
 // A device buffer that only grows. Contents are not kept across growth.
 struct GrowBuf {
@@ -54,6 +57,30 @@ struct Snapshot {
   volatile uint64_t arena_top;
   volatile uint64_t seq_end;
 };
+
+// What the host reads back of the device state, written by the device into pinned host memory
+// (a one-wavefront kernel is quicker than a copy command for these few words).
+struct StateView {
+  uint64_t count;       // keys held, the side slot included
+  uint64_t arena_top;
+  uint64_t scan_total;
+  uint64_t same_epoch;
+  unsigned error, req_error, special_present, pad;
+};
+
+__global__ void k_read_state(const DevState* st, StateView* out) {
+  unsigned long long c = threadIdx.x < kCountShards ? st->count_shard[threadIdx.x * kShardStride] : 0ull;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
+  if (threadIdx.x != 0) return;
+  out->count = c;
+  out->arena_top = st->arena_top;
+  out->scan_total = st->scan_total;
+  out->same_epoch = st->same_epoch;
+  out->error = st->error;
+  out->req_error = st->req_error;
+  out->special_present = st->special_present;
+}
 
 // One wavefront, launched in front of a request's kernels when the table is close to a limit.
 __global__ void k_publish(const DevState* st, Snapshot* out, uint64_t seq) {
@@ -98,7 +125,7 @@ struct pskv_table {
   uint64_t log_keys[kLog] = {0}, log_units[kLog] = {0};
   Snapshot* snap = nullptr;  // pinned host memory the device publishes into
   DevState* st = nullptr;  // device
-  DevState* st_host = nullptr;  // pinned mirror for read-backs
+  StateView* st_host = nullptr;  // pinned: what read_state() last read of the device state
 
   // row modes
   float* arena = nullptr;
@@ -108,6 +135,8 @@ struct pskv_table {
   GrowBuf ws;         // per-request workspace (row references, offsets)
   GrowBuf tiles;      // VARLEN: first key of every request-side tile
   GrowBuf tiles_aff;  // VARLEN: arena offset of the tiles whose rows lie back to back
+  char* small_in = nullptr;   // pinned, kSmallBytes: small host-resident requests, read in place
+  char* small_out = nullptr;  // pinned, kSmallBytes: their responses, written in place
   GrowBuf stage;      // device copies of host-resident request buffers
   GrowBuf stage_out;  // device-side response of a host-resident or undersized pull
   bool no_growth = false;  // set while dumping: every key is known to be present
@@ -213,10 +242,10 @@ struct Carver {
 };
 
 int read_state(pskv_table* t) {
-  PSKV_HIP(hipMemcpyAsync(t->st_host, t->st, sizeof(DevState), hipMemcpyDeviceToHost, t->stream));
+  k_read_state<<<dim3(1), dim3(64), 0, t->stream>>>(t->st, t->st_host);
+  PSKV_HIP(hipGetLastError());
   PSKV_HIP(hipStreamSynchronize(t->stream));
-  uint64_t c = 0;
-  for (int i = 0; i < kCountShards; ++i) c += t->st_host->count_shard[i * kShardStride];
+  const uint64_t c = t->st_host->count;
   t->count = c;
   // everything enqueued so far is complete: the bounds become exact
   t->base_seq = t->seq;
@@ -360,6 +389,8 @@ struct Request {
   uint64_t out_nvals;    // result
   bool lazy_out;         // VARLEN pull into host memory: `out` is allocated once the size is known
   bool need_total;       // VARLEN pull: the caller wants the response size back (forces a wait)
+  char* small_out;       // lazy_out: pinned room the response may go to when it fits
+  uint64_t small_out_floats;
 };
 
 int run_scalar(pskv_table* t, Request& r) {
@@ -622,9 +653,13 @@ int run_varlen(pskv_table* t, Request& r) {
                        (unsigned long long)total, (unsigned long long)r.out_cap);
     if (total) {
       if (r.lazy_out) {
-        rc = grow(t, &t->stage_out, total * sizeof(float));
-        if (rc) return rc;
-        r.out = static_cast<float*>(t->stage_out.ptr);
+        if (r.small_out && total <= r.small_out_floats) {
+          r.out = reinterpret_cast<float*>(r.small_out);
+        } else {
+          rc = grow(t, &t->stage_out, total * sizeof(float));
+          if (rc) return rc;
+          r.out = static_cast<float*>(t->stage_out.ptr);
+        }
       }
       if (!r.out) return set_error(PSKV_EINVAL, "null out");
       rc = make_tile_tables(t, off, r.n, total, &p, tag);
@@ -710,6 +745,8 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
   if (rc) return rc;
   const bool host = memkind == PSKV_MEM_HOST;
   const bool varlen = t->mode == PSKV_MODE_VARLEN;
+  bool small = false;        // host-resident request served from the pinned buffers
+  size_t small_out_at = 0;   // bytes of small_out already given away
 
   // SCALAR and FIXED know the response size up front. A response that does not fit is
   // still computed (into scratch) so that the store ends up as the reference's would:
@@ -735,28 +772,52 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
   } else {
     const bool want_lens = push && varlen;
     const bool want_out_lens = pull && varlen;
-    const size_t need = Carver::need(n, 8) + Carver::need(r.nvals, 4) +
-                        Carver::need(want_lens ? n : 0, 4) + Carver::need(want_out_lens ? n : 0, 4);
-    rc = grow(t, &t->stage, need);
-    if (rc) return rc;
-    Carver c(t->stage.ptr);
+    const size_t in_need =
+        Carver::need(n, 8) + Carver::need(r.nvals, 4) + Carver::need(want_lens ? n : 0, 4);
+    const size_t out_lens_need = Carver::need(want_out_lens ? n : 0, 4);
+    small = in_need <= kSmallBytes && out_lens_need <= kSmallBytes;
+    char* base = t->small_in;
+    if (!small) {
+      rc = grow(t, &t->stage, in_need + out_lens_need);
+      if (rc) return rc;
+      base = static_cast<char*>(t->stage.ptr);
+    }
+    Carver c(base);
     uint64_t* dkeys = c.take<uint64_t>(n);
     float* dvals = c.take<float>(r.nvals);
     int32_t* dlens = c.take<int32_t>(want_lens ? n : 0);
-    int32_t* dout_lens = c.take<int32_t>(want_out_lens ? n : 0);
-    if (n) PSKV_HIP(hipMemcpyAsync(dkeys, keys, n * 8, hipMemcpyHostToDevice, t->stream));
-    if (r.nvals) PSKV_HIP(hipMemcpyAsync(dvals, vals, r.nvals * 4, hipMemcpyHostToDevice, t->stream));
-    if (want_lens && n) PSKV_HIP(hipMemcpyAsync(dlens, lens, n * 4, hipMemcpyHostToDevice, t->stream));
+    int32_t* dout_lens = nullptr;
+    if (small) {
+      // every host-resident request ends with a wait, so the previous one is done with the buffers
+      if (n) std::memcpy(dkeys, keys, n * 8);
+      if (r.nvals) std::memcpy(dvals, vals, r.nvals * 4);
+      if (want_lens && n) std::memcpy(dlens, lens, n * 4);
+      small_out_at = out_lens_need;
+      if (want_out_lens) dout_lens = reinterpret_cast<int32_t*>(t->small_out);
+    } else {
+      dout_lens = c.take<int32_t>(want_out_lens ? n : 0);
+      if (n) PSKV_HIP(hipMemcpyAsync(dkeys, keys, n * 8, hipMemcpyHostToDevice, t->stream));
+      if (r.nvals) PSKV_HIP(hipMemcpyAsync(dvals, vals, r.nvals * 4, hipMemcpyHostToDevice, t->stream));
+      if (want_lens && n) PSKV_HIP(hipMemcpyAsync(dlens, lens, n * 4, hipMemcpyHostToDevice, t->stream));
+    }
     r.keys = dkeys;
     r.vals = dvals;
     r.lens = dlens;
     r.out_lens = want_out_lens ? dout_lens : nullptr;
     r.lazy_out = pull && varlen;
+    if (small && r.lazy_out) {
+      r.small_out = t->small_out + small_out_at;
+      r.small_out_floats = (kSmallBytes - small_out_at) / sizeof(float);
+    }
   }
   if (pull && !varlen && (host || too_small) && fixed_out) {
-    rc = grow(t, &t->stage_out, fixed_out * sizeof(float));
-    if (rc) return rc;
-    r.out = static_cast<float*>(t->stage_out.ptr);
+    if (small && !too_small && fixed_out * sizeof(float) <= kSmallBytes - small_out_at) {
+      r.out = reinterpret_cast<float*>(t->small_out + small_out_at);
+    } else {
+      rc = grow(t, &t->stage_out, fixed_out * sizeof(float));
+      if (rc) return rc;
+      r.out = static_cast<float*>(t->stage_out.ptr);
+    }
     r.out_cap = fixed_out;
   }
 
@@ -775,15 +836,27 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
                      (unsigned long long)fixed_out, (unsigned long long)out_cap);
 
   if (host) {
-    if (pull && r.out_nvals)
+    const bool out_pinned = pull && r.out_nvals && r.out >= reinterpret_cast<float*>(t->small_out) &&
+                            r.out < reinterpret_cast<float*>(t->small_out + kSmallBytes);
+    const bool lens_pinned = r.out_lens == reinterpret_cast<int32_t*>(t->small_out);
+    if (pull && r.out_nvals && !out_pinned)
       PSKV_HIP(hipMemcpyAsync(out, r.out, r.out_nvals * 4, hipMemcpyDeviceToHost, t->stream));
-    if (pull && varlen && out_lens && n)
+    if (pull && varlen && out_lens && n && !lens_pinned)
       PSKV_HIP(hipMemcpyAsync(out_lens, r.out_lens, n * 4, hipMemcpyDeviceToHost, t->stream));
-    rc = read_state(t);  // also waits for the copies above
-    if (rc) return rc;
-    rc = report_device_errors(t);
-    if (rc) t->cache_valid = false;
-    return rc;
+    if (t->mode == PSKV_MODE_SCALAR) {
+      // no device-detected errors in this mode: waiting for the stream is all that is left
+      PSKV_HIP(hipStreamSynchronize(t->stream));
+    } else {
+      rc = read_state(t);  // also waits for the copies above
+      if (rc) return rc;
+      rc = report_device_errors(t);
+      if (rc) {
+        t->cache_valid = false;
+        return rc;
+      }
+    }
+    if (out_pinned) std::memcpy(out, r.out, r.out_nvals * 4);
+    if (pull && varlen && out_lens && n && lens_pinned) std::memcpy(out_lens, r.out_lens, n * 4);
   }
   return PSKV_OK;
 }
@@ -831,9 +904,14 @@ int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
   if (rc) return fail(rc);
   if (hipMalloc(reinterpret_cast<void**>(&t->st), sizeof(DevState)) != hipSuccess ||
       hipMemsetAsync(t->st, 0, sizeof(DevState), t->stream) != hipSuccess ||
-      hipHostMalloc(reinterpret_cast<void**>(&t->st_host), sizeof(DevState), hipHostMallocDefault) !=
+      hipHostMalloc(reinterpret_cast<void**>(&t->st_host), sizeof(StateView), hipHostMallocCoherent) !=
           hipSuccess ||
       hipHostMalloc(reinterpret_cast<void**>(&t->snap), sizeof(Snapshot), hipHostMallocDefault) !=
+          hipSuccess ||
+      // coherent: the GPU does not cache these two, so each request sees what the host just wrote
+      hipHostMalloc(reinterpret_cast<void**>(&t->small_in), kSmallBytes, hipHostMallocCoherent) !=
+          hipSuccess ||
+      hipHostMalloc(reinterpret_cast<void**>(&t->small_out), kSmallBytes, hipHostMallocCoherent) !=
           hipSuccess)
     return fail(set_error(PSKV_ENOMEM, "cannot allocate table state"));
   std::memset(t->snap, 0, sizeof(Snapshot));
@@ -866,6 +944,8 @@ int pskv_table_destroy(pskv_table* t) {
   if (t->st) (void)hipFree(t->st);
   if (t->st_host) (void)hipHostFree(t->st_host);
   if (t->snap) (void)hipHostFree(t->snap);
+  if (t->small_in) (void)hipHostFree(t->small_in);
+  if (t->small_out) (void)hipHostFree(t->small_out);
   if (t->arena) (void)hipFree(t->arena);
   if (t->ws.ptr) (void)hipFree(t->ws.ptr);
   if (t->stage.ptr) (void)hipFree(t->stage.ptr);
