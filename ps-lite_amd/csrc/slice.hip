@@ -2,6 +2,7 @@
 // (include/ps/kv_app.h:517-572) and the device-side reassembly of pulled slices
 // that mirrors the callback of KVWorker::AddPullCB (kv_app.h:663-714).
 #include <algorithm>
+#include <cstring>
 #include <limits>
 #include <mutex>
 #include <numeric>
@@ -48,16 +49,33 @@ __global__ __launch_bounds__(kBlock) void k_bounds(const uint64_t* __restrict__ 
 // kv_app.h:528-541: pos[0] = lower_bound(keys, ranges[0].begin); every further
 // boundary is searched in the suffix that starts at the previous one, which for
 // sorted keys is max(previous, lower_bound over the whole array).
+// One wavefront. `pos` is device memory (read by the lens sums), `pos_host` pinned host
+// memory the caller reads after the stream wait; `sums` (may be null) is cleared for
+// the kernel that follows.
 __global__ void k_bounds_chain(const uint64_t* __restrict__ lb, uint64_t S,
-                               uint64_t* __restrict__ pos) {
-  if (blockIdx.x != 0 || threadIdx.x != 0) return;
+                               uint64_t* __restrict__ pos, uint64_t* __restrict__ pos_host,
+                               unsigned long long* __restrict__ sums) {
+  if (blockIdx.x != 0) return;
+  if (sums)
+    for (uint64_t i = threadIdx.x; i < S; i += blockDim.x) sums[i] = 0ull;
+  if (threadIdx.x != 0) return;
   uint64_t p = lb[0];
   pos[0] = p;
+  pos_host[0] = p;
   for (uint64_t i = 0; i < S; ++i) {
     const uint64_t e = lb[i + 1];
     p = e > p ? e : p;
     pos[i + 1] = p;
+    pos_host[i + 1] = p;
   }
+}
+
+// Hands the per-slice sums to the host (pinned memory).
+__global__ void k_export_sums(const unsigned long long* __restrict__ sums, uint64_t S,
+                              unsigned long long* __restrict__ sums_host) {
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < S;
+       i += (uint64_t)gridDim.x * blockDim.x)
+    sums_host[i] = sums[i];
 }
 
 // kv_app.h:565 `for (int l : kv.lens) val_end += l;` for every slice at once:
@@ -101,11 +119,16 @@ struct SliceCtx {
   hipStream_t stream = nullptr;
   void* dev = nullptr;      // device scratch: targets, lower bounds, positions, sums
   size_t dev_bytes = 0;
-  void* pinned = nullptr;   // host-visible copy of the small arrays
+  void* pinned = nullptr;   // pinned host memory the kernels read targets from and answer into
   size_t pinned_bytes = 0;
   void* stage = nullptr;    // device copy of host-resident keys / lens
   size_t stage_bytes = 0;
+  void* small = nullptr;    // pinned, kSmallStage bytes: small host-resident keys / lens, read in place
 };
+
+// Host-resident keys (+ lens) up to this size are not copied to the device: the search reads
+// a few hundred of them, and the sums one pass, straight from pinned host memory.
+constexpr size_t kSmallStage = 1024u << 10;
 
 std::mutex g_pool_mu;
 std::vector<SliceCtx*> g_pool;
@@ -156,7 +179,8 @@ int ctx_reserve(SliceCtx* c, size_t dev_bytes, size_t pinned_bytes, size_t stage
     if (c->pinned) PSKV_HIP(hipHostFree(c->pinned));
     c->pinned = nullptr;
     c->pinned_bytes = 0;
-    PSKV_HIP(hipHostMalloc(&c->pinned, pinned_bytes, hipHostMallocDefault));
+    // coherent: never cached by the GPU, so every call sees what the host wrote for it
+    PSKV_HIP(hipHostMalloc(&c->pinned, pinned_bytes, hipHostMallocCoherent));
     c->pinned_bytes = pinned_bytes;
   }
   if (stage_bytes > c->stage_bytes) {
@@ -228,52 +252,55 @@ int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, 
     SliceCtx* c = lease.c;
     if (!c) return set_error(PSKV_EHIP, "cannot create a slicer context on device %d", device);
     const bool do_sums = has_lens && nlens == n;
-    // small arrays: targets[S+1] | lb[S+1] | pos[S+1] | sums[S]
-    const size_t small = 4 * pad256((S + 1) * 8);
+    if (do_sums && S > 65535) return set_error(PSKV_EINVAL, "more than 65535 ranges with lens");
+    // device: lb[S+1] | pos[S+1] | sums[S]      pinned: targets[S+1] | pos[S+1] | sums[S]
+    const size_t arr = pad256((S + 1) * 8);
     const bool host = memkind == PSKV_MEM_HOST;
-    const size_t stage_need = host ? pad256(n * 8) + (do_sums ? pad256(n * 4) : 0) : 0;
-    int rc = ctx_reserve(c, small, small, stage_need);
+    const size_t in_bytes = pad256(n * 8) + (do_sums ? pad256(n * 4) : 0);
+    const bool in_place = host && in_bytes <= kSmallStage;
+    int rc = ctx_reserve(c, 3 * arr, 3 * arr, host && !in_place ? in_bytes : 0);
     if (rc) return rc;
+    if (in_place && !c->small) PSKV_HIP(hipHostMalloc(&c->small, kSmallStage, hipHostMallocCoherent));
     char* d = static_cast<char*>(c->dev);
-    uint64_t* d_targets = reinterpret_cast<uint64_t*>(d);
-    uint64_t* d_lb = reinterpret_cast<uint64_t*>(d + pad256((S + 1) * 8));
-    uint64_t* d_pos = reinterpret_cast<uint64_t*>(d + 2 * pad256((S + 1) * 8));
-    unsigned long long* d_sums = reinterpret_cast<unsigned long long*>(d + 3 * pad256((S + 1) * 8));
+    uint64_t* d_lb = reinterpret_cast<uint64_t*>(d);
+    uint64_t* d_pos = reinterpret_cast<uint64_t*>(d + arr);
+    unsigned long long* d_sums = reinterpret_cast<unsigned long long*>(d + 2 * arr);
     char* h = static_cast<char*>(c->pinned);
     uint64_t* h_targets = reinterpret_cast<uint64_t*>(h);
-    uint64_t* h_pos = reinterpret_cast<uint64_t*>(h + 2 * pad256((S + 1) * 8));
-    unsigned long long* h_sums = reinterpret_cast<unsigned long long*>(h + 3 * pad256((S + 1) * 8));
+    uint64_t* h_pos = reinterpret_cast<uint64_t*>(h + arr);
+    unsigned long long* h_sums = reinterpret_cast<unsigned long long*>(h + 2 * arr);
 
     const uint64_t* d_keys = keys;
     const int32_t* d_lens = lens;
     if (host) {
-      uint64_t* sk = static_cast<uint64_t*>(c->stage);
-      PSKV_HIP(hipMemcpyAsync(sk, keys, n * 8, hipMemcpyHostToDevice, c->stream));
-      d_keys = sk;
-      if (do_sums) {
-        int32_t* sl = reinterpret_cast<int32_t*>(static_cast<char*>(c->stage) + pad256(n * 8));
-        PSKV_HIP(hipMemcpyAsync(sl, lens, n * 4, hipMemcpyHostToDevice, c->stream));
-        d_lens = sl;
+      char* base = static_cast<char*>(in_place ? c->small : c->stage);
+      uint64_t* sk = reinterpret_cast<uint64_t*>(base);
+      int32_t* sl = reinterpret_cast<int32_t*>(base + pad256(n * 8));
+      if (in_place) {
+        std::memcpy(sk, keys, n * 8);
+        if (do_sums) std::memcpy(sl, lens, n * 4);
+      } else {
+        PSKV_HIP(hipMemcpyAsync(sk, keys, n * 8, hipMemcpyHostToDevice, c->stream));
+        if (do_sums) PSKV_HIP(hipMemcpyAsync(sl, lens, n * 4, hipMemcpyHostToDevice, c->stream));
       }
+      d_keys = sk;
+      if (do_sums) d_lens = sl;
     }
     h_targets[0] = range_begin[0];
     for (size_t i = 0; i < S; ++i) h_targets[i + 1] = range_end[i];
-    PSKV_HIP(hipMemcpyAsync(d_targets, h_targets, (S + 1) * 8, hipMemcpyHostToDevice, c->stream));
-    rc = launch_bounds_search(d_keys, n, d_targets, S + 1, d_lb, c->stream);
+    rc = launch_bounds_search(d_keys, n, h_targets, S + 1, d_lb, c->stream);
     if (rc) return rc;
-    k_bounds_chain<<<dim3(1), dim3(64), 0, c->stream>>>(d_lb, S, d_pos);
+    k_bounds_chain<<<dim3(1), dim3(64), 0, c->stream>>>(d_lb, S, d_pos, h_pos, do_sums ? d_sums : nullptr);
     PSKV_HIP(hipGetLastError());
     if (do_sums) {
-      if (S > 65535) return set_error(PSKV_EINVAL, "more than 65535 ranges with lens");
-      PSKV_HIP(hipMemsetAsync(d_sums, 0, S * 8, c->stream));
       uint64_t per = n / S / (kBlock * 8) + 1;
       if (per > 1024) per = 1024;
       k_segment_sums<<<dim3((unsigned)per, (unsigned)S), dim3(kBlock), 0, c->stream>>>(d_lens, d_pos,
                                                                                       d_sums);
       PSKV_HIP(hipGetLastError());
-      PSKV_HIP(hipMemcpyAsync(h_sums, d_sums, S * 8, hipMemcpyDeviceToHost, c->stream));
+      k_export_sums<<<dim3((unsigned)((S + 255) / 256)), dim3(256), 0, c->stream>>>(d_sums, S, h_sums);
+      PSKV_HIP(hipGetLastError());
     }
-    PSKV_HIP(hipMemcpyAsync(h_pos, d_pos, (S + 1) * 8, hipMemcpyDeviceToHost, c->stream));
     PSKV_HIP(hipStreamSynchronize(c->stream));
     for (size_t i = 0; i <= S; ++i) pos[i] = h_pos[i];
     if (do_sums)
