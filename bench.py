@@ -51,6 +51,20 @@ def traffic(kind, units):
     return TRAFFIC.get((kind, int(units)))
 
 
+def host_info():
+    """The CPU the baseline ran on and how the oracle was compiled."""
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for l in f:
+                if l.startswith("model name"):
+                    model = l.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"cpu": model, "logical_cpus": os.cpu_count(), "oracle_flags": "g++ -O3 -std=c++11"}
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -73,21 +87,29 @@ def to_dev(a, dev):
 
 
 def kernel_stats(tables, kernel):
-    n, ms = 0, 0.0
+    """(launches, summed ms, per-launch ms) of one kernel over several tables."""
+    n, ms, samples = 0, 0.0, []
     for t in tables:
         a, b = t.prof_read(kernel)
         n += a
         ms += b
-    return n, ms
+        samples.append(t.prof_samples(kernel))
+    return n, ms, np.concatenate(samples) if samples else np.zeros(0, np.float32)
 
 
-def roofline(alg_bytes_per_launch, launches, total_ms, traffic=None):
+def roofline(alg_bytes_per_launch, launches, total_ms, traffic=None, samples=None):
+    """`achieved` is algorithmic bytes over the AVERAGE launch duration; the median and the
+    minimum over the launches are given beside it."""
     avg_s = total_ms / launches * 1e-3 if launches else float("nan")
     achieved = alg_bytes_per_launch / avg_s / 1e9 if launches else 0.0
-    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-            "launches": launches, "avg_us": round(avg_s * 1e6, 2),
-            "alg_bytes_per_launch": int(alg_bytes_per_launch)}
+    r = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+         "launches": launches, "avg_us": round(avg_s * 1e6, 2),
+         "alg_bytes_per_launch": int(alg_bytes_per_launch)}
+    if samples is not None and len(samples):
+        r["median_us"] = round(float(np.median(samples)) * 1e3, 2)
+        r["min_us"] = round(float(np.min(samples)) * 1e3, 2)
+    return r
 
 
 # ------------------------------------------------------------------------------------
@@ -167,8 +189,8 @@ def run_sparse_lr(args, capi, dev):
     for i in range(args.warmup + args.steps, total_steps):
         step(i)
     drain()
-    push_n, push_ms = kernel_stats(tables, capi.KERNEL_PUSH_SCALAR)
-    pull_n, pull_ms = kernel_stats(tables, capi.KERNEL_PULL_SCALAR)
+    push_n, push_ms, push_s = kernel_stats(tables, capi.KERNEL_PUSH_SCALAR)
+    pull_n, pull_ms, pull_s = kernel_stats(tables, capi.KERNEL_PULL_SCALAR)
     for t in tables:
         t.prof_enable(False)
     # the slicer alone on an idle GPU: two small launches and one read-back of S+1 positions
@@ -186,10 +208,10 @@ def run_sparse_lr(args, capi, dev):
                    "store_keys_after_timed_steps": held},
         # every pushed key is new: 8 key + 4 val in, 8 slot read, 8 key + 4 val written
         "roofline": dict(roofline(32.0 * keys_per_launch, push_n, push_ms,
-                                  traffic("push_scalar", keys_per_launch)),
+                                  traffic("push_scalar", keys_per_launch), push_s),
                          kernel="k_scalar<push> (find-or-insert + add)", bytes_per_key=32),
         "kernels": {"pull_scalar": dict(roofline(24.0 * keys_per_launch, pull_n, pull_ms,
-                                                 traffic("pull_scalar", keys_per_launch)),
+                                                 traffic("pull_scalar", keys_per_launch), pull_s),
                                         bytes_per_key=24),
                     "slicer": {"wall_us_per_call": round(slice_us, 1), "keys": n, "ranges": S}},
     }
@@ -251,25 +273,26 @@ def measure_dense(capi, dev, steps, warmup, nk=64, k=4194304):
         t.push(keys, vals)
         t.pull(keys, out)
     t.sync()
-    acc = t.prof_read(capi.KERNEL_ROWS_ACC)
-    gat = t.prof_read(capi.KERNEL_ROWS_GATHER)
-    t.prof_enable(False)
+    acc = kernel_stats([t], capi.KERNEL_ROWS_ACC)
+    gat = kernel_stats([t], capi.KERNEL_ROWS_GATHER)
     # closed form: every float holds (1 + warmup + 2*steps) * v, accumulated one add at a time
     idx = torch.randint(0, nk * k, (4096,), device=dev)
     ref = torch.zeros(4096, device=dev)
     for _ in range(1 + warmup + 2 * steps):
         ref = ref + vals[idx]
     assert torch.equal(out[idx], ref), "dense sums differ from sequential float adds"
-    # one plain copy of the same 1 GiB: the known-size launch that memory-traffic counters are
-    # scaled by, and the copy ceiling next to the accumulate kernel
-    t.copy_probe(out, vals)
-    t.sync()
+    # plain copies of the same 1 GiB: the known-size launch that memory-traffic counters are
+    # scaled by, and the copy ceiling of this GPU next to the accumulate kernel
+    for _ in range(3):
+        t.copy_probe(out, vals)
+    cp = kernel_stats([t], capi.KERNEL_COPY)
+    t.prof_enable(False)
     t.close()
-    return dt, acc, gat, nk, k
+    return dt, acc, gat, cp, nk, k
 
 
 def run_dense(args, capi, dev):
-    dt, acc, gat, nk, k = measure_dense(capi, dev, args.steps, args.warmup)
+    dt, acc, gat, cp, nk, k = measure_dense(capi, dev, args.steps, args.warmup)
     floats = nk * k
     res = {
         "value": 20.0 * floats * args.steps / dt / 1e9, "unit": "GB/s",
@@ -277,11 +300,13 @@ def run_dense(args, capi, dev):
         "config": {"workload": "dense: 64 keys x 4,194,304 f32 (1 GiB), push-accumulate then full pull",
                    "keys_per_step": nk, "value_len": k},
         # 4 B in + 4 B row read + 4 B row write per float
-        "roofline": dict(roofline(12.0 * floats, acc[0], acc[1], traffic("rows_acc_fixed", floats)),
+        "roofline": dict(roofline(12.0 * floats, acc[0], acc[1], traffic("rows_acc_fixed", floats), acc[2]),
                          kernel="k_rows<acc,fixed> (row += in)", bytes_per_float=12),
         "kernels": {"rows_gather": dict(roofline(8.0 * floats, gat[0], gat[1],
-                                                 traffic("rows_gather_fixed", floats)),
-                                        bytes_per_float=8)},
+                                                 traffic("rows_gather_fixed", floats), gat[2]),
+                                        bytes_per_float=8),
+                    "copy_ceiling": dict(roofline(8.0 * floats, cp[0], cp[1], 8.0 * floats, cp[2]),
+                                         kernel="k_copy (plain copy of the same 1 GiB)")},
     }
     return res
 
@@ -381,10 +406,10 @@ def run_varlen(args, capi, dev):
                    "ranges": S},
         "gbps": (20.0 * nvals + 56.0 * n) * args.steps / dt / 1e9,
         "roofline": dict(roofline(12.0 * floats_per_launch, acc[0], acc[1],
-                                  traffic("rows_acc_varlen", floats_per_launch)),
+                                  traffic("rows_acc_varlen", floats_per_launch), acc[2]),
                          kernel="k_rows<acc,varlen> (row += in)", bytes_per_float=12),
         "kernels": {"rows_gather": dict(roofline(8.0 * floats_per_launch, gat[0], gat[1],
-                                                 traffic("rows_gather_varlen", floats_per_launch)),
+                                                 traffic("rows_gather_varlen", floats_per_launch), gat[2]),
                                         bytes_per_float=8)},
     }
     return res, (keys, lens, nvals, n, S)
@@ -441,12 +466,14 @@ def main():
     if args.workload == "sparse_lr" and not args.no_extra:
         # the dense-chunk kernels carry the bandwidth target of this path; measure them
         # beside the default workload (10 push+pull steps of 1 GiB, well under a second)
-        dt, acc, gat, nk, k = measure_dense(capi, dev, 10, 2)
+        dt, acc, gat, cp, nk, k = measure_dense(capi, dev, 10, 2)
         extra["dense_chunk"] = {
-            "rows_acc": dict(roofline(12.0 * nk * k, acc[0], acc[1], traffic("rows_acc_fixed", nk * k)),
+            "rows_acc": dict(roofline(12.0 * nk * k, acc[0], acc[1], traffic("rows_acc_fixed", nk * k), acc[2]),
                              bytes_per_float=12),
             "rows_gather": dict(roofline(8.0 * nk * k, gat[0], gat[1],
-                                         traffic("rows_gather_fixed", nk * k)), bytes_per_float=8),
+                                         traffic("rows_gather_fixed", nk * k), gat[2]), bytes_per_float=8),
+            "copy_ceiling": dict(roofline(8.0 * nk * k, cp[0], cp[1], 8.0 * nk * k, cp[2]),
+                                 kernel="k_copy (plain copy of 1 GiB)"),
         }
 
     cpu = None
@@ -459,6 +486,7 @@ def main():
             cpu = cpu_dense(orc)
         else:
             cpu = cpu_varlen(orc, *varlen_inputs)
+        cpu["host"] = host_info()
 
     line = {
         "metric": "push+pull keys/sec and achieved GB/s (% of HBM peak) on 1 MI355X",

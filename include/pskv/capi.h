@@ -62,7 +62,8 @@ extern "C" {
 #define PSKV_KERNEL_ROWS_GATHER 3 /* pull gather of rows */
 #define PSKV_KERNEL_LOOKUP 4      /* key -> row lookup / insert of the row modes */
 #define PSKV_KERNEL_REHASH 5
-#define PSKV_KERNEL_COUNT 6
+#define PSKV_KERNEL_COPY 6        /* the plain copy of pskv_copy_probe */
+#define PSKV_KERNEL_COUNT 7
 
 typedef struct pskv_table pskv_table;
 
@@ -158,6 +159,10 @@ int pskv_assemble_pull(int device, const uint64_t* req_keys, size_t n, size_t R,
 int pskv_prof_enable(pskv_table* t, int on);
 int pskv_prof_reset(pskv_table* t);
 int pskv_prof_read(pskv_table* t, int kernel, uint64_t* launches, double* total_ms);
+/* The durations of the individual launches (in launch order) since the last
+ * pskv_prof_reset, for medians and minima: writes min(*n, cap) values to out_ms and
+ * the number recorded to *n. At most 65536 launches per kernel are kept. */
+int pskv_prof_samples(pskv_table* t, int kernel, float* out_ms, size_t cap, size_t* n);
 
 /* Plain device-to-device copy kernel of `bytes` bytes (multiple of 16) on the
  * table's stream; used to calibrate memory-traffic counters and as the measured

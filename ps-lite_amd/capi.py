@@ -26,7 +26,7 @@ MODE_FIXED = 1
 MODE_VARLEN = 2
 MAX_VARLEN_ROW = (1 << 28) - 1
 KERNEL_PUSH_SCALAR, KERNEL_PULL_SCALAR, KERNEL_ROWS_ACC, KERNEL_ROWS_GATHER, KERNEL_LOOKUP, \
-    KERNEL_REHASH = range(6)
+    KERNEL_REHASH, KERNEL_COPY = range(7)
 
 ERROR_NAMES = {
     EUNCOVERED_KEY: "PSKV_EUNCOVERED_KEY", ESIZE_MISMATCH: "PSKV_ESIZE_MISMATCH",
@@ -38,7 +38,7 @@ ERROR_NAMES = {
 SYMBOLS = [
     "pskv_table_create", "pskv_table_destroy", "pskv_push", "pskv_pull", "pskv_pushpull",
     "pskv_sync", "pskv_size", "pskv_dump", "pskv_slice", "pskv_server_ranges",
-    "pskv_assemble_pull", "pskv_prof_enable", "pskv_prof_reset", "pskv_prof_read",
+    "pskv_assemble_pull", "pskv_prof_enable", "pskv_prof_reset", "pskv_prof_read", "pskv_prof_samples",
     "pskv_copy_probe", "pskv_host_alloc", "pskv_host_free", "pskv_host_trim", "pskv_last_error",
     "pskv_version",
 ]
@@ -92,6 +92,7 @@ def load():
     lib.pskv_prof_enable.argtypes = [vp, i32]
     lib.pskv_prof_reset.argtypes = [vp]
     lib.pskv_prof_read.argtypes = [vp, i32, ctypes.POINTER(u64), ctypes.POINTER(ctypes.c_double)]
+    lib.pskv_prof_samples.argtypes = [vp, i32, vp, sz, ctypes.POINTER(sz)]
     lib.pskv_copy_probe.argtypes = [vp, vp, vp, sz]
     lib.pskv_host_alloc.argtypes = [sz]
     lib.pskv_host_alloc.restype = vp
@@ -222,6 +223,15 @@ class Table:
         n, ms = ctypes.c_uint64(0), ctypes.c_double(0.0)
         _check(self._lib.pskv_prof_read(self._h, kernel, ctypes.byref(n), ctypes.byref(ms)))
         return n.value, ms.value
+
+    def prof_samples(self, kernel):
+        """Durations (ms) of the individual launches since the last prof_reset."""
+        n = ctypes.c_size_t(0)
+        _check(self._lib.pskv_prof_samples(self._h, kernel, None, 0, ctypes.byref(n)))
+        out = np.zeros(n.value, np.float32)
+        if n.value:
+            _check(self._lib.pskv_prof_samples(self._h, kernel, out.ctypes.data, out.size, ctypes.byref(n)))
+        return out
 
     def copy_probe(self, dst, src):
         assert dst.is_cuda and src.is_cuda

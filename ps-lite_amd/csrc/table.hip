@@ -35,6 +35,7 @@ namespace {
 constexpr uint64_t kDefaultCapacity = 1u << 20;
 constexpr uint64_t kMinSlots = 1024;
 constexpr unsigned kMaxGrid = 1u << 20;
+constexpr size_t kMaxProfSamples = 65536;
 // Host-resident requests up to this size (per direction) skip the copy commands: the kernels
 // read the request from, and write the response to, pinned host memory mapped into the GPU.
 constexpr size_t kSmallBytes = 1024u << 10;
@@ -156,6 +157,7 @@ struct pskv_table {
   std::vector<EventPair> free_events;
   uint64_t launches[PSKV_KERNEL_COUNT] = {0};
   double total_ms[PSKV_KERNEL_COUNT] = {0};
+  std::vector<float> samples[PSKV_KERNEL_COUNT];  // per-launch durations, bounded
 };
 
 namespace {
@@ -199,6 +201,7 @@ int prof_collect(pskv_table* t) {
       if (hipEventElapsedTime(&ms, ev.a, ev.b) == hipSuccess) {
         t->total_ms[k] += ms;
         t->launches[k] += 1;
+        if (t->samples[k].size() < kMaxProfSamples) t->samples[k].push_back(ms);
       }
       t->free_events.push_back(ev);
     }
@@ -1083,6 +1086,7 @@ int pskv_prof_reset(pskv_table* t) {
   for (int k = 0; k < PSKV_KERNEL_COUNT; ++k) {
     t->launches[k] = 0;
     t->total_ms[k] = 0.0;
+    t->samples[k].clear();
   }
   return rc;
 }
@@ -1097,6 +1101,18 @@ int pskv_prof_read(pskv_table* t, int kernel, uint64_t* launches, double* total_
   return rc;
 }
 
+int pskv_prof_samples(pskv_table* t, int kernel, float* out_ms, size_t cap, size_t* n) {
+  if (!t || !n) return set_error(PSKV_EINVAL, "null argument");
+  if (kernel < 0 || kernel >= PSKV_KERNEL_COUNT) return set_error(PSKV_EINVAL, "bad kernel id");
+  DeviceGuard guard(t->device);
+  int rc = prof_collect(t);
+  const std::vector<float>& v = t->samples[kernel];
+  *n = v.size();
+  if (out_ms)
+    for (size_t i = 0; i < v.size() && i < cap; ++i) out_ms[i] = v[i];
+  return rc;
+}
+
 int pskv_copy_probe(pskv_table* t, void* dst, const void* src, size_t bytes) {
   if (!t) return set_error(PSKV_EINVAL, "null table");
   if ((bytes & 15) || (reinterpret_cast<uintptr_t>(dst) & 15) || (reinterpret_cast<uintptr_t>(src) & 15))
@@ -1105,8 +1121,8 @@ int pskv_copy_probe(pskv_table* t, void* dst, const void* src, size_t bytes) {
   DeviceGuard guard(t->device);
   const uint64_t n16 = bytes / 16;
   if ((n16 + kBlock - 1) / kBlock > 0x7fffffffull) return set_error(PSKV_EINVAL, "copy too large");
-  k_copy<<<dim3((unsigned)((n16 + kBlock - 1) / kBlock)), dim3(kBlock), 0, t->stream>>>(
-      static_cast<f32x4*>(dst), static_cast<const f32x4*>(src), n16);
+  launch(t, PSKV_KERNEL_COPY, k_copy, dim3((unsigned)((n16 + kBlock - 1) / kBlock)), dim3(kBlock),
+         static_cast<f32x4*>(dst), static_cast<const f32x4*>(src), n16);
   PSKV_HIP(hipGetLastError());
   return PSKV_OK;
 }
