@@ -53,6 +53,7 @@ struct __align__(16) Slot {
 // of workgroups.
 constexpr int kCountShards = 32;
 constexpr int kShardStride = 16;  // in 8-byte words: one shard per 128-byte line
+constexpr int kTicketShards = 32;
 
 struct DevState {
   unsigned long long arena_top;        // FIXED: rows handed out; VARLEN: 16-byte units handed out
@@ -62,10 +63,9 @@ struct DevState {
   unsigned int error;                  // sticky error bits of finished requests
   unsigned int req_error;              // error bits of the request in flight
   unsigned int misaligned;             // OR of (len & 3) over the lens of the current request
-  unsigned int scan_bits;              // the same, while the lens scan is still collecting it
-  unsigned int scan_bad;               // a length out of range seen by the lens scan in flight
-  unsigned int scan_ticket;            // workgroups of the lens scan that have finished
-  unsigned int pad0;
+  unsigned int req_flags;              // kReq* facts the workgroups of the kernel in flight have found
+  unsigned int ticket_top;             // second level of the last-workgroup ticket (ticket_last)
+  unsigned int pad0[2];
   // "Same keys as the request that last filled the workspace" fast path of the row modes.
   // Every row-mode request has a number (epoch). cache_epoch is the request whose keys, lens,
   // row references, offsets and tile table the workspace and the key cache hold; bad_epoch ==
@@ -74,10 +74,25 @@ struct DevState {
   unsigned long long cache_epoch;
   unsigned long long bad_epoch;
   unsigned long long same_epoch;
-  unsigned int same_diff;    // a workgroup of the compare kernel found a difference
-  unsigned int same_ticket;  // workgroups of the compare kernel that have finished
   // keys held (slot array plus the side slot) = sum of the shards
   unsigned long long count_shard[kCountShards * kShardStride];
+  // first level of the last-workgroup ticket: one counter per 128-byte line
+  unsigned int ticket_sub[kTicketShards * 32];
+};
+
+// Facts about the request that workgroups report into DevState::req_flags.
+constexpr unsigned kReqMisaligned = 3u;  // OR of (len & 3)
+constexpr unsigned kReqBadLen = 4u;      // a length negative or above the maximum
+constexpr unsigned kReqDiffer = 8u;      // a key or length differs from the cached request
+
+// Counters of the table as of the start of request `seq`, written by the device into pinned
+// host memory so that the host can bound the counters without waiting for the stream.
+// seq_begin == seq_end marks a consistent record.
+struct Snapshot {
+  volatile uint64_t seq_begin;
+  volatile uint64_t count;
+  volatile uint64_t arena_top;
+  volatile uint64_t seq_end;
 };
 
 // What a row-mode kernel needs to know about the request it belongs to.
@@ -100,6 +115,38 @@ __device__ __forceinline__ bool cache_same(const DevState* st, const ReqTag& tag
 __device__ __forceinline__ void raise_error(DevState* st, unsigned bit, unsigned long long epoch) {
   atomicOr(&st->req_error, bit);
   st->bad_epoch = epoch;
+}
+
+// Finds the workgroup of a grid that finishes last. Thread 0 of EVERY workgroup calls it once,
+// after the writes the last workgroup is to see; it returns true in exactly one of them,
+// and that thread then sees those writes.
+// What the callers hand to the last workgroup must have been written with device-scope
+// atomics (atomicOr, publish_u64 below): those are performed at the memory side, past the
+// per-XCD L2, so all a workgroup has to do before its ticket is wait for its own
+// outstanding operations. A full release fence would write the L2 back instead, once per
+// workgroup, which for a grid of 2,000 workgroups costs tens of microseconds.
+// Two levels of counters, the first spread over kTicketShards cache lines, because atomics
+// on one address are served one at a time (about 15 ns each).
+// The counters are left at zero; kernels that use it must not overlap on one table.
+__device__ __forceinline__ bool ticket_last(DevState* st) {
+  const unsigned shards = gridDim.x < (unsigned)kTicketShards ? gridDim.x : (unsigned)kTicketShards;
+  const unsigned sub = blockIdx.x % shards;
+  const unsigned members = (gridDim.x - sub + shards - 1) / shards;  // workgroups b with b % shards == sub
+  unsigned* c = &st->ticket_sub[sub * 32];
+  // this thread's atomics and atomic stores are complete before its ticket is taken
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0);
+  if (atomicAdd(c, 1u) != members - 1) return false;
+  *c = 0;
+  if (atomicAdd(&st->ticket_top, 1u) != shards - 1) return false;
+  st->ticket_top = 0;
+  __threadfence();  // acquire, once per grid: nothing stale is left in this XCD's L2
+  return true;
+}
+
+// A 64-bit value for the workgroup that ticket_last elects: stored past the L2.
+__device__ __forceinline__ void publish_u64(unsigned long long* p, unsigned long long v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Adds the workgroup's total of `x` to one shard of the key counter. Every thread of
@@ -168,6 +215,23 @@ __device__ __forceinline__ unsigned long long wave_incl_scan_u64(unsigned long l
     if (lane >= (unsigned)d) x += y;
   }
   return x;
+}
+
+// Writes the table's counters to `out` (pinned host memory). Called by all 64 lanes of one
+// wavefront, at a point of the stream where no kernel is changing the counters.
+__device__ __forceinline__ void publish_snapshot(const DevState* st, Snapshot* out, uint64_t seq) {
+  static_assert(kCountShards <= 64, "one lane per shard");
+  const unsigned lane = threadIdx.x & 63;
+  unsigned long long c = lane < kCountShards ? st->count_shard[lane * kShardStride] : 0ull;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
+  if (lane != 0) return;
+  out->seq_begin = seq;
+  __threadfence_system();
+  out->count = c;
+  out->arena_top = st->arena_top;
+  __threadfence_system();
+  out->seq_end = seq;
 }
 
 // Finds `key` or claims an empty slot for it. Returns the address of the slot's

@@ -50,15 +50,6 @@ struct EventPair {
   hipEvent_t a, b;
 };
 
-// Counters of the table as of the start of request `seq`, written by the device into
-// pinned host memory. seq_begin == seq_end marks a consistent record.
-struct Snapshot {
-  volatile uint64_t seq_begin;
-  volatile uint64_t count;
-  volatile uint64_t arena_top;
-  volatile uint64_t seq_end;
-};
-
 // What the host reads back of the device state, written by the device into pinned host memory
 // (a one-wavefront kernel is quicker than a copy command for these few words).
 struct StateView {
@@ -83,19 +74,10 @@ __global__ void k_read_state(const DevState* st, StateView* out) {
   out->special_present = st->special_present;
 }
 
-// One wavefront, launched in front of a request's kernels when the table is close to a limit.
+// One wavefront, launched in front of a request's kernels when the table is close to a limit
+// and no kernel of the request can carry the record.
 __global__ void k_publish(const DevState* st, Snapshot* out, uint64_t seq) {
-  static_assert(kCountShards <= 64, "one lane per shard");
-  unsigned long long c = threadIdx.x < kCountShards ? st->count_shard[threadIdx.x * kShardStride] : 0ull;
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
-  if (threadIdx.x != 0) return;
-  out->seq_begin = seq;
-  __threadfence_system();
-  out->count = c;
-  out->arena_top = st->arena_top;
-  __threadfence_system();
-  out->seq_end = seq;
+  publish_snapshot(st, out, seq);
 }
 
 }  // namespace
@@ -338,7 +320,19 @@ int grow_arena(pskv_table* t, uint64_t floats_needed, uint64_t live_floats) {
 // Grows the slot array / the arena first if the bounds say they could overflow. The fast
 // path touches no device state; the next best reads the snapshot the device published;
 // only then does it wait for the stream and read the counters.
-int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit) {
+//
+// Close to a limit the device publishes its counters in front of the request, so that a later
+// request can move the base forward without waiting for the stream. With `carry` the caller
+// promises to hand the record to a kernel of the request that runs before any of its
+// kernels changes a counter (carry->snap is set when a record is wanted); without it a
+// one-wavefront kernel is launched here.
+struct PublishReq {
+  Snapshot* snap = nullptr;
+  uint64_t seq = 0;
+};
+
+int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
+            PublishReq* carry = nullptr) {
   if (t->no_growth) return PSKV_OK;
   const double limit = (double)t->max_load * (double)t->cap;
   auto slots_short = [&]() { return (double)(t->base_count + t->pend_keys + n) > limit; };
@@ -365,15 +359,18 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit)
   t->log_units[q % pskv_table::kLog] = units;
   t->pend_keys += n;
   t->pend_units += units;
-  // Close to a limit: let the device publish its counters in front of this request, so that
-  // a later request can move the base forward without waiting for the stream.
   const double limit_now = (double)t->max_load * (double)t->cap;
   const bool tight_slots = (double)(t->base_count + t->pend_keys + 2 * n) > limit_now;
   const bool tight_arena =
       units && (t->base_top + t->pend_units + 2 * units) * floats_per_unit > t->arena_cap;
   if (tight_slots || tight_arena || t->seq - t->base_seq >= (uint64_t)pskv_table::kLog / 2) {
-    k_publish<<<dim3(1), dim3(64), 0, t->stream>>>(t->st, t->snap, q);
-    PSKV_HIP(hipGetLastError());
+    if (carry) {
+      carry->snap = t->snap;
+      carry->seq = q;
+    } else {
+      k_publish<<<dim3(1), dim3(64), 0, t->stream>>>(t->st, t->snap, q);
+      PSKV_HIP(hipGetLastError());
+    }
   }
   return PSKV_OK;
 }
@@ -440,17 +437,32 @@ int launch_rows(pskv_table* t, int op, const RowsParams& p) {
   return PSKV_OK;
 }
 
+// Numbers a row-mode request and says whether the key cache has the right shape for it.
+ReqTag next_tag(pskv_table* t, const Request& r) {
+  ReqTag tag;
+  tag.epoch = ++t->epoch;
+  tag.pad = 0;
+  tag.try_cache = (t->cache_valid && t->cache_n == r.n) ? 1u : 0u;
+  return tag;
+}
+
 // Starts a row-mode request: numbers it and, when the key cache has the right shape, lets the
 // device compare the request with the cached one. Call after every buffer the cache lives in
-// has been grown for this request.
-int begin_row_request(pskv_table* t, const Request& r, bool with_lens, ReqTag* tag) {
-  tag->epoch = ++t->epoch;
-  tag->pad = 0;
-  tag->try_cache = (t->cache_valid && t->cache_n == r.n) ? 1u : 0u;
+// has been grown for this request. A counter record the request has to publish (`pub`) rides
+// on the compare kernel, or gets a launch of its own when there is none.
+int begin_row_request(pskv_table* t, const Request& r, bool with_lens, ReqTag* tag,
+                      const PublishReq* pub) {
+  *tag = next_tag(t, r);
+  Snapshot* snap = pub ? pub->snap : nullptr;
+  const uint64_t seq = pub ? pub->seq : 0;
   if (tag->try_cache) {
-    k_same_keys<<<dim3(grid_for(r.n, kBlock * 4, 4096)), dim3(kBlock), 0, t->stream>>>(
+    k_same_keys<<<dim3((unsigned)((r.n + kBlock * 4 - 1) / (kBlock * 4))), dim3(kBlock), 0, t->stream>>>(
         r.keys, with_lens ? r.lens : nullptr, static_cast<const uint64_t*>(t->cache_keys.ptr),
-        with_lens ? static_cast<const int32_t*>(t->cache_lens.ptr) : nullptr, r.n, t->st, *tag);
+        with_lens ? static_cast<const int32_t*>(t->cache_lens.ptr) : nullptr, r.n, t->st, *tag, snap,
+        seq);
+    PSKV_HIP(hipGetLastError());
+  } else if (snap) {
+    k_publish<<<dim3(1), dim3(64), 0, t->stream>>>(t->st, snap, seq);
     PSKV_HIP(hipGetLastError());
   }
   return PSKV_OK;
@@ -460,7 +472,8 @@ int run_fixed(pskv_table* t, Request& r) {
   const uint64_t k = t->row_len;
   r.out_nvals = r.pull ? r.n * k : 0;
   if (r.n == 0) return PSKV_OK;
-  int rc = reserve(t, r.n, r.n, k);
+  PublishReq pub;
+  int rc = reserve(t, r.n, r.n, k, &pub);
   if (rc) return rc;
   rc = grow(t, &t->ws, Carver::need(r.n, sizeof(uint64_t)));
   if (rc) return rc;
@@ -470,7 +483,7 @@ int run_fixed(pskv_table* t, Request& r) {
   uint64_t* ref = c.take<uint64_t>(r.n);
   uint64_t* cache_keys = static_cast<uint64_t*>(t->cache_keys.ptr);
   ReqTag tag;
-  rc = begin_row_request(t, r, false, &tag);
+  rc = begin_row_request(t, r, false, &tag, &pub);
   if (rc) return rc;
   if (r.n >= kLookupLargeKeys) {
     launch(t, PSKV_KERNEL_LOOKUP, k_lookup_fixed<kLookupItemsLarge>,
@@ -518,22 +531,38 @@ int grow_tile_tables(pskv_table* t, uint64_t floats, uint64_t* ntiles_cap) {
   return grow(t, &t->tiles_aff, (*ntiles_cap + 1) * sizeof(uint64_t));
 }
 
-// Fills the tile table of a pull whose offsets come from the stored lens (the row kernel
-// fills the other one).
-int make_tile_tables(pskv_table* t, const uint64_t* off, uint64_t n, uint64_t floats,
-                     RowsParams* p, const ReqTag& tag) {
+// The kernels of a var-len request that work key by key: one workgroup per kBlock*items keys,
+// `items` per thread, the same split in every kernel of the request (the scan's
+// per-workgroup totals are indexed by it).
+template <typename K1, typename K4, typename... Args>
+void launch_keys(pskv_table* t, int prof_kernel, uint64_t n, K1 k1, K4 k4, Args... args) {
+  const dim3 grid((unsigned)scan_num_parts(n)), block(kBlock);
+  if (scan_items(n) == kScanItemsLarge) {
+    launch(t, prof_kernel, k4, grid, block, args...);
+  } else {
+    launch(t, prof_kernel, k1, grid, block, args...);
+  }
+}
+
+// Pass 2 of a pull's scan: the request-side offsets of the response and the tile table for
+// `floats` floats of room (the row kernel fills the other table).
+int make_tile_tables(pskv_table* t, const int32_t* lens_out, const unsigned long long* part,
+                     uint64_t* off, uint64_t n, uint64_t floats, RowsParams* p, const ReqTag& tag) {
   uint64_t ntiles_cap = 0;
   int rc = grow_tile_tables(t, floats, &ntiles_cap);
   if (rc) return rc;
   uint32_t* tk = static_cast<uint32_t*>(t->tiles.ptr);
-  k_tile_keys<<<dim3(grid_for(n, kBlock, kMaxGrid)), dim3(kBlock), 0, t->stream>>>(
-      off, n, tk, ntiles_cap, (uint64_t)kTileVar, (const DevState*)t->st, tag);
+  launch_keys(t, -1, n, k_var_offsets<1>, k_var_offsets<kScanItemsLarge>, lens_out, n, part, off, tk,
+              ntiles_cap, (uint64_t)kTileVar, (const DevState*)t->st, tag);
   PSKV_HIP(hipGetLastError());
   p->tile_key = tk;
   p->tile_aff = static_cast<uint64_t*>(t->tiles_aff.ptr);
   return PSKV_OK;
 }
 
+// Launches per var-len request: a push takes three (compare + scan pass 1 + counter record;
+// scan pass 2 + find-or-create; rows), a pull four (compare; stored lengths + scan pass 1;
+// scan pass 2 + tile table; rows).
 int run_varlen(pskv_table* t, Request& r) {
   r.out_nvals = 0;
   if (r.n == 0) return PSKV_OK;
@@ -562,7 +591,6 @@ int run_varlen(pskv_table* t, Request& r) {
   int32_t* tmp_lens = c.take<int32_t>(r.n);
   uint64_t* cache_keys = static_cast<uint64_t*>(t->cache_keys.ptr);
   int32_t* cache_lens = static_cast<int32_t*>(t->cache_lens.ptr);
-  const dim3 kgrid(grid_for(r.n, kBlock, kMaxGrid)), block(kBlock);
 
   RowsParams p{};
   p.ref = ref;
@@ -571,25 +599,22 @@ int run_varlen(pskv_table* t, Request& r) {
   p.n = r.n;
 
   if (r.push) {
-    rc = reserve(t, r.n, r.nvals / 4 + r.n, 4);
+    PublishReq pub;
+    rc = reserve(t, r.n, r.nvals / 4 + r.n, 4, &pub);
     if (rc) return rc;
     if (t->cache_nvals != r.nvals) t->cache_valid = false;  // same lens would mean the same total
-    ReqTag tag;
-    rc = begin_row_request(t, r, true, &tag);
-    if (rc) return rc;
-    // the scan also fills the tile table of the request side (tile sizes are those of nvals;
-    // a request whose lens do not add up to nvals is refused by the lookup kernel)
+    const ReqTag tag = next_tag(t, r);
+    launch_keys(t, -1, r.n, k_var_push_begin<1>, k_var_push_begin<kScanItemsLarge>, r.keys, r.lens, r.n,
+                (const uint64_t*)cache_keys, (const int32_t*)cache_lens, part, t->st,
+                (unsigned)PSKV_MAX_VARLEN_ROW, tag, pub.snap, pub.seq);
+    PSKV_HIP(hipGetLastError());
+    // pass 2 also fills the tile table of the request side (tile sizes are those of nvals; a
+    // request whose lens do not add up to nvals is refused before it gets there)
     uint32_t* push_tile_key = static_cast<uint32_t*>(t->tiles.ptr);
-    PSKV_HIP(launch_lens_scan(r.lens, r.n, off, part, &t->st->scan_ticket, t->st, PSKV_MAX_VARLEN_ROW,
-                              r.nvals ? push_tile_key : nullptr, tiles_cap, kTileVar, tag, t->stream));
-    if (r.n >= kLookupLargeKeys) {
-      launch(t, PSKV_KERNEL_LOOKUP, k_lookup_var_push<kLookupItemsLarge>,
-             dim3(grid_for(r.n, kBlock * kLookupItemsLarge, kMaxGrid)), block, t->slots, t->cap - 1,
-             t->st, r.keys, r.lens, r.n, r.nvals, ref, cache_keys, cache_lens, tag);
-    } else {
-      launch(t, PSKV_KERNEL_LOOKUP, k_lookup_var_push<1>, kgrid, block, t->slots, t->cap - 1, t->st,
-             r.keys, r.lens, r.n, r.nvals, ref, cache_keys, cache_lens, tag);
-    }
+    launch_keys(t, PSKV_KERNEL_LOOKUP, r.n, k_var_push_lookup<1>, k_var_push_lookup<kScanItemsLarge>,
+                t->slots, t->cap - 1, t->st, r.keys, r.lens, r.n, r.nvals,
+                (const unsigned long long*)part, off, r.nvals ? push_tile_key : (uint32_t*)nullptr,
+                tiles_cap, (uint64_t)kTileVar, ref, cache_keys, cache_lens, tag);
     PSKV_HIP(hipGetLastError());
     t->cache_valid = true;  // whichever way the device decided, the cache now is this request
     t->cache_n = r.n;
@@ -619,21 +644,20 @@ int run_varlen(pskv_table* t, Request& r) {
     // A pull with the keys of the cached push finds every key present with the cached length
     // and reuses its references; any other pull recomputes them and so ends the cache.
     ReqTag tag;
-    rc = begin_row_request(t, r, false, &tag);
+    rc = begin_row_request(t, r, false, &tag, nullptr);
     if (rc) return rc;
     if (!tag.try_cache) t->cache_valid = false;
-    launch(t, PSKV_KERNEL_LOOKUP, k_lookup_var_pull, kgrid, block, (const Slot*)t->slots, t->cap - 1,
-           t->st, r.keys, r.n, ref, lens_out, (const int32_t*)cache_lens, tag);
+    launch_keys(t, PSKV_KERNEL_LOOKUP, r.n, k_var_pull_lookup<1>, k_var_pull_lookup<kScanItemsLarge>,
+                (const Slot*)t->slots, t->cap - 1, t->st, r.keys, r.n, ref, lens_out,
+                (const int32_t*)cache_lens, part, tag);
     PSKV_HIP(hipGetLastError());
-    PSKV_HIP(launch_lens_scan(lens_out, r.n, off, part, &t->st->scan_ticket, t->st,
-                              PSKV_MAX_VARLEN_ROW, nullptr, 0, kTileVar, tag, t->stream));
     p.tag = tag;
     if (async_pull) {
       // No host round trip: the grid covers the caller's buffer, the kernels take the real
       // size from the scan, and a response that does not fit is reported by the next sync.
       if (r.out_cap) {
         if (!r.out) return set_error(PSKV_EINVAL, "null out");
-        rc = make_tile_tables(t, off, r.n, r.out_cap, &p, tag);
+        rc = make_tile_tables(t, lens_out, part, off, r.n, r.out_cap, &p, tag);
         if (rc) return rc;
         p.req = r.out;
         p.arena = t->arena;
@@ -665,7 +689,7 @@ int run_varlen(pskv_table* t, Request& r) {
         }
       }
       if (!r.out) return set_error(PSKV_EINVAL, "null out");
-      rc = make_tile_tables(t, off, r.n, total, &p, tag);
+      rc = make_tile_tables(t, lens_out, part, off, r.n, total, &p, tag);
       if (rc) return rc;
       p.req = r.out;
       p.arena = t->arena;

@@ -8,6 +8,7 @@
 #ifndef PSKV_TABLE_KERNELS_H_
 #define PSKV_TABLE_KERNELS_H_
 #include "device_common.h"
+#include "scan.h"
 
 namespace pskv {
 
@@ -49,40 +50,57 @@ __global__ __launch_bounds__(kBlock) void k_scalar(Slot* __restrict__ slots, uin
 // Row modes, step 1: key -> row reference.
 // ---------------------------------------------------------------------------------
 
-// Compares a request with the cached one (keys, and lens when given) and reaches the decision
-// for the whole request: the workgroup that finishes last (ticket counter) sees whether any
-// workgroup found a difference and whether the cache is usable at all, and writes same_epoch.
-// If the decision is "different", the request is going to refill the cache, so it becomes the
-// cached request right here. Epochs start at 1.
-__global__ __launch_bounds__(kBlock) void k_same_keys(const uint64_t* __restrict__ keys,
-                                                     const int32_t* __restrict__ lens,
-                                                     const uint64_t* __restrict__ cache_keys,
-                                                     const int32_t* __restrict__ cache_lens,
-                                                     uint64_t n, DevState* st, ReqTag tag) {
-  __shared__ unsigned s_ticket;
-  bool differ = false;
-  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
-    differ |= keys[i] != cache_keys[i];
-    if (lens) differ |= lens[i] != cache_lens[i];
-  }
-  const int any = __syncthreads_or(differ ? 1 : 0);
-  if (threadIdx.x == 0) {
-    if (any) atomicOr(&st->same_diff, 1u);
-    __threadfence();
-    s_ticket = atomicAdd(&st->same_ticket, 1u);
-  }
-  __syncthreads();
-  if (s_ticket != gridDim.x - 1 || threadIdx.x != 0) return;
-  __threadfence();
-  st->same_ticket = 0;
-  const bool different = atomicExch(&st->same_diff, 0u) != 0u;
-  const bool usable = st->cache_epoch != 0ull && st->bad_epoch != st->cache_epoch;
+// The decision about a request that may repeat the cached one, taken by one thread after
+// every workgroup has compared its share (`different`: any of them found a difference). If
+// the decision is "different" (or the cache was not usable, or not even tried), the request
+// is going to refill the cache, so it becomes the cached request right here. Epochs start
+// at 1.
+__device__ __forceinline__ void decide_same(DevState* st, const ReqTag& tag, bool different) {
+  const bool usable =
+      tag.try_cache && st->cache_epoch != 0ull && st->bad_epoch != st->cache_epoch;
   if (!different && usable) {
     st->same_epoch = tag.epoch;
   } else {
     st->cache_epoch = tag.epoch;
   }
+}
+
+// Compares a request with the cached one (keys, and lens when given) and reaches the decision
+// for the whole request: the workgroup that finishes last sees whether any workgroup found a
+// difference and writes same_epoch. With `snap` it also publishes the table's counters,
+// which no kernel is changing at this point of the stream.
+__global__ __launch_bounds__(kBlock) void k_same_keys(const uint64_t* __restrict__ keys,
+                                                     const int32_t* __restrict__ lens,
+                                                     const uint64_t* __restrict__ cache_keys,
+                                                     const int32_t* __restrict__ cache_lens,
+                                                     uint64_t n, DevState* st, ReqTag tag,
+                                                     Snapshot* snap, uint64_t snap_seq) {
+  __shared__ unsigned s_last;
+  constexpr int kItems = 4;
+  const uint64_t base = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * kItems;
+  // all loads first, then the compares
+  uint64_t a[kItems], b[kItems];
+  int32_t la[kItems], lb[kItems];
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) {
+    const bool in = base + j < n;
+    a[j] = in ? keys[base + j] : 0;
+    b[j] = in ? cache_keys[base + j] : 0;
+    la[j] = in && lens ? lens[base + j] : 0;
+    lb[j] = in && lens ? cache_lens[base + j] : 0;
+  }
+  bool differ = false;
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) differ |= (a[j] != b[j]) | (la[j] != lb[j]);
+  const int any = __syncthreads_or(differ ? 1 : 0);
+  if (threadIdx.x == 0) {
+    if (any) atomicOr(&st->req_flags, kReqDiffer);
+    s_last = ticket_last(st) ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!s_last) return;
+  if (threadIdx.x == 0) decide_same(st, tag, (atomicExch(&st->req_flags, 0u) & kReqDiffer) != 0u);
+  if (snap && threadIdx.x < 64) publish_snapshot(st, snap, snap_seq);
 }
 
 // Keys per thread and round of the creating lookups: 4 for large requests (fewer atomic adds on
@@ -160,134 +178,197 @@ __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slot
   block_count_add(st, created, cred);
 }
 
-// VARLEN push: find or create; a created row gets ceil(len/4) 16-byte units of the
-// arena, so every row starts 16-byte aligned. A present row must have the pushed length.
-template <int kLookupItems>
-__global__ __launch_bounds__(kBlock) void k_lookup_var_push(
+// VARLEN push, first kernel: one pass over the request's keys and lens that
+//   - compares them with the cached request (when the host found the cache usable),
+//   - takes pass 1 of the lens scan (per-workgroup totals, flags),
+// and whose last workgroup decides whether the request repeats the cached one, scans the
+// totals and, with `snap`, publishes the table's counters. Always launched for a push, so
+// the decision, the scan and the record cost no launch of their own.
+template <int kItems>
+__global__ __launch_bounds__(kBlock) void k_var_push_begin(
+    const uint64_t* __restrict__ keys, const int32_t* __restrict__ lens, uint64_t n,
+    const uint64_t* __restrict__ cache_keys, const int32_t* __restrict__ cache_lens,
+    unsigned long long* __restrict__ part, DevState* st, unsigned max_len, ReqTag tag,
+    Snapshot* snap, uint64_t snap_seq) {
+  __shared__ unsigned long long red[kBlock / 64];
+  __shared__ unsigned fred[kBlock / 64];
+  __shared__ unsigned long long carry_s;
+  __shared__ unsigned s_last;
+  const uint64_t base = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * kItems;
+  // all loads first, then the arithmetic
+  int32_t l[kItems], cl[kItems];
+  uint64_t k[kItems], ck[kItems];
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) {
+    const bool in = base + j < n;
+    l[j] = in ? lens[base + j] : 0;
+    k[j] = ck[j] = 0;
+    cl[j] = l[j];
+    if (in && tag.try_cache) {
+      k[j] = keys[base + j];
+      ck[j] = cache_keys[base + j];
+      cl[j] = cache_lens[base + j];
+    }
+  }
+  unsigned long long s = 0;
+  unsigned flags = 0;
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) {
+    s += (unsigned long long)(long long)l[j];
+    flags |= (unsigned)l[j] & kReqMisaligned;
+    flags |= (l[j] < 0 || (unsigned)l[j] > max_len) ? kReqBadLen : 0u;
+    flags |= (k[j] != ck[j] || l[j] != cl[j]) ? kReqDiffer : 0u;
+  }
+  if (!scan_pass1_block(s, flags, part, st, red, fred, &s_last)) return;
+  flags = scan_pass1_last(part, st, tag.epoch, red, &carry_s);
+  if (threadIdx.x == 0) decide_same(st, tag, (flags & kReqDiffer) != 0u);
+  if (snap && threadIdx.x < 64) publish_snapshot(st, snap, snap_seq);
+}
+
+// VARLEN push, second kernel: pass 2 of the lens scan (request-side offsets and the tile
+// table) and, for the same keys, find-or-create: a created row gets ceil(len/4) 16-byte
+// units of the arena, so every row starts 16-byte aligned; a present row must have the
+// pushed length. A workgroup handles kBlock*kItems consecutive keys: every thread claims
+// slots for its keys, then the workgroup takes the rows of all created keys from the arena
+// with ONE atomic add and a workgroup-wide scan hands them out in request order, so rows of
+// neighbouring keys are neighbours in the arena.
+template <int kItems>
+__global__ __launch_bounds__(kBlock) void k_var_push_lookup(
     Slot* __restrict__ slots, uint64_t mask, DevState* st, const uint64_t* __restrict__ keys,
-    const int32_t* __restrict__ lens, uint64_t n, uint64_t nvals, uint64_t* __restrict__ ref,
+    const int32_t* __restrict__ lens, uint64_t n, uint64_t nvals,
+    const unsigned long long* __restrict__ part, uint64_t* __restrict__ off,
+    uint32_t* __restrict__ tile_key, uint64_t ntiles, uint64_t tile, uint64_t* __restrict__ ref,
     uint64_t* __restrict__ cache_keys, int32_t* __restrict__ cache_lens, ReqTag tag) {
-  if (cache_same(st, tag)) return;  // the references of the cached request are this request's
-  if (blockIdx.x == 0 && threadIdx.x == 0) st->cache_epoch = cache_keys ? tag.epoch : 0ull;
+  if (cache_same(st, tag)) return;  // offsets, tile table and references of the cached request hold
   // the request is refused as a whole when its lens are invalid or do not add up to vals.size()
   if (st->req_error & (kDevErrBadLen | kDevErrSizeMismatch)) return;
   if (st->scan_total != nvals) {
     if (blockIdx.x == 0 && threadIdx.x == 0) raise_error(st, kDevErrSizeMismatch, tag.epoch);
     return;
   }
+  __shared__ unsigned long long wsum[kBlock / 64];
   __shared__ unsigned long long red[kBlock / 64];
   __shared__ unsigned cred[kBlock / 64];
   __shared__ unsigned long long s_first;
-  unsigned created = 0;
-  constexpr uint64_t kRound = (uint64_t)kBlock * kLookupItems;
-  for (uint64_t base = (uint64_t)blockIdx.x * kRound; base < n; base += (uint64_t)gridDim.x * kRound) {
-    uint64_t* p[kLookupItems];
-    uint64_t seen[kLookupItems];
-    uint64_t len[kLookupItems];
-    bool is_new[kLookupItems];
-    unsigned long long units = 0;
-    unsigned mine = 0;
+  const uint64_t base = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * kItems;
+  unsigned long long len[kItems];
 #pragma unroll
-    for (int j = 0; j < kLookupItems; ++j) {
-      const uint64_t i = base + (uint64_t)threadIdx.x * kLookupItems + j;
-      p[j] = nullptr;
-      is_new[j] = false;
-      seen[j] = 0;
-      len[j] = 0;
-      if (i < n) {
-        const uint64_t key = keys[i];
-        len[j] = (uint64_t)(uint32_t)lens[i];
-        if (cache_keys) {
-          cache_keys[i] = key;
-          cache_lens[i] = (int32_t)len[j];
-        }
-        p[j] = find_or_insert(slots, mask, st, key, is_new[j], seen[j]);
-        if (p[j] && !is_new[j] && seen[j] == kPayloadUnset) {
-          atomicOr(&st->error, kDevErrDuplicate);  // the same key twice in this request
-          st->bad_epoch = tag.epoch;
-          p[j] = nullptr;
-        }
-      }
-      if (p[j] && is_new[j]) {
-        units += (len[j] + 3) >> 2;
-        ++mine;
+  for (int j = 0; j < kItems; ++j) len[j] = base + j < n ? (unsigned long long)(uint32_t)lens[base + j] : 0ull;
+  scan_pass2_offsets<kItems>(len, base, n, part[blockIdx.x], off, tile_key, ntiles, tile, wsum);
+
+  uint64_t* p[kItems];
+  uint64_t seen[kItems];
+  bool is_new[kItems];
+  unsigned long long units = 0;
+  unsigned mine = 0;
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) {
+    const uint64_t i = base + j;
+    p[j] = nullptr;
+    is_new[j] = false;
+    seen[j] = 0;
+    if (i < n) {
+      const uint64_t key = keys[i];
+      cache_keys[i] = key;
+      cache_lens[i] = (int32_t)len[j];
+      p[j] = find_or_insert(slots, mask, st, key, is_new[j], seen[j]);
+      if (p[j] && !is_new[j] && seen[j] == kPayloadUnset) {
+        atomicOr(&st->error, kDevErrDuplicate);  // the same key twice in this request
+        st->bad_epoch = tag.epoch;
+        p[j] = nullptr;
       }
     }
-    unsigned long long total;
-    unsigned long long at = block_excl_scan_u64(units, red, total);
-    if (threadIdx.x == 0 && total) s_first = atomicAdd(&st->arena_top, total);
-    __syncthreads();
-    at += total ? s_first : 0ull;
-#pragma unroll
-    for (int j = 0; j < kLookupItems; ++j) {
-      const uint64_t i = base + (uint64_t)threadIdx.x * kLookupItems + j;
-      if (i >= n) continue;
-      if (!p[j]) {
-        ref[i] = kRefAbsent;
-        continue;
-      }
-      uint64_t payload = seen[j];
-      if (is_new[j]) {
-        payload = ((uint64_t)at << kLenBits) | len[j];
-        at += (len[j] + 3) >> 2;
-        *p[j] = payload;
-      } else if ((payload & kLenMask) != len[j]) {
-        raise_error(st, kDevErrLenChanged, tag.epoch);
-      }
-      ref[i] = payload | (is_new[j] ? kRefNew : 0ull);
+    if (p[j] && is_new[j]) {
+      units += (len[j] + 3) >> 2;
+      ++mine;
     }
-    created += mine;
-    __syncthreads();
   }
-  block_count_add(st, created, cred);
+  unsigned long long total;
+  unsigned long long at = block_excl_scan_u64(units, red, total);
+  if (threadIdx.x == 0 && total) s_first = atomicAdd(&st->arena_top, total);
+  __syncthreads();
+  at += total ? s_first : 0ull;
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) {
+    const uint64_t i = base + j;
+    if (i >= n) continue;
+    if (!p[j]) {
+      ref[i] = kRefAbsent;
+      continue;
+    }
+    uint64_t payload = seen[j];
+    if (is_new[j]) {
+      payload = ((uint64_t)at << kLenBits) | len[j];
+      at += (len[j] + 3) >> 2;
+      *p[j] = payload;
+    } else if ((payload & kLenMask) != len[j]) {
+      raise_error(st, kDevErrLenChanged, tag.epoch);
+    }
+    ref[i] = payload | (is_new[j] ? kRefNew : 0ull);
+  }
+  block_count_add(st, mine, cred);
 }
 
-// VARLEN pull: an absent key answers length 0 and is not created.
-// With the keys of the cached push the answer is known without a single probe: every key is
-// present with the cached length.
-__global__ __launch_bounds__(kBlock) void k_lookup_var_pull(const Slot* __restrict__ slots,
-                                                           uint64_t mask, DevState* st,
-                                                           const uint64_t* __restrict__ keys,
-                                                           uint64_t n, uint64_t* __restrict__ ref,
-                                                           int32_t* __restrict__ out_lens,
-                                                           const int32_t* __restrict__ cache_lens,
-                                                           ReqTag tag) {
-  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+// VARLEN pull, first kernel: the stored length of every key (an absent key answers length 0
+// and is not created) together with pass 1 of the scan over those lengths. With the keys of
+// the cached push the answer is known without a single probe: every key is present with the
+// cached length, and the offsets of that push are the offsets of this response.
+template <int kItems>
+__global__ __launch_bounds__(kBlock) void k_var_pull_lookup(
+    const Slot* __restrict__ slots, uint64_t mask, DevState* st, const uint64_t* __restrict__ keys,
+    uint64_t n, uint64_t* __restrict__ ref, int32_t* __restrict__ out_lens,
+    const int32_t* __restrict__ cache_lens, unsigned long long* __restrict__ part, ReqTag tag) {
+  __shared__ unsigned long long red[kBlock / 64];
+  __shared__ unsigned fred[kBlock / 64];
+  __shared__ unsigned long long carry_s;
+  __shared__ unsigned s_last;
+  const uint64_t base = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * kItems;
   if (cache_same(st, tag)) {
-    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride)
-      out_lens[i] = cache_lens[i];
+#pragma unroll
+    for (int j = 0; j < kItems; ++j)
+      if (base + j < n) out_lens[base + j] = cache_lens[base + j];
     return;
   }
   // this pull rewrites the references and offsets in the workspace: the cached push is gone
   if (blockIdx.x == 0 && threadIdx.x == 0) st->bad_epoch = st->cache_epoch;
-  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
-    uint64_t payload;
-    const bool hit = find_only(slots, mask, st, keys[i], payload);
-    ref[i] = hit ? payload : kRefAbsent;
-    out_lens[i] = hit ? (int32_t)(payload & kLenMask) : 0;
+  unsigned long long s = 0;
+  unsigned bits = 0;
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) {
+    const uint64_t i = base + j;
+    if (i < n) {
+      uint64_t payload;
+      const bool hit = find_only(slots, mask, st, keys[i], payload);
+      const uint32_t l = hit ? (uint32_t)(payload & kLenMask) : 0u;
+      ref[i] = hit ? payload : kRefAbsent;
+      out_lens[i] = (int32_t)l;
+      s += l;
+      bits |= l & 3u;
+    }
   }
+  if (!scan_pass1_block(s, bits, part, st, red, fred, &s_last)) return;
+  scan_pass1_last(part, st, tag.epoch, red, &carry_s);
 }
 
-// VARLEN: first key of every request-side tile. Key j owns floats [off[j], off[j+1]);
-// it writes its index for each tile whose first float it owns, so every tile gets
-// exactly one writer and no search is needed later. Entry `ntiles` closes the table.
-// `ntiles_cap` is the room in the table; the tiles in use follow from the scanned total off[n].
-__global__ __launch_bounds__(kBlock) void k_tile_keys(const uint64_t* __restrict__ off, uint64_t n,
-                                                     uint32_t* __restrict__ tile_key,
-                                                     uint64_t ntiles_cap, uint64_t tile,
-                                                     const DevState* st, ReqTag tag) {
-  if (cache_same(st, tag)) return;  // the tile table of the cached request is this request's
-  uint64_t ntiles = (off[n] + tile - 1) / tile;
+// VARLEN pull, second kernel: pass 2 of the scan over the answered lengths: the request-side
+// offsets of the response and its tile table. `ntiles_cap` is the room in the table; the
+// tiles in use follow from the scanned total.
+template <int kItems>
+__global__ __launch_bounds__(kBlock) void k_var_offsets(const int32_t* __restrict__ lens, uint64_t n,
+                                                       const unsigned long long* __restrict__ part,
+                                                       uint64_t* __restrict__ off,
+                                                       uint32_t* __restrict__ tile_key,
+                                                       uint64_t ntiles_cap, uint64_t tile,
+                                                       const DevState* st, ReqTag tag) {
+  if (cache_same(st, tag)) return;  // offsets and tile table of the cached request hold
+  __shared__ unsigned long long wsum[kBlock / 64];
+  uint64_t ntiles = (st->scan_total + tile - 1) / tile;
   if (ntiles > ntiles_cap) ntiles = ntiles_cap;
-  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-  for (uint64_t j = (uint64_t)blockIdx.x * kBlock + threadIdx.x; j < n; j += stride) {
-    const uint64_t a = off[j], b = off[j + 1];
-    if (j == 0) tile_key[ntiles] = (uint32_t)(n - 1);
-    if (b <= a) continue;
-    uint64_t t = (a + tile - 1) / tile;
-    const uint64_t t_last = (b - 1) / tile;
-    for (; t <= t_last && t < ntiles; ++t) tile_key[t] = (uint32_t)j;
-  }
+  const uint64_t base = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * kItems;
+  unsigned long long len[kItems];
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) len[j] = base + j < n ? (unsigned long long)(uint32_t)lens[base + j] : 0ull;
+  scan_pass2_offsets<kItems>(len, base, n, part[blockIdx.x], off, tile_key, ntiles, tile, wsum);
 }
 
 // ---------------------------------------------------------------------------------
