@@ -193,24 +193,27 @@ def run_sparse_lr(args, capi, dev):
     pull_n, pull_ms, pull_s = kernel_stats(tables, capi.KERNEL_PULL_SCALAR)
     for t in tables:
         t.prof_enable(False)
-    # The same timed steps once more on fresh tables that keep the library's default of one
-    # stream per table: kernels of different key ranges then overlap, so whole-job throughput
-    # is higher, but a kernel's duration is no longer its own, which is why the headline
-    # figures above come from the shared-stream run.
-    own = [capi.Table(capi.MODE_SCALAR, initial_capacity=cap) for _ in range(S)]
-    shared, tables = tables, own
-    for i in range(args.warmup):
-        step(i)
-    drain()
-    t1 = time.perf_counter()
-    for i in range(args.warmup, args.warmup + args.steps):
-        step(i)
-    drain()
-    dt_own = time.perf_counter() - t1
-    assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32)), "pulled values differ"
-    for t in own:
-        t.close()
-    tables = shared
+    # On request, the same timed steps once more on fresh tables that keep the library's default
+    # of one stream per table: kernels of different key ranges then overlap, so whole-job
+    # throughput is higher, but a kernel's duration is no longer its own, which is why the
+    # headline figures come from the shared-stream run (and why this pass is not part of the
+    # default command, whose kernel statistics a profiler run is compared with).
+    dt_own = None
+    if args.own_streams:
+        own = [capi.Table(capi.MODE_SCALAR, initial_capacity=cap) for _ in range(S)]
+        shared, tables = tables, own
+        for i in range(args.warmup):
+            step(i)
+        drain()
+        t1 = time.perf_counter()
+        for i in range(args.warmup, args.warmup + args.steps):
+            step(i)
+        drain()
+        dt_own = time.perf_counter() - t1
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32)), "pulled values differ"
+        for t in own:
+            t.close()
+        tables = shared
     # the slicer alone on an idle GPU: two small launches and one read-back of S+1 positions
     t_s = time.perf_counter()
     for _ in range(50):
@@ -232,10 +235,11 @@ def run_sparse_lr(args, capi, dev):
                                                  traffic("pull_scalar", keys_per_launch), pull_s),
                                         bytes_per_key=24),
                     "slicer": {"wall_us_per_call": round(slice_us, 1), "keys": n, "ranges": S}},
-        "own_streams": {"value": 2.0 * n * args.steps / dt_own, "unit": "keys/s",
-                        "ms_per_step": dt_own / args.steps * 1e3,
-                        "note": "same steps, one stream per table (kernels of different ranges overlap)"},
     }
+    if dt_own is not None:
+        res["own_streams"] = {"value": 2.0 * n * args.steps / dt_own, "unit": "keys/s",
+                              "ms_per_step": dt_own / args.steps * 1e3,
+                              "note": "same steps, one stream per table (kernels of different ranges overlap)"}
     return res, batches[args.warmup:args.warmup + args.steps], (n, S)
 
 
@@ -418,28 +422,26 @@ def run_varlen(args, capi, dev):
     for _ in range(1 + args.warmup + 2 * args.steps):
         ref = ref + dv[idx]
     assert torch.equal(out[idx], ref), "var-len sums differ from sequential float adds"
-    # once more with the library's default of one stream per table (launches of different
-    # ranges overlap; durations are then no longer a kernel's own, hence not the headline)
-    for t in tables:
-        t.close()
-    tables = [capi.Table(capi.MODE_VARLEN, initial_capacity=int(n / S * 1.2) * 4,
-                         arena_floats=int(nvals / S * 1.5) + 8 * n // S) for _ in range(S)]
-    step()
-    for _ in range(args.warmup):
+    # on request, once more with the library's default of one stream per table (launches of
+    # different ranges overlap; durations are then no longer a kernel's own, hence not the headline)
+    dt_own = None
+    if args.own_streams:
+        for t in tables:
+            t.close()
+        tables = [capi.Table(capi.MODE_VARLEN, initial_capacity=int(n / S * 1.2) * 4,
+                             arena_floats=int(nvals / S * 1.5) + 8 * n // S) for _ in range(S)]
         step()
-    drain()
-    t1 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    drain()
-    dt_own = time.perf_counter() - t1
-    assert torch.equal(out_lens, dl), "pulled lens differ"
+        for _ in range(args.warmup):
+            step()
+        drain()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        drain()
+        dt_own = time.perf_counter() - t1
+        assert torch.equal(out_lens, dl), "pulled lens differ"
     floats_per_launch = nvals / S
     res = {
-        "own_streams": {"value": 2.0 * n * args.steps / dt_own, "unit": "keys/s",
-                        "ms_per_step": dt_own / args.steps * 1e3,
-                        "gbps": (20.0 * nvals + 56.0 * n) * args.steps / dt_own / 1e9,
-                        "note": "same steps, one stream per table (kernels of different ranges overlap)"},
         "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
         "dtype": "f32",
         "config": {"workload": "varlen: 2M keys, lens in {8,16,32,64,128}, 16 key ranges, push then "
@@ -453,6 +455,11 @@ def run_varlen(args, capi, dev):
                                                  traffic("rows_gather_varlen", floats_per_launch), gat[2]),
                                         bytes_per_float=8)},
     }
+    if dt_own is not None:
+        res["own_streams"] = {"value": 2.0 * n * args.steps / dt_own, "unit": "keys/s",
+                              "ms_per_step": dt_own / args.steps * 1e3,
+                              "gbps": (20.0 * nvals + 56.0 * n) * args.steps / dt_own / 1e9,
+                              "note": "same steps, one stream per table (kernels of different ranges overlap)"}
     return res, (keys, lens, nvals, n, S)
 
 
@@ -484,6 +491,9 @@ def main():
     ap.add_argument("--keys", type=int, default=0, help="keys per step (default: the config's)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the dense-chunk side measurement")
+    ap.add_argument("--own-streams", action="store_true",
+                    help="sparse_lr / varlen: also time the steps with one stream per table "
+                         "(reported under extra.own_streams; kernels of different ranges overlap)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures ONE GPU: a table lives on one device and nothing here uses a "

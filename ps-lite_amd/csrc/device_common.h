@@ -129,15 +129,18 @@ __device__ __forceinline__ void raise_error(DevState* st, unsigned bit, unsigned
 // on one address are served one at a time (about 15 ns each).
 // The counters are left at zero; kernels that use it must not overlap on one table.
 __device__ __forceinline__ bool ticket_last(DevState* st) {
-  const unsigned shards = gridDim.x < (unsigned)kTicketShards ? gridDim.x : (unsigned)kTicketShards;
-  const unsigned sub = blockIdx.x % shards;
-  const unsigned members = (gridDim.x - sub + shards - 1) / shards;  // workgroups b with b % shards == sub
-  unsigned* c = &st->ticket_sub[sub * 32];
   // this thread's atomics and atomic stores are complete before its ticket is taken
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_s_waitcnt(0);
-  if (atomicAdd(c, 1u) != members - 1) return false;
-  *c = 0;
+  unsigned shards = gridDim.x;  // a small grid goes straight to the second level
+  if (gridDim.x > (unsigned)kTicketShards) {
+    shards = (unsigned)kTicketShards;
+    const unsigned sub = blockIdx.x % shards;
+    const unsigned members = (gridDim.x - sub + shards - 1) / shards;  // workgroups b with b % shards == sub
+    unsigned* c = &st->ticket_sub[sub * 32];
+    if (atomicAdd(c, 1u) != members - 1) return false;
+    *c = 0;
+  }
   if (atomicAdd(&st->ticket_top, 1u) != shards - 1) return false;
   st->ticket_top = 0;
   __threadfence();  // acquire, once per grid: nothing stale is left in this XCD's L2
