@@ -339,6 +339,8 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
   auto arena_short = [&]() {
     return units && (t->base_top + t->pend_units + units) * floats_per_unit > t->arena_cap;
   };
+  // an ageing base is refreshed from the newest record whenever one has arrived (a host read)
+  if (t->seq - t->base_seq >= (uint64_t)pskv_table::kLog / 4) adopt_snapshot(t);
   if (slots_short() || arena_short() || t->seq - t->base_seq >= (uint64_t)pskv_table::kLog - 1) {
     adopt_snapshot(t);
     if (slots_short() || arena_short() || t->seq - t->base_seq >= (uint64_t)pskv_table::kLog - 1) {
@@ -363,7 +365,10 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
   const bool tight_slots = (double)(t->base_count + t->pend_keys + 2 * n) > limit_now;
   const bool tight_arena =
       units && (t->base_top + t->pend_units + 2 * units) * floats_per_unit > t->arena_cap;
-  if (tight_slots || tight_arena || t->seq - t->base_seq >= (uint64_t)pskv_table::kLog / 2) {
+  // (a base that merely grows old asks for a record every eighth request, not every one)
+  const uint64_t age = t->seq - t->base_seq;
+  const bool old_base = age >= (uint64_t)pskv_table::kLog / 4 && (age % 8 == 0 || age >= (uint64_t)pskv_table::kLog - 8);
+  if (tight_slots || tight_arena || old_base) {
     if (carry) {
       carry->snap = t->snap;
       carry->seq = q;
@@ -854,6 +859,9 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
     default: rc = run_varlen(t, r); break;
   }
   if (out_nvals) *out_nvals = r.out_nvals;
+  // Kernels of this request may still be reading the pinned request buffer, which the next
+  // host-resident request overwrites from the host: no early return without a wait.
+  if (small && (rc || too_small)) (void)hipStreamSynchronize(t->stream);
   if (rc) {
     t->cache_valid = false;
     return rc;
