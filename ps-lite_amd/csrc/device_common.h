@@ -85,7 +85,7 @@ constexpr unsigned kReqMisaligned = 3u;  // OR of (len & 3)
 constexpr unsigned kReqBadLen = 4u;      // a length negative or above the maximum
 constexpr unsigned kReqDiffer = 8u;      // a key or length differs from the cached request
 
-// Counters of the table as of the start of request `seq`, written by the device into pinned
+// Counters of the table as they are after request `seq`, written by the device into pinned
 // host memory so that the host can bound the counters without waiting for the stream.
 // seq_begin == seq_end marks a consistent record.
 struct Snapshot {

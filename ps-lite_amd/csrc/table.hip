@@ -74,8 +74,8 @@ __global__ void k_read_state(const DevState* st, StateView* out) {
   out->special_present = st->special_present;
 }
 
-// One wavefront, launched in front of a request's kernels when the table is close to a limit
-// and no kernel of the request can carry the record.
+// One wavefront, launched behind the kernel of a SCALAR request when the table is close to a
+// limit (the row modes let their lookup kernels write the record).
 __global__ void k_publish(const DevState* st, Snapshot* out, uint64_t seq) {
   publish_snapshot(st, out, seq);
 }
@@ -265,7 +265,8 @@ int alloc_slots(uint64_t cap, Slot** out, hipStream_t stream) {
   return PSKV_OK;
 }
 
-// Moves the base of the bounds forward to the newest record the device has published.
+// Moves the base of the bounds forward to the newest record the device has published: the
+// counters after request `seq_end`.
 void adopt_snapshot(pskv_table* t) {
   const Snapshot* sn = t->snap;
   const uint64_t s1 = sn->seq_end;
@@ -273,12 +274,12 @@ void adopt_snapshot(pskv_table* t) {
   const uint64_t c = sn->count, top = sn->arena_top;
   std::atomic_thread_fence(std::memory_order_acquire);
   const uint64_t s0 = sn->seq_begin;
-  if (s0 != s1 || s1 <= t->base_seq || s1 > t->seq) return;
-  for (uint64_t r = t->base_seq; r < s1; ++r) {
+  if (s0 != s1 || s1 < t->base_seq || s1 >= t->seq) return;  // (the initial record is all ones)
+  for (uint64_t r = t->base_seq; r <= s1; ++r) {
     t->pend_keys -= t->log_keys[r % pskv_table::kLog];
     t->pend_units -= t->log_units[r % pskv_table::kLog];
   }
-  t->base_seq = s1;
+  t->base_seq = s1 + 1;
   t->base_count = c;
   t->base_top = top;
 }
@@ -321,18 +322,16 @@ int grow_arena(pskv_table* t, uint64_t floats_needed, uint64_t live_floats) {
 // path touches no device state; the next best reads the snapshot the device published;
 // only then does it wait for the stream and read the counters.
 //
-// Close to a limit the device publishes its counters in front of the request, so that a later
-// request can move the base forward without waiting for the stream. With `carry` the caller
-// promises to hand the record to a kernel of the request that runs before any of its
-// kernels changes a counter (carry->snap is set when a record is wanted); without it a
-// one-wavefront kernel is launched here.
+// Close to a limit the device publishes its counters as they are after the request, so that a
+// later request can move the base forward without waiting for the stream: `pub->snap` is
+// set when a record is wanted, and the caller hands it to the kernel of the request that
+// changes the counters (or launches k_publish behind it).
 struct PublishReq {
   Snapshot* snap = nullptr;
   uint64_t seq = 0;
 };
 
-int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
-            PublishReq* carry = nullptr) {
+int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit, PublishReq* pub) {
   if (t->no_growth) return PSKV_OK;
   const double limit = (double)t->max_load * (double)t->cap;
   auto slots_short = [&]() { return (double)(t->base_count + t->pend_keys + n) > limit; };
@@ -369,13 +368,8 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
   const uint64_t age = t->seq - t->base_seq;
   const bool old_base = age >= (uint64_t)pskv_table::kLog / 4 && (age % 8 == 0 || age >= (uint64_t)pskv_table::kLog - 8);
   if (tight_slots || tight_arena || old_base) {
-    if (carry) {
-      carry->snap = t->snap;
-      carry->seq = q;
-    } else {
-      k_publish<<<dim3(1), dim3(64), 0, t->stream>>>(t->st, t->snap, q);
-      PSKV_HIP(hipGetLastError());
-    }
+    pub->snap = t->snap;
+    pub->seq = q;
   }
   return PSKV_OK;
 }
@@ -401,7 +395,8 @@ struct Request {
 int run_scalar(pskv_table* t, Request& r) {
   r.out_nvals = r.pull ? r.n : 0;
   if (r.n == 0) return PSKV_OK;
-  int rc = reserve(t, r.n, 0, 0);
+  PublishReq pub;
+  int rc = reserve(t, r.n, 0, 0, &pub);
   if (rc) return rc;
   const dim3 grid(grid_for(r.n, kBlock, kMaxGrid)), block(kBlock);
   const uint64_t mask = t->cap - 1;
@@ -415,6 +410,7 @@ int run_scalar(pskv_table* t, Request& r) {
     launch(t, PSKV_KERNEL_PULL_SCALAR, k_scalar<false, true>, grid, block, t->slots, mask, t->st,
            r.keys, (const float*)nullptr, r.out, r.n);
   }
+  if (pub.snap) k_publish<<<dim3(1), dim3(64), 0, t->stream>>>(t->st, pub.snap, pub.seq);
   PSKV_HIP(hipGetLastError());
   return PSKV_OK;
 }
@@ -453,21 +449,13 @@ ReqTag next_tag(pskv_table* t, const Request& r) {
 
 // Starts a row-mode request: numbers it and, when the key cache has the right shape, lets the
 // device compare the request with the cached one. Call after every buffer the cache lives in
-// has been grown for this request. A counter record the request has to publish (`pub`) rides
-// on the compare kernel, or gets a launch of its own when there is none.
-int begin_row_request(pskv_table* t, const Request& r, bool with_lens, ReqTag* tag,
-                      const PublishReq* pub) {
+// has been grown for this request.
+int begin_row_request(pskv_table* t, const Request& r, bool with_lens, ReqTag* tag) {
   *tag = next_tag(t, r);
-  Snapshot* snap = pub ? pub->snap : nullptr;
-  const uint64_t seq = pub ? pub->seq : 0;
   if (tag->try_cache) {
     k_same_keys<<<dim3((unsigned)((r.n + kBlock * 4 - 1) / (kBlock * 4))), dim3(kBlock), 0, t->stream>>>(
         r.keys, with_lens ? r.lens : nullptr, static_cast<const uint64_t*>(t->cache_keys.ptr),
-        with_lens ? static_cast<const int32_t*>(t->cache_lens.ptr) : nullptr, r.n, t->st, *tag, snap,
-        seq);
-    PSKV_HIP(hipGetLastError());
-  } else if (snap) {
-    k_publish<<<dim3(1), dim3(64), 0, t->stream>>>(t->st, snap, seq);
+        with_lens ? static_cast<const int32_t*>(t->cache_lens.ptr) : nullptr, r.n, t->st, *tag);
     PSKV_HIP(hipGetLastError());
   }
   return PSKV_OK;
@@ -488,15 +476,16 @@ int run_fixed(pskv_table* t, Request& r) {
   uint64_t* ref = c.take<uint64_t>(r.n);
   uint64_t* cache_keys = static_cast<uint64_t*>(t->cache_keys.ptr);
   ReqTag tag;
-  rc = begin_row_request(t, r, false, &tag, &pub);
+  rc = begin_row_request(t, r, false, &tag);
   if (rc) return rc;
   if (r.n >= kLookupLargeKeys) {
     launch(t, PSKV_KERNEL_LOOKUP, k_lookup_fixed<kLookupItemsLarge>,
            dim3(grid_for(r.n, kBlock * kLookupItemsLarge, kMaxGrid)), dim3(kBlock), t->slots,
-           t->cap - 1, t->st, r.keys, r.n, ref, cache_keys, tag);
+           t->cap - 1, t->st, r.keys, r.n, ref, cache_keys, tag, pub.snap, pub.seq);
   } else {
     launch(t, PSKV_KERNEL_LOOKUP, k_lookup_fixed<1>, dim3(grid_for(r.n, kBlock, kMaxGrid)),
-           dim3(kBlock), t->slots, t->cap - 1, t->st, r.keys, r.n, ref, cache_keys, tag);
+           dim3(kBlock), t->slots, t->cap - 1, t->st, r.keys, r.n, ref, cache_keys, tag, pub.snap,
+           pub.seq);
   }
   PSKV_HIP(hipGetLastError());
   // push and pull both create absent keys, so either leaves references for all n keys behind
@@ -565,8 +554,8 @@ int make_tile_tables(pskv_table* t, const int32_t* lens_out, const unsigned long
   return PSKV_OK;
 }
 
-// Launches per var-len request: a push takes three (compare + scan pass 1 + counter record;
-// scan pass 2 + find-or-create; rows), a pull four (compare; stored lengths + scan pass 1;
+// Launches per var-len request: a push takes three (compare + scan pass 1; scan pass 2 +
+// find-or-create + counter record; rows), a pull four (compare; stored lengths + scan pass 1;
 // scan pass 2 + tile table; rows).
 int run_varlen(pskv_table* t, Request& r) {
   r.out_nvals = 0;
@@ -611,7 +600,7 @@ int run_varlen(pskv_table* t, Request& r) {
     const ReqTag tag = next_tag(t, r);
     launch_keys(t, -1, r.n, k_var_push_begin<1>, k_var_push_begin<kScanItemsLarge>, r.keys, r.lens, r.n,
                 (const uint64_t*)cache_keys, (const int32_t*)cache_lens, part, t->st,
-                (unsigned)PSKV_MAX_VARLEN_ROW, tag, pub.snap, pub.seq);
+                (unsigned)PSKV_MAX_VARLEN_ROW, tag);
     PSKV_HIP(hipGetLastError());
     // pass 2 also fills the tile table of the request side (tile sizes are those of nvals; a
     // request whose lens do not add up to nvals is refused before it gets there)
@@ -619,7 +608,7 @@ int run_varlen(pskv_table* t, Request& r) {
     launch_keys(t, PSKV_KERNEL_LOOKUP, r.n, k_var_push_lookup<1>, k_var_push_lookup<kScanItemsLarge>,
                 t->slots, t->cap - 1, t->st, r.keys, r.lens, r.n, r.nvals,
                 (const unsigned long long*)part, off, r.nvals ? push_tile_key : (uint32_t*)nullptr,
-                tiles_cap, (uint64_t)kTileVar, ref, cache_keys, cache_lens, tag);
+                tiles_cap, (uint64_t)kTileVar, ref, cache_keys, cache_lens, tag, pub.snap, pub.seq);
     PSKV_HIP(hipGetLastError());
     t->cache_valid = true;  // whichever way the device decided, the cache now is this request
     t->cache_n = r.n;
@@ -649,7 +638,7 @@ int run_varlen(pskv_table* t, Request& r) {
     // A pull with the keys of the cached push finds every key present with the cached length
     // and reuses its references; any other pull recomputes them and so ends the cache.
     ReqTag tag;
-    rc = begin_row_request(t, r, false, &tag, nullptr);
+    rc = begin_row_request(t, r, false, &tag);
     if (rc) return rc;
     if (!tag.try_cache) t->cache_valid = false;
     launch_keys(t, PSKV_KERNEL_LOOKUP, r.n, k_var_pull_lookup<1>, k_var_pull_lookup<kScanItemsLarge>,
@@ -949,7 +938,7 @@ int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
       hipHostMalloc(reinterpret_cast<void**>(&t->small_out), kSmallBytes, hipHostMallocCoherent) !=
           hipSuccess)
     return fail(set_error(PSKV_ENOMEM, "cannot allocate table state"));
-  std::memset(t->snap, 0, sizeof(Snapshot));
+  std::memset(t->snap, 0xFF, sizeof(Snapshot));  // names no request
   if (t->mode != PSKV_MODE_SCALAR && opts->arena_floats) {
     t->arena_cap = (opts->arena_floats + 1023) & ~(uint64_t)1023;
     if (hipMalloc(reinterpret_cast<void**>(&t->arena), t->arena_cap * sizeof(float)) != hipSuccess)

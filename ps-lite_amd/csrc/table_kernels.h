@@ -67,14 +67,12 @@ __device__ __forceinline__ void decide_same(DevState* st, const ReqTag& tag, boo
 
 // Compares a request with the cached one (keys, and lens when given) and reaches the decision
 // for the whole request: the workgroup that finishes last sees whether any workgroup found a
-// difference and writes same_epoch. With `snap` it also publishes the table's counters,
-// which no kernel is changing at this point of the stream.
+// difference and writes same_epoch.
 __global__ __launch_bounds__(kBlock) void k_same_keys(const uint64_t* __restrict__ keys,
                                                      const int32_t* __restrict__ lens,
                                                      const uint64_t* __restrict__ cache_keys,
                                                      const int32_t* __restrict__ cache_lens,
-                                                     uint64_t n, DevState* st, ReqTag tag,
-                                                     Snapshot* snap, uint64_t snap_seq) {
+                                                     uint64_t n, DevState* st, ReqTag tag) {
   __shared__ unsigned s_last;
   constexpr int kItems = 4;
   const uint64_t base = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * kItems;
@@ -100,7 +98,18 @@ __global__ __launch_bounds__(kBlock) void k_same_keys(const uint64_t* __restrict
   __syncthreads();
   if (!s_last) return;
   if (threadIdx.x == 0) decide_same(st, tag, (atomicExch(&st->req_flags, 0u) & kReqDiffer) != 0u);
-  if (snap && threadIdx.x < 64) publish_snapshot(st, snap, snap_seq);
+}
+
+// The counter record of a request, written by the kernel that creates its keys once every
+// workgroup has taken its rows (or at once when the request creates nothing): the record then
+// holds the counters as they are AFTER the request. Every thread of the workgroup calls it;
+// `s_last` is one word of LDS.
+__device__ __forceinline__ void publish_after_lookup(DevState* st, Snapshot* snap, uint64_t seq,
+                                                     unsigned* s_last) {
+  if (!snap) return;
+  if (threadIdx.x == 0) *s_last = ticket_last(st) ? 1u : 0u;
+  __syncthreads();
+  if (*s_last && threadIdx.x < 64) publish_snapshot(st, snap, seq);
 }
 
 // Keys per thread and round of the creating lookups: 4 for large requests (fewer atomic adds on
@@ -120,12 +129,17 @@ __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slot
                                                         const uint64_t* __restrict__ keys,
                                                         uint64_t n, uint64_t* __restrict__ ref,
                                                         uint64_t* __restrict__ cache_keys,
-                                                        ReqTag tag) {
-  if (cache_same(st, tag)) return;  // the references of the cached request are this request's
+                                                        ReqTag tag, Snapshot* snap,
+                                                        uint64_t snap_seq) {
+  if (cache_same(st, tag)) {  // the references of the cached request are this request's
+    if (snap && blockIdx.x == 0 && threadIdx.x < 64) publish_snapshot(st, snap, snap_seq);
+    return;
+  }
   if (blockIdx.x == 0 && threadIdx.x == 0) st->cache_epoch = cache_keys ? tag.epoch : 0ull;
   __shared__ unsigned long long red[kBlock / 64];
   __shared__ unsigned cred[kBlock / 64];
   __shared__ unsigned long long s_first;
+  __shared__ unsigned s_last;
   unsigned created = 0;
   constexpr uint64_t kRound = (uint64_t)kBlock * kLookupItems;
   for (uint64_t base = (uint64_t)blockIdx.x * kRound; base < n; base += (uint64_t)gridDim.x * kRound) {
@@ -176,20 +190,20 @@ __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slot
     __syncthreads();  // s_first and red are reused by the next round
   }
   block_count_add(st, created, cred);
+  publish_after_lookup(st, snap, snap_seq, &s_last);
 }
 
 // VARLEN push, first kernel: one pass over the request's keys and lens that
 //   - compares them with the cached request (when the host found the cache usable),
 //   - takes pass 1 of the lens scan (per-workgroup totals, flags),
-// and whose last workgroup decides whether the request repeats the cached one, scans the
-// totals and, with `snap`, publishes the table's counters. Always launched for a push, so
-// the decision, the scan and the record cost no launch of their own.
+// and whose last workgroup decides whether the request repeats the cached one and scans the
+// totals. Always launched for a push, so the decision and the scan cost no launch of their
+// own.
 template <int kItems>
 __global__ __launch_bounds__(kBlock) void k_var_push_begin(
     const uint64_t* __restrict__ keys, const int32_t* __restrict__ lens, uint64_t n,
     const uint64_t* __restrict__ cache_keys, const int32_t* __restrict__ cache_lens,
-    unsigned long long* __restrict__ part, DevState* st, unsigned max_len, ReqTag tag,
-    Snapshot* snap, uint64_t snap_seq) {
+    unsigned long long* __restrict__ part, DevState* st, unsigned max_len, ReqTag tag) {
   __shared__ unsigned long long red[kBlock / 64];
   __shared__ unsigned fred[kBlock / 64];
   __shared__ unsigned long long carry_s;
@@ -222,7 +236,6 @@ __global__ __launch_bounds__(kBlock) void k_var_push_begin(
   if (!scan_pass1_block(s, flags, part, st, red, fred, &s_last)) return;
   flags = scan_pass1_last(part, st, tag.epoch, red, &carry_s);
   if (threadIdx.x == 0) decide_same(st, tag, (flags & kReqDiffer) != 0u);
-  if (snap && threadIdx.x < 64) publish_snapshot(st, snap, snap_seq);
 }
 
 // VARLEN push, second kernel: pass 2 of the lens scan (request-side offsets and the tile
@@ -238,8 +251,12 @@ __global__ __launch_bounds__(kBlock) void k_var_push_lookup(
     const int32_t* __restrict__ lens, uint64_t n, uint64_t nvals,
     const unsigned long long* __restrict__ part, uint64_t* __restrict__ off,
     uint32_t* __restrict__ tile_key, uint64_t ntiles, uint64_t tile, uint64_t* __restrict__ ref,
-    uint64_t* __restrict__ cache_keys, int32_t* __restrict__ cache_lens, ReqTag tag) {
-  if (cache_same(st, tag)) return;  // offsets, tile table and references of the cached request hold
+    uint64_t* __restrict__ cache_keys, int32_t* __restrict__ cache_lens, ReqTag tag,
+    Snapshot* snap, uint64_t snap_seq) {
+  if (cache_same(st, tag)) {  // offsets, tile table and references of the cached request hold
+    if (snap && blockIdx.x == 0 && threadIdx.x < 64) publish_snapshot(st, snap, snap_seq);
+    return;
+  }
   // the request is refused as a whole when its lens are invalid or do not add up to vals.size()
   if (st->req_error & (kDevErrBadLen | kDevErrSizeMismatch)) return;
   if (st->scan_total != nvals) {
@@ -250,6 +267,7 @@ __global__ __launch_bounds__(kBlock) void k_var_push_lookup(
   __shared__ unsigned long long red[kBlock / 64];
   __shared__ unsigned cred[kBlock / 64];
   __shared__ unsigned long long s_first;
+  __shared__ unsigned s_last;
   const uint64_t base = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * kItems;
   unsigned long long len[kItems];
 #pragma unroll
@@ -307,6 +325,7 @@ __global__ __launch_bounds__(kBlock) void k_var_push_lookup(
     ref[i] = payload | (is_new[j] ? kRefNew : 0ull);
   }
   block_count_add(st, mine, cred);
+  publish_after_lookup(st, snap, snap_seq, &s_last);
 }
 
 // VARLEN pull, first kernel: the stored length of every key (an absent key answers length 0
