@@ -36,6 +36,7 @@ constexpr uint64_t kDefaultCapacity = 1u << 20;
 constexpr uint64_t kMinSlots = 1024;
 constexpr unsigned kMaxGrid = 1u << 20;
 constexpr size_t kMaxProfSamples = 65536;
+constexpr uint64_t kSlackBytes = 256ull << 20;  // tables up to this size trade memory for fewer waits
 // Host-resident requests up to this size (per direction) skip the copy commands: the kernels
 // read the request from, and write the response to, pinned host memory mapped into the GPU.
 constexpr size_t kSmallBytes = 1024u << 10;
@@ -345,12 +346,19 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
     if (slots_short() || arena_short() || t->seq - t->base_seq >= (uint64_t)pskv_table::kLog - 1) {
       int rc = read_state(t);  // exact counters, stream idle
       if (rc) return rc;
-      if (slots_short()) {
-        rc = grow_slots(t, t->base_count + n);
+      // The wait happened because requests in flight had to be assumed to create all their
+      // keys. Small tables get room for two more such requests, so that a caller who keeps
+      // requests of this size in flight does not wait again on every one of them; for large
+      // tables the wait is short next to their kernels and the memory is not.
+      const uint64_t slack_n = t->cap * sizeof(Slot) <= kSlackBytes ? 2 * n : 0;
+      const uint64_t slack_u = t->arena_cap * sizeof(float) <= kSlackBytes ? 2 * units : 0;
+      if ((double)(t->base_count + n + slack_n) > limit) {
+        rc = grow_slots(t, t->base_count + n + slack_n);
         if (rc) return rc;
       }
-      if (arena_short()) {
-        rc = grow_arena(t, (t->base_top + units) * floats_per_unit, t->base_top * floats_per_unit);
+      if (units && (t->base_top + units + slack_u) * floats_per_unit > t->arena_cap) {
+        rc = grow_arena(t, (t->base_top + units + slack_u) * floats_per_unit,
+                        t->base_top * floats_per_unit);
         if (rc) return rc;
       }
     }
