@@ -109,6 +109,94 @@ def test_scalar_growth(capi, orc, dev):
     _check_dump(t, o, "growth")
 
 
+@pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
+def test_many_requests_in_flight_while_the_table_grows(capi, orc, dev, mode):
+    """Device-resident requests are enqueued without waiting, so the host only has bounds on the
+    table's counters (every key of a request in flight may be new) and moves them forward from the
+    records the device publishes. 240 requests without a single sync from the caller, with key sets
+    that repeat, overlap and bring new keys, a table that starts at its minimum size and, for the row
+    modes, an arena that starts empty: slots and arena must always have been grown in time."""
+    import torch
+    announce("requests_in_flight", mode)
+    rng = np.random.default_rng({"scalar": 11, "fixed": 12, "varlen": 13}[mode])
+    m = {"scalar": capi.MODE_SCALAR, "fixed": capi.MODE_FIXED, "varlen": capi.MODE_VARLEN}[mode]
+    om = {"scalar": orc.MODE_SCALAR, "fixed": orc.MODE_FIXED, "varlen": orc.MODE_VARLEN}[mode]
+    k = 8
+    t = capi.Table(m, initial_capacity=1, row_len=k if mode == "fixed" else 0)
+    o = orc.Store(om)
+    universe = unique_keys(rng, 60000)
+    len_of = rng.choice(np.array([4, 8, 12, 16], np.int32), size=universe.size)
+    keep = []  # device buffers of requests in flight must stay alive
+    prev = None
+    for rep in range(240):
+        r = rng.random()
+        if prev is not None and r < 0.5:
+            idx = prev  # the same keys again: the steady state of a parameter server
+        elif r < 0.8:
+            lo = int(rng.integers(0, universe.size - 3000))
+            idx = np.arange(lo, lo + int(rng.integers(1, 3000)))
+        else:
+            idx = np.flatnonzero(rng.random(universe.size) < 0.02 * (1 + rep % 5))
+        prev = idx
+        keys = universe[idx]
+        if mode == "scalar":
+            lens, vals = None, rng.standard_normal(keys.size).astype(np.float32)
+        elif mode == "fixed":
+            lens, vals = None, rng.standard_normal(keys.size * k).astype(np.float32)
+        else:
+            lens = len_of[idx]
+            vals = rng.standard_normal(int(lens.sum())).astype(np.float32)
+        dk, dv = to_dev(keys, dev), to_dev(vals, dev)
+        dl = to_dev(lens, dev) if lens is not None else None
+        keep.append((dk, dv, dl))
+        t.push(dk, dv, dl)
+        o.push(keys, vals, lens)
+        if rep % 7 == 3 and mode != "varlen":  # pulls create keys too (not in var-len mode)
+            extra = universe[rng.integers(0, universe.size, size=50)]
+            extra = np.unique(extra)
+            de = to_dev(extra, dev)
+            out = torch.empty(extra.size * (k if mode == "fixed" else 1), dtype=torch.float32, device=dev)
+            keep.append((de, out, None))
+            t.pull(de, out)
+            o.pull(extra)
+    t.sync()
+    _check_dump(t, o, "requests in flight")
+
+
+def test_device_time_accounting(capi, dev):
+    """pskv_prof_*: every launch of the listed kernels is timed by its own pair of events; the samples
+    add up to the total, and the copy probe moves what it says."""
+    import torch
+    announce("prof")
+    n = 100000
+    keys = to_dev(unique_keys(np.random.default_rng(3), n), dev)
+    vals = torch.ones(n, dtype=torch.float32, device=dev)
+    out = torch.zeros(n, dtype=torch.float32, device=dev)
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=2 * n)
+    t.push(keys, vals)  # not counted: profiling is off
+    t.prof_enable(True)
+    t.prof_reset()
+    for _ in range(5):
+        t.push(keys, vals)
+    t.pull(keys, out)
+    src = torch.arange(1 << 20, dtype=torch.float32, device=dev)
+    dst = torch.zeros(1 << 20, dtype=torch.float32, device=dev)
+    t.copy_probe(dst, src)
+    launches, total_ms = t.prof_read(capi.KERNEL_PUSH_SCALAR)
+    samples = t.prof_samples(capi.KERNEL_PUSH_SCALAR)
+    assert launches == 5 and samples.size == 5
+    assert np.all(samples > 0) and abs(float(samples.sum()) - total_ms) < 1e-3 * max(total_ms, 1e-3) + 1e-4
+    assert t.prof_read(capi.KERNEL_PULL_SCALAR)[0] == 1
+    assert t.prof_read(capi.KERNEL_COPY)[0] == 1
+    assert torch.equal(dst, src)
+    assert np.all(from_dev(out) == 6.0)
+    t.prof_enable(False)
+    t.push(keys, vals)
+    assert t.prof_read(capi.KERNEL_PUSH_SCALAR)[0] == 5
+    t.prof_reset()
+    assert t.prof_read(capi.KERNEL_PUSH_SCALAR) == (0, 0.0) and t.prof_samples(capi.KERNEL_PUSH_SCALAR).size == 0
+
+
 def test_scalar_size_checks(capi, dev):
     announce("scalar_size_checks")
     t = capi.Table(capi.MODE_SCALAR)
