@@ -12,6 +12,8 @@ Workloads (BASELINE.json `configs`):
       1 GiB followed by one full pull. value = algorithmic GB/s.
   varlen (configs[4]): 2,000,000 keys with lens in {8,16,32,64,128} over 16 ranges; a
       step is one push of all keys followed by a pull with lens. value = keys/s.
+  zipf (configs[3]): one table; a step pushes 4,000,000 distinct Zipf(1.1)-popular keys
+      of a 100M-key universe and pulls them back; 8 steps. value = keys/s.
 
 Prints ONE JSON line. Inputs are resident in HBM before the clock starts. `value` comes
 from exactly K timed steps. `roofline` is the dominant kernel of the workload: after the
@@ -482,12 +484,97 @@ def cpu_varlen(orc, keys, lens, nvals, n, S, budget_s=15.0):
             "sample": "%d full steps (slice + push + pull of %d keys, %d floats), one thread" % (done, n, nvals)}
 
 
+# ------------------------------------------------------------------------------------
+# zipf: configs[3]
+# ------------------------------------------------------------------------------------
+def zipf_unique_keys(rng, n, universe, s=1.1):
+    """n distinct keys whose ranks in [0, universe) have Zipf(s) popularity, sorted. A rank
+    becomes a key through an injective scatter over the covered key space."""
+    got = np.zeros(0, np.int64)
+    while got.size < n:
+        r = rng.zipf(s, size=2 * n).astype(np.int64) - 1
+        got = np.unique(np.concatenate([got, r[(r >= 0) & (r < universe)]]))
+    if got.size > n:
+        got = np.sort(rng.choice(got, size=n, replace=False))
+    keys = (got.astype(np.uint64) * np.uint64(0x9E3779B97F4A7C15)) >> np.uint64(1)
+    return np.sort(keys)
+
+
+def run_zipf(args, capi, dev):
+    """A step is one worker's push of 4M Zipf-popular keys (a growing share of them already
+    stored) followed by a pull of the same keys; one table, which grows (and rehashes) inside
+    the timed region as it would in service."""
+    import torch
+    n, universe = args.keys or 4000000, 100000000
+    total = args.warmup + args.steps
+    log("generating %d Zipf batches of %d keys" % (total, n))
+    batches = []
+    for w in range(total):
+        rng = np.random.default_rng(0x21F + w)
+        batches.append((zipf_unique_keys(rng, n, universe), rng.standard_normal(n).astype(np.float32)))
+    d_batches = [(to_dev(k, dev), to_dev(v, dev)) for k, v in batches]
+    out = torch.empty(n, dtype=torch.float32, device=dev)
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=1 << 20)
+    t.prof_enable(True)  # one launch per request: per-launch events cost nothing that matters here
+
+    def step(i):
+        dk, dv = d_batches[i]
+        t.push(dk, dv)
+        t.pull(dk, out)
+
+    for i in range(args.warmup):
+        step(i)
+    t.sync()
+    t.prof_reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.warmup, total):
+        step(i)
+    t.sync()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    push = kernel_stats([t], capi.KERNEL_PUSH_SCALAR)
+    pull = kernel_stats([t], capi.KERNEL_PULL_SCALAR)
+    rehash = kernel_stats([t], capi.KERNEL_REHASH)
+    held = t.size()[0]
+    res = {
+        "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
+        "dtype": "f32",
+        "config": {"workload": "zipf: pushes of 4M distinct Zipf(1.1)-popular keys from a 100M-key "
+                               "universe into one table, each followed by a pull of the same keys",
+                   "keys_per_step": n, "ranges": 1, "value_len": 1, "key_dtype": "u64",
+                   "store_keys_after_timed_steps": held},
+        # between a hit (28 B/key) and an insert (32 B/key); priced as inserts
+        "roofline": dict(roofline(32.0 * n, push[0], push[1], None, push[2]),
+                         kernel="k_scalar<push> (find-or-insert + add)", bytes_per_key=32),
+        "kernels": {"pull_scalar": dict(roofline(24.0 * n, pull[0], pull[1], None, pull[2]), bytes_per_key=24),
+                    "rehash": {"launches": rehash[0], "total_us": round(rehash[1] * 1e3, 1)}},
+    }
+    return res, batches[args.warmup:], n
+
+
+def cpu_zipf(orc, batches, n, budget_s=25.0):
+    store = orc.Store(orc.MODE_SCALAR)
+    done = 0
+    t0 = time.perf_counter()
+    for keys, vals in batches:
+        store.push(keys, vals)
+        store.handle(False, True, keys, out_cap=n)
+        done += 1
+        if time.perf_counter() - t0 > budget_s:
+            break
+    dt = time.perf_counter() - t0
+    return {"value": 2.0 * n * done / dt, "unit": "keys/s", "cores": 1, "kind": "port",
+            "sample": "first %d of the timed steps (push + pull of %d keys each), one "
+                      "std::unordered_map store, one thread" % (done, n)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="sparse_lr", choices=["sparse_lr", "dense", "varlen"])
+    ap.add_argument("--workload", default="sparse_lr", choices=["sparse_lr", "dense", "varlen", "zipf"])
     ap.add_argument("--keys", type=int, default=0, help="keys per step (default: the config's)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the dense-chunk side measurement")
@@ -510,6 +597,10 @@ def main():
         res, timed_batches, (n, S) = run_sparse_lr(args, capi, dev)
     elif args.workload == "dense":
         res = run_dense(args, capi, dev)
+    elif args.workload == "zipf":
+        if args.steps == 20:
+            args.steps = 8  # the configuration has 8 worker pushes
+        res, zipf_batches, zipf_n = run_zipf(args, capi, dev)
     else:
         res, varlen_inputs = run_varlen(args, capi, dev)
 
@@ -535,6 +626,8 @@ def main():
             cpu = cpu_sparse_lr(orc, timed_batches, n, S)
         elif args.workload == "dense":
             cpu = cpu_dense(orc)
+        elif args.workload == "zipf":
+            cpu = cpu_zipf(orc, zipf_batches, zipf_n)
         else:
             cpu = cpu_varlen(orc, *varlen_inputs)
         cpu["host"] = host_info()
