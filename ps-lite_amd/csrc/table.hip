@@ -602,7 +602,8 @@ int run_varlen(pskv_table* t, Request& r) {
 
   if (r.push) {
     PublishReq pub;
-    rc = reserve(t, r.n, r.nvals / 4 + r.n, 4, &pub);
+    // every key may round its row up to a 16-byte unit, every workgroup may pad its rows' start
+    rc = reserve(t, r.n, r.nvals / 4 + r.n + kArenaPadUnits * nparts, 4, &pub);
     if (rc) return rc;
     if (t->cache_nvals != r.nvals) t->cache_valid = false;  // same lens would mean the same total
     const ReqTag tag = next_tag(t, r);
