@@ -163,6 +163,61 @@ def test_many_requests_in_flight_while_the_table_grows(capi, orc, dev, mode):
     _check_dump(t, o, "requests in flight")
 
 
+def test_tables_driven_from_other_threads(capi, orc, dev):
+    """ps-lite calls a request handle on the Customer thread of its KVServer (src/customer.cc:49-63),
+    not on the thread that built it, and the servers of different apps run at the same time: four
+    tables made here are each driven from a thread of their own, with host buffers, concurrently."""
+    import threading
+    announce("tables_on_threads")
+    modes = [(capi.MODE_SCALAR, orc.MODE_SCALAR), (capi.MODE_FIXED, orc.MODE_FIXED),
+             (capi.MODE_VARLEN, orc.MODE_VARLEN), (capi.MODE_SCALAR, orc.MODE_SCALAR)]
+    tables = [capi.Table(m, initial_capacity=64, row_len=4 if m == capi.MODE_FIXED else 0) for m, _ in modes]
+    failures = []
+
+    def drive(i):
+        try:
+            t, (m, om) = tables[i], modes[i]
+            o = orc.Store(om)
+            rng = np.random.default_rng(500 + i)
+            universe = unique_keys(rng, 4000)
+            lens_all = rng.choice(np.array([4, 8, 20], np.int32), size=universe.size)
+            for rep in range(40):
+                idx = np.flatnonzero(rng.random(universe.size) < 0.3)
+                keys = universe[idx]
+                if m == capi.MODE_SCALAR:
+                    lens, vals = None, rng.standard_normal(keys.size).astype(np.float32)
+                elif m == capi.MODE_FIXED:
+                    lens, vals = None, rng.standard_normal(keys.size * 4).astype(np.float32)
+                else:
+                    lens = lens_all[idx]
+                    vals = rng.standard_normal(int(lens.sum())).astype(np.float32)
+                t.push(keys, vals, lens)
+                o.push(keys, vals, lens)
+                if rep % 5 == 4:
+                    want, want_lens = o.pull(keys)
+                    got = np.zeros(want.size, np.float32)
+                    got_lens = np.zeros(keys.size, np.int32) if m == capi.MODE_VARLEN else None
+                    t.pull(keys, got, got_lens)
+                    assert_bits_equal(got, want, "thread %d pull" % i)
+                    if got_lens is not None:
+                        assert np.array_equal(got_lens, want_lens)
+            # an error on this thread is this thread's: the message names this table's problem
+            with pytest.raises(capi.PskvError) as e:
+                t.push(universe[:3], np.zeros(7 if m != capi.MODE_VARLEN else 5, np.float32),
+                       np.array([1, 2, 3], np.int32) if m == capi.MODE_VARLEN else None)
+            assert e.value.code == capi.ESIZE_MISMATCH
+            _check_dump(t, o, "thread %d" % i)
+        except BaseException as exc:  # noqa: BLE001 - reported on the main thread
+            failures.append((i, repr(exc)))
+
+    threads = [threading.Thread(target=drive, args=(i,)) for i in range(len(tables))]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not failures, failures
+
+
 def test_device_time_accounting(capi, dev):
     """pskv_prof_*: every launch of the listed kernels is timed by its own pair of events; the samples
     add up to the total, and the copy probe moves what it says."""
