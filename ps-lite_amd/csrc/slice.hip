@@ -14,6 +14,8 @@
 namespace pskv {
 namespace {
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 // One wavefront per search target: a 64-ary lower_bound. Each round the 64 lanes probe
 // evenly spaced keys of the remaining interval, a ballot counts how many are below
 // the target (the probes are sorted, so the votes are a prefix of ones) and the
@@ -109,6 +111,48 @@ __global__ void k_response_ends(const uint64_t* const* __restrict__ resp_keys,
   if (r >= R) return;
   targets[2 * r] = resp_keys[r][0];
   targets[2 * r + 1] = resp_keys[r][resp_nkeys[r] - 1] + 1;  // wraps to 0 for kMaxKey, as Key does
+}
+
+// One piece of a concatenation: `bytes` bytes (a multiple of 4, 4-byte aligned) from src to dst.
+struct Segment {
+  const char* src;
+  char* dst;
+  uint64_t bytes;
+};
+
+struct __attribute__((packed, aligned(4))) Words4 {
+  uint32_t w[4];
+};
+
+// Copies all segments of a table (blockIdx.y = segment; the workgroups of a row stride over
+// it). The destination is written with aligned 128-bit stores whatever its start: the first
+// lanes move single words up to the next 16-byte boundary, and the loads that feed the
+// stores may then sit on any 4-byte boundary, which global memory allows.
+__global__ __launch_bounds__(kBlock) void k_concat(const Segment* __restrict__ segs) {
+  const Segment sg = segs[blockIdx.y];
+  if (sg.bytes == 0) return;
+  uint64_t head = (16 - (reinterpret_cast<uintptr_t>(sg.dst) & 15)) & 15;  // bytes to the boundary
+  if (head > sg.bytes) head = sg.bytes;
+  const uint64_t body = (sg.bytes - head) / 16;  // 128-bit pieces
+  const uint64_t tail_at = head + body * 16;
+  const uint64_t t0 = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (t0 < head / 4)
+    reinterpret_cast<uint32_t*>(sg.dst)[t0] = reinterpret_cast<const uint32_t*>(sg.src)[t0];
+  if (t0 < (sg.bytes - tail_at) / 4)
+    reinterpret_cast<uint32_t*>(sg.dst + tail_at)[t0] =
+        reinterpret_cast<const uint32_t*>(sg.src + tail_at)[t0];
+  const Words4* src = reinterpret_cast<const Words4*>(sg.src + head);
+  f32x4* dst = reinterpret_cast<f32x4*>(sg.dst + head);
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t i = t0; i < body; i += stride) {
+    const Words4 x = src[i];
+    f32x4 y;
+    y.x = __uint_as_float(x.w[0]);
+    y.y = __uint_as_float(x.w[1]);
+    y.z = __uint_as_float(x.w[2]);
+    y.w = __uint_as_float(x.w[3]);
+    __builtin_nontemporal_store(y, dst + i);
+  }
 }
 
 // Per-call state of the slicer. Calls may come from any thread at once
@@ -368,31 +412,26 @@ int pskv_assemble_pull(int device, const uint64_t* req_keys, size_t n, size_t R,
     CtxLease lease(device);
     SliceCtx* c = lease.c;
     if (!c) return set_error(PSKV_EHIP, "cannot create a context on device %d", device);
-    // device scratch: key pointers[R] | nkeys[R] | targets[2R] | lb[2R]
-    const size_t a = pad256(R * 8), b = pad256(2 * R * 8);
-    int rc = ctx_reserve(c, 2 * a + 2 * b, 2 * a + 2 * b, 0);
+    // pinned, read and written by the kernels in place:
+    //   key pointers[R] | nkeys[R] | targets[2R] | lower bounds[2R] | segments[2R]
+    const size_t a = pad256(R * 8), b = pad256(2 * R * 8), sg = pad256(2 * R * sizeof(Segment));
+    int rc = ctx_reserve(c, 0, 2 * a + 2 * b + sg, 0);
     if (rc) return rc;
-    char* d = static_cast<char*>(c->dev);
     char* h = static_cast<char*>(c->pinned);
-    const uint64_t** d_ptrs = reinterpret_cast<const uint64_t**>(d);
-    uint64_t* d_nk = reinterpret_cast<uint64_t*>(d + a);
-    uint64_t* d_targets = reinterpret_cast<uint64_t*>(d + 2 * a);
-    uint64_t* d_lb = reinterpret_cast<uint64_t*>(d + 2 * a + b);
     const uint64_t** h_ptrs = reinterpret_cast<const uint64_t**>(h);
     uint64_t* h_nk = reinterpret_cast<uint64_t*>(h + a);
     uint64_t* h_targets = reinterpret_cast<uint64_t*>(h + 2 * a);
     uint64_t* h_lb = reinterpret_cast<uint64_t*>(h + 2 * a + b);
+    Segment* h_segs = reinterpret_cast<Segment*>(h + 2 * a + 2 * b);
     for (size_t r = 0; r < R; ++r) {
       h_ptrs[r] = resp_keys[r];
       h_nk[r] = resp_nkeys[r];
     }
-    PSKV_HIP(hipMemcpyAsync(d, h, 2 * a, hipMemcpyHostToDevice, c->stream));
-    k_response_ends<<<dim3((unsigned)((R + 63) / 64)), dim3(64), 0, c->stream>>>(d_ptrs, d_nk, R,
-                                                                                 d_targets);
+    k_response_ends<<<dim3((unsigned)((R + 63) / 64)), dim3(64), 0, c->stream>>>(h_ptrs, h_nk, R,
+                                                                                 h_targets);
     PSKV_HIP(hipGetLastError());
-    rc = launch_bounds_search(req_keys, n, d_targets, 2 * R, d_lb, c->stream);
+    rc = launch_bounds_search(req_keys, n, h_targets, 2 * R, h_lb, c->stream);
     if (rc) return rc;
-    PSKV_HIP(hipMemcpyAsync(h_targets, d_targets, 2 * b, hipMemcpyDeviceToHost, c->stream));
     PSKV_HIP(hipStreamSynchronize(c->stream));
     for (size_t r = 0; r < R; ++r) {  // kv_app.h:670-677
       const uint64_t lower = h_targets[2 * r], upper = h_targets[2 * r + 1];
@@ -411,17 +450,29 @@ int pskv_assemble_pull(int device, const uint64_t* req_keys, size_t n, size_t R,
     std::iota(order.begin(), order.end(), (size_t)0);
     std::sort(order.begin(), order.end(),  // kv_app.h:681-684
               [&](size_t x, size_t y) { return ends[2 * x] < ends[2 * y]; });
-    size_t voff = 0, koff = 0;
-    for (size_t i = 0; i < R; ++i) {  // kv_app.h:701-708
+    // kv_app.h:701-708: one launch copies every slice to its place
+    size_t voff = 0, koff = 0, nseg = 0;
+    uint64_t longest = 0;
+    for (size_t i = 0; i < R; ++i) {
       const size_t r = order[i];
-      if (resp_nvals[r])
-        PSKV_HIP(hipMemcpyAsync(out + voff, resp_vals[r], resp_nvals[r] * sizeof(float),
-                                hipMemcpyDeviceToDevice, c->stream));
+      if (resp_nvals[r]) {
+        h_segs[nseg++] = Segment{reinterpret_cast<const char*>(resp_vals[r]),
+                                 reinterpret_cast<char*>(out + voff), resp_nvals[r] * sizeof(float)};
+        longest = std::max<uint64_t>(longest, resp_nvals[r] * sizeof(float));
+      }
       voff += resp_nvals[r];
-      if (out_lens && resp_lens)
-        PSKV_HIP(hipMemcpyAsync(out_lens + koff, resp_lens[r], resp_nkeys[r] * sizeof(int32_t),
-                                hipMemcpyDeviceToDevice, c->stream));
+      if (out_lens && resp_lens) {
+        h_segs[nseg++] = Segment{reinterpret_cast<const char*>(resp_lens[r]),
+                                 reinterpret_cast<char*>(out_lens + koff), resp_nkeys[r] * sizeof(int32_t)};
+        longest = std::max<uint64_t>(longest, resp_nkeys[r] * sizeof(int32_t));
+      }
       koff += resp_nkeys[r];
+    }
+    for (size_t first = 0; first < nseg; first += 65535) {  // gridDim.y holds 65535 segments
+      const size_t now = std::min<size_t>(nseg - first, 65535);
+      const uint64_t per = std::min<uint64_t>(longest / (16 * kBlock) + 1, 4096);
+      k_concat<<<dim3((unsigned)per, (unsigned)now), dim3(kBlock), 0, c->stream>>>(h_segs + first);
+      PSKV_HIP(hipGetLastError());
     }
     PSKV_HIP(hipStreamSynchronize(c->stream));
     return PSKV_OK;

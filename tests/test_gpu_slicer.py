@@ -163,6 +163,45 @@ def test_slice_push_pull_round_trip(capi, orc, dev):
     assert_bits_equal(o_vals, want, "oracle reassembly")
 
 
+@pytest.mark.parametrize("R", [1, 3, 7])
+def test_assemble_pieces_on_any_word_boundary(capi, dev, R):
+    """The reassembly copies every slice to its place with one launch; slices of 1, 2, 3, 5... floats
+    make sources and destinations start on any 4-byte boundary, and some are shorter than 16 bytes."""
+    import torch
+    announce("assemble_unaligned", R)
+    rng = np.random.default_rng(70 + R)
+    n = 5000
+    keys = unique_keys(rng, n)
+    lens = rng.choice(np.array([0, 1, 2, 3, 5, 7, 33], np.int32), size=n).astype(np.int32)
+    cuts = np.sort(rng.choice(np.arange(1, n), size=R - 1, replace=False)) if R > 1 else np.zeros(0, np.int64)
+    pos = np.concatenate([[0], cuts, [n]]).astype(np.int64)
+    off = np.concatenate([[0], np.cumsum(lens.astype(np.int64))])
+    vals = rng.standard_normal(int(off[-1])).astype(np.float32)
+    dk = to_dev(keys, dev)
+    # every response lives at an odd offset of a larger buffer, so its start is not 16-byte aligned
+    responses = []
+    for r in range(R):
+        a, b = int(pos[r]), int(pos[r + 1])
+        pad = int(rng.integers(1, 4))
+        vbuf = torch.zeros(int(off[b] - off[a]) + pad, dtype=torch.float32, device=dev)
+        vbuf[pad:] = to_dev(vals[off[a]:off[b]], dev)
+        lbuf = torch.zeros(b - a + pad, dtype=torch.int32, device=dev)
+        lbuf[pad:] = to_dev(lens[a:b], dev)
+        responses.append((dk[a:b], vbuf[pad:], lbuf[pad:]))
+    order = rng.permutation(R)
+    responses = [responses[i] for i in order]
+    guard = 3
+    out = torch.full((vals.size + 2 * guard,), 7.0, dtype=torch.float32, device=dev)
+    out_lens = torch.full((n + 2 * guard,), -1, dtype=torch.int32, device=dev)
+    got = capi.assemble_pull(dk, responses, out[guard:guard + vals.size], out_lens[guard:guard + n])
+    assert got == vals.size
+    o, ol = from_dev(out), from_dev(out_lens)
+    assert_bits_equal(o[guard:guard + vals.size], vals, "assembled values")
+    assert np.array_equal(ol[guard:guard + n], lens)
+    assert np.all(o[:guard] == 7.0) and np.all(o[guard + vals.size:] == 7.0), "wrote outside the response"
+    assert np.all(ol[:guard] == -1) and np.all(ol[guard + n:] == -1), "wrote outside the lens"
+
+
 def test_assemble_errors(capi, dev):
     import torch
     announce("assemble_errors")
