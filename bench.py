@@ -45,7 +45,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 TRAFFIC = {
     ("push_scalar", 250000): 60.9e6, ("pull_scalar", 250000): 36.2e6,
     ("rows_acc_fixed", 268435456): 3.0 * 2**30, ("rows_gather_fixed", 268435456): 2.0 * 2**30,
-    ("rows_acc_varlen", 6192336): 77.1e6, ("rows_gather_varlen", 6192336): 51.4e6,
+    ("rows_acc_varlen", 6192336): 76.4e6, ("rows_gather_varlen", 6192336): 50.9e6,
 }
 
 
