@@ -465,6 +465,42 @@ def run_varlen(args, capi, dev):
     return res, (keys, lens, nvals, n, S)
 
 
+def cpu_dense_all_cores(orc, threads=16, nk=64, k=4194304, budget_s=8.0):
+    """The same row loop sharded by key over `threads` host threads, each with a store of its
+    own (keys are independent, so this is how a multi-threaded CPU server would split the
+    work). Labelled as such: the reference runs its handle on one thread."""
+    import threading
+    per = nk // threads
+    rng = np.random.default_rng(0xD15E)
+    vals = rng.uniform(-1, 1, size=per * k).astype(np.float32)  # every thread pushes the same floats
+    stores, keysets = [], []
+    for t in range(threads):
+        keys = np.uint64(KMAX // nk) * np.arange(t * per, (t + 1) * per, dtype=np.uint64)
+        st = orc.Store(orc.MODE_FIXED, k)
+        st.push(keys, vals)
+        stores.append(st)
+        keysets.append(keys)
+    counts = [0] * threads
+    stop = time.perf_counter() + budget_s
+
+    def work(t):
+        while time.perf_counter() < stop:
+            stores[t].push(keysets[t], vals)
+            stores[t].handle(False, True, keysets[t], out_cap=vals.size)
+            counts[t] += 1
+
+    ths = [threading.Thread(target=work, args=(t,)) for t in range(threads)]
+    t0 = time.perf_counter()
+    for th in ths:
+        th.start()
+    for th in ths:
+        th.join()
+    dt = time.perf_counter() - t0
+    return {"value": 20.0 * vals.size * sum(counts) / dt / 1e9, "unit": "GB/s", "cores": threads,
+            "kind": "port", "sample": "all-core variant: %d threads, each push + pull of %d rows of %d "
+                                      "floats into its own store, %d steps in total" % (threads, per, k, sum(counts))}
+
+
 def cpu_varlen(orc, keys, lens, nvals, n, S, budget_s=15.0):
     rng = np.random.default_rng(0xE3D)
     vals = rng.normal(0, 0.1, size=nvals).astype(np.float32)
@@ -626,6 +662,7 @@ def main():
             cpu = cpu_sparse_lr(orc, timed_batches, n, S)
         elif args.workload == "dense":
             cpu = cpu_dense(orc)
+            extra["cpu_baseline_all_cores"] = cpu_dense_all_cores(orc)
         elif args.workload == "zipf":
             cpu = cpu_zipf(orc, zipf_batches, zipf_n)
         else:
