@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 REPO = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libpskv.so")
-SOURCES = ["table.hip", "slice.hip", "hostmem.hip"]
+SOURCES = ["table.hip", "slice.hip", "hostmem.hip", "meta_codec.cc"]
 HEADERS = ["device_common.h", "host_common.h", "scan.h", "table_kernels.h"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -39,7 +39,7 @@ def build_lib(verbose=False):
     objs = []
     procs = []
     for src in SOURCES:
-        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
         cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
