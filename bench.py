@@ -378,6 +378,7 @@ def run_varlen(args, capi, dev):
     dv = torch.randn(nvals, device=dev, generator=g) * 0.1
     out = torch.empty(nvals, dtype=torch.float32, device=dev)
     out_lens = torch.empty(n, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()  # the raw-pointer calls below do not wait for torch's stream
     stream = torch.cuda.Stream()  # one stream for all ranges: kernels run one at a time
     tables = [capi.Table(capi.MODE_VARLEN, initial_capacity=int(n / S * 1.2) * 4,
                          arena_floats=int(nvals / S * 1.5) + 8 * n // S, stream=stream.cuda_stream)

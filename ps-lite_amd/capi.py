@@ -129,7 +129,15 @@ def _buf(x, dtype_np, dtype_name):
 def _memkind(*kinds):
     ks = {k for k in kinds if k is not None}
     assert len(ks) <= 1, "all buffers of a call must live in the same kind of memory"
-    return ks.pop() if ks else MEM_HOST
+    kind = ks.pop() if ks else MEM_HOST
+    if kind == MEM_DEVICE:
+        # The C ABI wants device buffers complete before the call (the library runs on streams of
+        # its own). torch fills and copies tensors asynchronously on ITS current stream, so the
+        # methods that take tensors wait for that stream first; the *_raw methods leave it to
+        # the caller.
+        import torch
+        torch.cuda.current_stream().synchronize()
+    return kind
 
 
 class Table:

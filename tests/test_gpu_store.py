@@ -440,12 +440,14 @@ def test_varlen_pull_without_host_round_trip(capi, orc, dev):
     dp = to_dev(probe, dev)
     out = torch.full((want.size + 4096,), 7.0, dtype=torch.float32, device=dev)  # more room than needed
     out_lens = torch.full((probe.size,), -1, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()  # raw pointers: torch's fills above must have landed
     t.pull_raw(dp.data_ptr(), probe.size, out.data_ptr(), out.numel(), out_lens.data_ptr())
     t.sync()
     assert np.array_equal(from_dev(out_lens), want_lens)
     assert_bits_equal(from_dev(out)[:want.size], want, "async pull")
     assert np.all(from_dev(out)[want.size:] == 7.0)  # nothing written past the response
     small = torch.full((want.size - 8,), 7.0, dtype=torch.float32, device=dev)
+    torch.cuda.synchronize()
     t.pull_raw(dp.data_ptr(), probe.size, small.data_ptr(), small.numel(), out_lens.data_ptr())
     with pytest.raises(capi.PskvError) as e:
         t.sync()
@@ -550,6 +552,7 @@ def test_repeated_and_alternating_key_sets(capi, orc, dev, mode, seed):
                 dk = to_dev(keys, dev)
                 out = torch.full((want.size + 64,), 7.0, dtype=torch.float32, device=dev)
                 out_lens = torch.full((keys.size,), -1, dtype=torch.int32, device=dev)
+                torch.cuda.synchronize()  # raw pointers: torch's fills above must have landed
                 t.pull_raw(dk.data_ptr(), keys.size, out.data_ptr(), out.numel(),
                            out_lens.data_ptr() if mode == "varlen" else None)
                 t.sync()
