@@ -16,11 +16,12 @@ Workloads (BASELINE.json `configs`):
       of a 100M-key universe and pulls them back; 8 steps. value = keys/s.
 
 Prints ONE JSON line. Inputs are resident in HBM before the clock starts. `value` comes
-from exactly K timed steps. `roofline` is the dominant kernel of the workload: after the
-timed steps the same steps run again with every launch of the store kernels carrying its
-own start/stop HIP events on the stream it runs on (per-launch events cost about 15 us of
-host time each, which is why they stay out of the timed region). `cpu_baseline` is the CPU
-oracle on the same inputs, one thread, on a bounded sample.
+from exactly K timed steps. `roofline` is the dominant kernel of the workload, timed inside
+those same steps: launches carry their own start/stop HIP events on the stream they run on
+(hipExtLaunchKernelGGL). A pair of events costs about 15 us of host time per launch (and a
+few on the GPU), so the steps are sampled: every fourth step times its launches, for the
+workloads with several tables those of ONE table, taken in turn. `cpu_baseline` is the CPU oracle on the same inputs, one thread, on a
+bounded sample.
 """
 import argparse
 import json
@@ -35,7 +36,11 @@ sys.path.insert(0, REPO)
 import __graft_entry__ as graft  # noqa: E402
 
 KMAX = (1 << 64) - 1
-HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+HBM_PEAK_GBS = 8000.0
+# Launches that carry their own start/stop events cost host time (about 15 us each) and a
+# few microseconds on the GPU, so the timed steps are sampled: every SAMPLE_EVERY-th step
+# times its launches (for the many-table workloads: those of one table, taken in turn).
+SAMPLE_EVERY = 4  # MI355X HBM3E, published
 
 # HBM bytes per launch (read + written) of the dominant kernels at the shapes below, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this very script, scaled by what the same
@@ -131,8 +136,7 @@ def gen_sparse_lr(steps, n, S):
 def run_sparse_lr(args, capi, dev):
     import torch
     n, S = args.keys or 1000000, 4
-    # the timed steps are followed by as many instrumented steps of the same shape
-    total_steps = args.warmup + 2 * args.steps
+    total_steps = args.warmup + args.steps
     log("generating %d batches of %d keys" % (total_steps, n))
     batches = gen_sparse_lr(total_steps, n, S)
     rb, re = capi.server_ranges(S)
@@ -142,11 +146,19 @@ def run_sparse_lr(args, capi, dev):
     # share one stream: their kernels run back to back, each with the whole GPU, so a
     # kernel's duration is its own and not that of four overlapping launches.
     stream = torch.cuda.Stream()
-    cap = int(n * total_steps / S * 1.1)
+    # sized so that the tables end the run about one third of the way to their first growth
+    cap = int(n * (args.warmup + 2 * args.steps) / S * 1.1)
     tables = [capi.Table(capi.MODE_SCALAR, initial_capacity=cap, stream=stream.cuda_stream)
               for _ in range(S)]
 
-    def step(i):
+    def step(i, sample=True):
+        # Kernel durations are sampled INSIDE the timed steps: in every SAMPLE_EVERY-th step the
+        # launches of one of the S tables (taken in turn) carry their own start/stop events.
+        # Events on every launch would cost more host time per step than the GPU needs for it.
+        if sample:
+            j = i - args.warmup
+            for s in range(S):
+                tables[s].prof_enable(j >= 0 and j % SAMPLE_EVERY == 0 and s == (j // SAMPLE_EVERY) % S)
         dk, dv = d_batches[i]
         kp, vp, op = dk.data_ptr(), dv.data_ptr(), out.data_ptr()
         pos, _, used = capi.slice_keys(dk, rb, re, nvals=n)
@@ -168,11 +180,17 @@ def run_sparse_lr(args, capi, dev):
     for i in range(args.warmup):
         step(i)
     drain()
+    for t in tables:
+        t.prof_reset()
     t0 = time.perf_counter()
     for i in range(args.warmup, args.warmup + args.steps):
         step(i)
     drain()
     dt = time.perf_counter() - t0
+    push_n, push_ms, push_s = kernel_stats(tables, capi.KERNEL_PUSH_SCALAR)
+    pull_n, pull_ms, pull_s = kernel_stats(tables, capi.KERNEL_PULL_SCALAR)
+    for t in tables:
+        t.prof_enable(False)
 
     # last pull must hold exactly the pushed values: each key was pushed once (0.0f + v)
     last = args.warmup + args.steps - 1
@@ -182,19 +200,6 @@ def run_sparse_lr(args, capi, dev):
     held = sum(t.size()[0] for t in tables)
     assert held == n * (args.warmup + args.steps), (held, n * (args.warmup + args.steps))
 
-    # Instrumented pass: the same steps continue with fresh keys while every launch of the
-    # store kernels is bracketed by HIP events on the stream it runs on. It is kept out of
-    # the timed region because an event pair per launch adds about 60 us to a 140 us step.
-    for t in tables:
-        t.prof_enable(True)
-        t.prof_reset()
-    for i in range(args.warmup + args.steps, total_steps):
-        step(i)
-    drain()
-    push_n, push_ms, push_s = kernel_stats(tables, capi.KERNEL_PUSH_SCALAR)
-    pull_n, pull_ms, pull_s = kernel_stats(tables, capi.KERNEL_PULL_SCALAR)
-    for t in tables:
-        t.prof_enable(False)
     # On request, the same timed steps once more on fresh tables that keep the library's default
     # of one stream per table: kernels of different key ranges then overlap, so whole-job
     # throughput is higher, but a kernel's duration is no longer its own, which is why the
@@ -205,11 +210,11 @@ def run_sparse_lr(args, capi, dev):
         own = [capi.Table(capi.MODE_SCALAR, initial_capacity=cap) for _ in range(S)]
         shared, tables = tables, own
         for i in range(args.warmup):
-            step(i)
+            step(i, sample=False)
         drain()
         t1 = time.perf_counter()
         for i in range(args.warmup, args.warmup + args.steps):
-            step(i)
+            step(i, sample=False)
         drain()
         dt_own = time.perf_counter() - t1
         assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32)), "pulled values differ"
@@ -286,26 +291,23 @@ def measure_dense(capi, dev, steps, warmup, nk=64, k=4194304):
         t.pull(keys, out)
     t.sync()
     torch.cuda.synchronize()
+    # the launches of every SAMPLE_EVERY-th timed step carry their own HIP events
+    t.prof_enable(True)
+    t.prof_reset()
     t0 = time.perf_counter()
-    for _ in range(steps):
+    for i in range(steps):
+        t.prof_enable(i % SAMPLE_EVERY == 0)
         t.push(keys, vals)
         t.pull(keys, out)
     t.sync()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    # instrumented pass: the same steps again, every launch carrying its own HIP events
-    t.prof_enable(True)
-    t.prof_reset()
-    for _ in range(steps):
-        t.push(keys, vals)
-        t.pull(keys, out)
-    t.sync()
     acc = kernel_stats([t], capi.KERNEL_ROWS_ACC)
     gat = kernel_stats([t], capi.KERNEL_ROWS_GATHER)
-    # closed form: every float holds (1 + warmup + 2*steps) * v, accumulated one add at a time
+    # closed form: every float holds (1 + warmup + steps) * v, accumulated one add at a time
     idx = torch.randint(0, nk * k, (4096,), device=dev)
     ref = torch.zeros(4096, device=dev)
-    for _ in range(1 + warmup + 2 * steps):
+    for _ in range(1 + warmup + steps):
         ref = ref + vals[idx]
     assert torch.equal(out[idx], ref), "dense sums differ from sequential float adds"
     # plain copies of the same 1 GiB: the known-size launch that memory-traffic counters are
@@ -406,23 +408,25 @@ def run_varlen(args, capi, dev):
     for _ in range(args.warmup):
         step()
     drain()
+    for t in tables:
+        t.prof_reset()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for i in range(args.steps):
+        # kernel durations are sampled inside the timed steps: in every SAMPLE_EVERY-th step the
+        # launches of one table, taken in turn, carry their own events
+        for s in range(S):
+            tables[s].prof_enable(i % SAMPLE_EVERY == 0 and s == (i // SAMPLE_EVERY) % S)
         step()
     drain()
     dt = time.perf_counter() - t0
-    for t in tables:
-        t.prof_enable(True)
-        t.prof_reset()
-    for _ in range(args.steps):
-        step()
-    drain()
     acc = kernel_stats(tables, capi.KERNEL_ROWS_ACC)
     gat = kernel_stats(tables, capi.KERNEL_ROWS_GATHER)
+    for t in tables:
+        t.prof_enable(False)
     assert torch.equal(out_lens, dl), "pulled lens differ"
     idx = torch.randint(0, nvals, (4096,), device=dev)
     ref = torch.zeros(4096, device=dev)
-    for _ in range(1 + args.warmup + 2 * args.steps):
+    for _ in range(1 + args.warmup + args.steps):
         ref = ref + dv[idx]
     assert torch.equal(out[idx], ref), "var-len sums differ from sequential float adds"
     # on request, once more with the library's default of one stream per table (launches of
