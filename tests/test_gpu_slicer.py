@@ -44,6 +44,28 @@ def test_slice_uniform(capi, orc, dev, memkind, n, S):
     assert _compare(capi, orc, keys, rb, re, None, 0, dev, memkind) == 0
 
 
+@pytest.mark.parametrize("S", [1, 64, 1024])
+def test_slice_sixteen_million_keys(capi, dev, S):
+    """The largest request of the benchmark configurations (a pull of 16M keys): positions against
+    numpy's searchsorted, the lens sums against cumsum, and the invariants of kv_app.h:528-542."""
+    announce("slice_16M", S)
+    n = 16000000
+    rng = np.random.default_rng(16 + S)
+    rb, re = capi.server_ranges(S)
+    keys = unique_keys(rng, n, S)
+    lens = rng.integers(0, 5, size=n).astype(np.int32)
+    dk, dl = to_dev(keys, dev), to_dev(lens, dev)
+    pos, vpos, used = capi.slice_keys(dk, rb, re, lens=dl, nvals=int(lens.sum()))
+    want = np.concatenate([[np.searchsorted(keys, rb[0], side="left")], np.searchsorted(keys, re, side="left")])
+    assert np.array_equal(pos.astype(np.int64), want.astype(np.int64))
+    assert pos[0] == 0 and pos[-1] == n and np.all(np.diff(pos.astype(np.int64)) >= 0)
+    off = np.concatenate([[0], np.cumsum(lens.astype(np.int64))])
+    assert np.array_equal(vpos.astype(np.int64), off[pos.astype(np.int64)])
+    assert np.array_equal(used.astype(bool), np.diff(pos.astype(np.int64)) > 0)
+    pos2, vpos2, _ = capi.slice_keys(dk, rb, re, nvals=2 * n)  # no lens: k = 2
+    assert np.array_equal(pos2, pos) and np.array_equal(vpos2.astype(np.int64), 2 * pos.astype(np.int64))
+
+
 @pytest.mark.parametrize("memkind", ["device", "host"])
 def test_slice_skewed_and_edges(capi, orc, dev, memkind):
     """All keys in one range, keys sitting exactly on range boundaries, empty middle slices."""
