@@ -296,3 +296,26 @@ def assemble_pull(req_keys, responses, out, out_lens=None, device=0):
 
 def version():
     return load().pskv_version().decode()
+
+
+def host_alloc(nbytes):
+    """A pinned host buffer (address) from the library's pool; give it back with host_free."""
+    p = load().pskv_host_alloc(nbytes)
+    if not p:
+        raise PskvError(ENOMEM, load().pskv_last_error().decode())
+    return p
+
+
+def host_free(ptr):
+    load().pskv_host_free(ptr)
+
+
+def host_trim():
+    _check(load().pskv_host_trim())
+
+
+def host_array(ptr, count, dtype):
+    """A numpy view of `count` elements of `dtype` at a pinned address from host_alloc."""
+    dt = np.dtype(dtype)
+    raw = (ctypes.c_char * (count * dt.itemsize)).from_address(ptr)
+    return np.frombuffer(raw, dtype=dt, count=count)

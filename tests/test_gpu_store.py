@@ -218,6 +218,72 @@ def test_tables_driven_from_other_threads(capi, orc, dev):
     assert not failures, failures
 
 
+def test_pinned_pool(capi, orc, dev):
+    """pskv_host_alloc / pskv_host_free / pskv_host_trim: buffers are pinned, reusable, may be given
+    back from any thread (a ps-lite response is released on a transport thread, zmq_van.h:20-26),
+    and serve as request and response buffers of host-resident calls of any size."""
+    import threading
+    announce("pinned_pool")
+    n, k = 40000, 16  # 2.5 MB of values: beyond the size that is served in place
+    rng = np.random.default_rng(31)
+    keys_np = unique_keys(rng, n)
+    pk, pv, po = capi.host_alloc(n * 8), capi.host_alloc(n * k * 4), capi.host_alloc(n * k * 4)
+    keys, vals, out = capi.host_array(pk, n, np.uint64), capi.host_array(pv, n * k, np.float32), \
+        capi.host_array(po, n * k, np.float32)
+    keys[:] = keys_np
+    t = capi.Table(capi.MODE_FIXED, initial_capacity=2 * n, row_len=k)
+    o = orc.Store(orc.MODE_FIXED, k)
+    for rep in range(3):
+        vals[:] = rng.standard_normal(n * k).astype(np.float32)
+        t.push(keys, vals)
+        o.push(keys_np, vals.copy())
+    out[:] = 7.0
+    assert t.pull(keys, out) == n * k
+    assert_bits_equal(out.copy(), o.pull(keys_np)[0], "pull into pinned memory")
+    # given back on another thread, the same buffers come out again (same size class)
+    th = threading.Thread(target=lambda: [capi.host_free(p) for p in (pv, po)])
+    th.start()
+    th.join()
+    again = {capi.host_alloc(n * k * 4), capi.host_alloc(n * k * 4 - 100)}
+    assert again == {pv, po}
+    # many threads allocating, writing and freeing at once: no buffer is handed out twice
+    seen, lock, errors = [], threading.Lock(), []
+
+    def churn(i):
+        try:
+            mine = []
+            for j in range(50):
+                p = capi.host_alloc(4096 * (1 + (i + j) % 5))
+                a = capi.host_array(p, 1024, np.uint32)
+                a[:] = i * 1000 + j
+                mine.append((p, i * 1000 + j))
+            for p, tag in mine:
+                assert np.all(capi.host_array(p, 1024, np.uint32) == tag), "a buffer was shared"
+            with lock:
+                seen.extend(p for p, _ in mine)
+            for p, _ in mine:
+                capi.host_free(p)
+        except BaseException as exc:  # noqa: BLE001
+            errors.append(repr(exc))
+
+    ths = [threading.Thread(target=churn, args=(i,)) for i in range(8)]
+    for th in ths:
+        th.start()
+    for th in ths:
+        th.join()
+    assert not errors, errors
+    for p in again | {pk}:
+        capi.host_free(p)
+    capi.host_free(0)          # null is ignored
+    capi.host_free(id(seen))   # an address the pool does not know is ignored
+    capi.host_trim()
+    capi.host_trim()           # nothing left: still fine
+    p = capi.host_alloc(1)
+    capi.host_array(p, 4096, np.uint8)[:] = 1
+    capi.host_free(p)
+    capi.host_trim()
+
+
 def test_device_time_accounting(capi, dev):
     """pskv_prof_*: every launch of the listed kernels is timed by its own pair of events; the samples
     add up to the total, and the copy probe moves what it says."""
