@@ -284,6 +284,42 @@ def test_pinned_pool(capi, orc, dev):
     capi.host_trim()
 
 
+@pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
+def test_dump_and_size_contract(capi, dev, mode):
+    """pskv_size counts keys and floats; pskv_dump with too little room answers PSKV_ESIZE_MISMATCH and
+    the sizes it needs, changes nothing, and works without the lens array."""
+    import ctypes
+    announce("dump_contract", mode)
+    m = {"scalar": capi.MODE_SCALAR, "fixed": capi.MODE_FIXED, "varlen": capi.MODE_VARLEN}[mode]
+    t = capi.Table(m, initial_capacity=16, row_len=3 if mode == "fixed" else 0)
+    assert t.size() == (0, 0)
+    assert [a.size for a in t.dump()] == [0, 0, 0]
+    keys = np.array([7, 1 << 40, KMAX - 1, KMAX], np.uint64)  # the last one lives in the side slot
+    lens = np.array([2, 0, 5, 1], np.int32)
+    per = {"scalar": [1, 1, 1, 1], "fixed": [3, 3, 3, 3], "varlen": lens.tolist()}[mode]
+    vals = np.arange(1, sum(per) + 1, dtype=np.float32)
+    t.push(keys, vals, lens if mode == "varlen" else None)
+    assert t.size() == (4, sum(per))
+    lib, h = capi.load(), t._h
+    nk, nv = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    k_small, v_small = np.zeros(3, np.uint64), np.zeros(sum(per), np.float32)
+    rc = lib.pskv_dump(h, k_small.ctypes.data, None, 3, v_small.ctypes.data, v_small.size,
+                       ctypes.byref(nk), ctypes.byref(nv))
+    assert rc == capi.ESIZE_MISMATCH and (nk.value, nv.value) == (4, sum(per))
+    k_ok, v_few = np.zeros(4, np.uint64), np.zeros(sum(per) - 1, np.float32)
+    rc = lib.pskv_dump(h, k_ok.ctypes.data, None, 4, v_few.ctypes.data, v_few.size,
+                       ctypes.byref(nk), ctypes.byref(nv))
+    assert rc == capi.ESIZE_MISMATCH and (nk.value, nv.value) == (4, sum(per))
+    v_ok = np.zeros(sum(per), np.float32)
+    rc = lib.pskv_dump(h, k_ok.ctypes.data, None, 4, v_ok.ctypes.data, v_ok.size, ctypes.byref(nk), ctypes.byref(nv))
+    assert rc == capi.OK and (nk.value, nv.value) == (4, sum(per))
+    assert k_ok.tolist() == keys.tolist()  # sorted by key, the side slot's key last
+    assert np.array_equal(v_ok, vals)      # 0.0f + v for every float, rows in key order
+    gk, gl, gv = t.dump()
+    assert gk.tolist() == keys.tolist() and gl.tolist() == per and np.array_equal(gv, vals)
+    assert t.size() == (4, sum(per))
+
+
 def test_device_time_accounting(capi, dev):
     """pskv_prof_*: every launch of the listed kernels is timed by its own pair of events; the samples
     add up to the total, and the copy probe moves what it says."""
