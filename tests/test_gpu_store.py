@@ -320,6 +320,38 @@ def test_dump_and_size_contract(capi, dev, mode):
     assert t.size() == (4, sum(per))
 
 
+def test_misuse_is_a_status_code(capi, dev):
+    """The C ABI never throws and never crashes on misuse: bad creation arguments, null handles and null
+    buffers come back as PSKV_EINVAL with a message."""
+    import ctypes
+    announce("misuse")
+    for kw in ({"mode": 7}, {"mode": -1}, {"max_load": 0.95}, {"max_load": -0.1}, {"device": 99}, {"device": -1}):
+        with pytest.raises(capi.PskvError) as e:
+            capi.Table(**kw)
+        assert e.value.code == capi.EINVAL, kw
+    lib = capi.load()
+    h = ctypes.c_void_p()
+    assert lib.pskv_table_create(ctypes.byref(h), None) == capi.EINVAL
+    assert lib.pskv_table_create(None, None) == capi.EINVAL
+    assert lib.pskv_table_destroy(None) == capi.OK
+    null = ctypes.c_void_p()
+    n1 = ctypes.c_size_t(0)
+    assert lib.pskv_push(null, None, 0, None, 0, None, 0, capi.MEM_HOST) == capi.EINVAL
+    assert lib.pskv_pull(null, None, 0, None, 0, None, ctypes.byref(n1), capi.MEM_HOST) == capi.EINVAL
+    assert lib.pskv_sync(null) == capi.EINVAL
+    assert b"null" in lib.pskv_last_error()
+    t = capi.Table(capi.MODE_SCALAR)
+    keys = np.array([1, 2, 3], np.uint64)
+    assert lib.pskv_push(t._h, None, 3, None, 3, None, 0, capi.MEM_HOST) == capi.EINVAL       # null keys
+    assert lib.pskv_push(t._h, keys.ctypes.data, 3, None, 3, None, 0, capi.MEM_HOST) == capi.EINVAL  # null vals
+    assert lib.pskv_push(t._h, keys.ctypes.data, 3, None, 3, None, 0, 5) == capi.EINVAL       # bad memkind
+    assert lib.pskv_pull(t._h, keys.ctypes.data, 3, None, 3, None, None, capi.MEM_HOST) == capi.EINVAL  # null out
+    assert lib.pskv_push(t._h, None, 0, None, 0, None, 0, capi.MEM_HOST) == capi.OK           # an empty request is fine
+    assert lib.pskv_pull(t._h, None, 0, None, 0, None, ctypes.byref(n1), capi.MEM_HOST) == capi.OK and n1.value == 0
+    assert lib.pskv_last_error() == b""  # a successful call clears the message
+    assert t.size() == (0, 0)
+
+
 def test_device_time_accounting(capi, dev):
     """pskv_prof_*: every launch of the listed kernels is timed by its own pair of events; the samples
     add up to the total, and the copy probe moves what it says."""
