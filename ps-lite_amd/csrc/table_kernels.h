@@ -15,9 +15,16 @@ namespace pskv {
 // ---------------------------------------------------------------------------------
 // SCALAR mode: one float per key, kept in the low word of the slot payload so that a
 // probe reads key and value with one 128-bit load.
-// One lane per key. Keys are unique within a request, so the value word of a slot is
-// only ever touched by the lane that owns the key: no atomics on values, and the
+// One lane per key. Keys are unique within a request (kv_app.h:17), so the value word of a
+// slot is only ever touched by the lane that owns the key: no atomics on values, and the
 // per-key sum order is the request order (requests are serialised on one stream).
+// The reference's handle is a plain loop over the request (kv_app.h:451-459), so even a
+// sorted request that repeats a key has a defined result there; it has the same result
+// here: the lane of the first occurrence serves the whole run in order, the other lanes of
+// the run stand back. Whether a lane starts or continues a run is read off the neighbouring
+// lanes' keys (a shuffle; only the first and the last lane of a wavefront look at memory), which
+// costs requests without repeats about 1 % of a push + pull step. An UNSORTED request that
+// repeats a key remains a caller error with an unspecified sum.
 // ---------------------------------------------------------------------------------
 template <bool PUSH, bool PULL>
 __global__ __launch_bounds__(kBlock) void k_scalar(Slot* __restrict__ slots, uint64_t mask,
@@ -28,8 +35,20 @@ __global__ __launch_bounds__(kBlock) void k_scalar(Slot* __restrict__ slots, uin
   __shared__ unsigned red[kBlock / 64];
   unsigned created = 0;
   const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
-    const uint64_t key = keys[i];
+  const unsigned lane = threadIdx.x & 63;
+  // whole wavefronts stay in the loop together: the shuffles below need every lane
+  for (uint64_t first = (uint64_t)blockIdx.x * kBlock; first < n; first += stride) {
+    const uint64_t i = first + threadIdx.x;
+    const bool live = i < n;
+    const uint64_t key = live ? keys[i] : 0;
+    uint64_t before = __shfl_up(key, 1);
+    uint64_t after = __shfl_down(key, 1);
+    // the first and the last lane look just outside the wavefront's 64 keys; their neighbours have
+    // fetched those lines already
+    if (lane == 0) before = (live && i > 0) ? keys[i - 1] : ~key;
+    if (lane == 63) after = (i + 1 < n) ? keys[i + 1] : ~key;
+    if (!live || (i > 0 && before == key)) continue;  // past the end, or inside a run
+    const bool run = i + 1 < n && after == key;
     float v = 0.0f;
     if (PUSH) v = vals[i];
     bool is_new;
@@ -39,8 +58,14 @@ __global__ __launch_bounds__(kBlock) void k_scalar(Slot* __restrict__ slots, uin
     // an absent key starts from Val() == 0, then `+=` (kv_app.h:454): 0.0f + v, not a copy
     float cur = is_new ? 0.0f : __uint_as_float((unsigned)seen);
     if (PUSH) cur = cur + v;
-    if (PUSH || is_new) *reinterpret_cast<float*>(p) = cur;
     if (PULL) out[i] = cur;
+    if (run) {  // the rest of the run, element by element like the reference's loop
+      for (uint64_t j = i + 1; j < n && keys[j] == key; ++j) {
+        if (PUSH) cur = cur + vals[j];
+        if (PULL) out[j] = cur;
+      }
+    }
+    if (PUSH || is_new) *reinterpret_cast<float*>(p) = cur;
     created += is_new ? 1u : 0u;
   }
   block_count_add(st, created, red);

@@ -600,10 +600,16 @@ def test_duplicate_keys_do_no_harm(capi, dev, mode):
     m = {"scalar": capi.MODE_SCALAR, "fixed": capi.MODE_FIXED, "varlen": capi.MODE_VARLEN}[mode]
     t = capi.Table(m, initial_capacity=16)
     if mode == "scalar":
+        # sorted repeats even have the reference's result, see test_scalar_sorted_repeats
         t.push(keys, np.ones(keys.size, np.float32))
         out = np.zeros(keys.size, np.float32)
         t.pull(keys, out)
-        assert t.size()[0] == 4  # which of the racing adds survives is unspecified
+        assert t.size()[0] == 4
+        assert np.array_equal(out, [1, 3, 3, 3, 2, 2, 1])
+        # unsorted repeats: which of the racing adds survives is unspecified, memory stays sound
+        mixed = np.array([9, 5, 9, 40, 5, 9, 77], np.uint64)
+        t.push(mixed, np.ones(mixed.size, np.float32))
+        assert t.size()[0] == 5
         return
     lens = np.full(keys.size, 8, np.int32)
     try:
@@ -619,6 +625,45 @@ def test_duplicate_keys_do_no_harm(capi, dev, mode):
     out = np.zeros(uniq.size * 8, np.float32)
     t.pull(uniq, out, np.zeros(uniq.size, np.int32) if mode == "varlen" else None)
     assert np.all(out >= 1.0)
+
+
+@pytest.mark.parametrize("memkind", ["device", "host"])
+@pytest.mark.parametrize("n", [7, 300, 100000])
+def test_scalar_sorted_repeats(capi, orc, dev, memkind, n):
+    """The reference's handle is a plain loop over the request (kv_app.h:451-459): a sorted request
+    that repeats a key adds the values in request order and every pulled position shows the sum so
+    far. Runs of every length, runs that cross wavefront and workgroup boundaries, a run at the very
+    start and one at the very end, through push, pull and push+pull."""
+    import torch
+    announce("scalar_sorted_repeats", memkind, n)
+    rng = np.random.default_rng(n)
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=16)
+    o = orc.Store(orc.MODE_SCALAR)
+    universe = unique_keys(rng, n)
+    for rep in range(5):
+        reps = rng.choice([1, 1, 1, 2, 3, 70, 300], size=n)
+        keys = np.sort(np.repeat(universe, reps)[:n] if rep % 2 == 0 else
+                       np.repeat(universe[::-1], reps)[-n:])
+        if rep == 4:
+            keys = np.full(n, universe[0], np.uint64)  # one run over the whole request
+        vals = rng.standard_normal(n).astype(np.float32)
+        want = o.handle(True, True, keys, vals, out_cap=n)[1]
+        if memkind == "device":
+            out = torch.full((n,), 7.0, dtype=torch.float32, device=dev)
+            t.pushpull(to_dev(keys, dev), to_dev(vals, dev), out)
+            t.sync()
+            got = from_dev(out)
+        else:
+            got = np.full(n, 7.0, np.float32)
+            t.pushpull(keys, vals, got)
+        assert_bits_equal(got, want, "push+pull %d" % rep)
+        vals = rng.standard_normal(n).astype(np.float32)
+        t.push(to_dev(keys, dev), to_dev(vals, dev)) if memkind == "device" else t.push(keys, vals)
+        o.push(keys, vals)
+        got = np.full(n, 7.0, np.float32)
+        t.pull(keys, got)
+        assert_bits_equal(got, o.pull(keys)[0], "pull %d" % rep)
+    _check_dump(t, o, "sorted repeats")
 
 
 @pytest.mark.parametrize("mode", ["fixed", "varlen"])
