@@ -50,6 +50,32 @@ def test_scalar_against_dict_model(orc):
     assert o.size() == (len(m.d), len(m.d))
 
 
+def test_scalar_request_that_repeats_keys(orc):
+    """The reference's handle is a loop over the request (kv_app.h:451-459), so a request that
+    repeats a key has a defined result: every occurrence adds, and with push+pull each position
+    shows the sum so far. Answer worked out by hand, then the dict model on random runs."""
+    o = orc.Store(orc.MODE_SCALAR)
+    keys = np.array([5, 9, 9, 9, 12, 12, 40], np.uint64)
+    rc, out, _, _ = o.handle(True, True, keys, np.ones(7, np.float32), out_cap=7)
+    assert rc == 0 and out.tolist() == [1, 1, 2, 3, 1, 2, 1]
+    rc, out, _, _ = o.handle(False, True, keys, out_cap=7)
+    assert rc == 0 and out.tolist() == [1, 3, 3, 3, 2, 2, 1]
+    rng = np.random.default_rng(2)
+    m = DictModel()
+    o = orc.Store(orc.MODE_SCALAR)
+    universe = unique_keys(rng, 200)
+    for it in range(30):
+        keys = np.sort(universe[rng.integers(0, universe.size, size=int(rng.integers(1, 900)))])
+        vals = rng.standard_normal(keys.size).astype(np.float32)
+        push, pull = [(True, False), (False, True), (True, True)][it % 3]
+        rc, out, _, _ = o.handle(push, pull, keys, vals if push else None, out_cap=keys.size)
+        want = m.handle(push, pull, keys, vals)
+        assert rc == 0
+        if pull:
+            assert_bits_equal(out, want, "op %d" % it)
+    assert_bits_equal(o.dump()[2], np.array([m.d[k] for k in sorted(m.d)], np.float32), "dump")
+
+
 def test_recorded_known_answers(orc):
     with open(KAT) as f:
         kat = json.load(f)
