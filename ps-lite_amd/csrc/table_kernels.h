@@ -23,8 +23,9 @@ namespace pskv {
 // here: the lane of the first occurrence serves the whole run in order, the other lanes of
 // the run stand back. Whether a lane starts or continues a run is read off the neighbouring
 // lanes' keys (a shuffle; only the first and the last lane of a wavefront look at memory), which
-// costs requests without repeats about 1 % of a push + pull step. An UNSORTED request that
-// repeats a key remains a caller error with an unspecified sum.
+// costs requests without repeats about 1 % of a push + pull step. One lane walks its run element
+// by element, so this is for the odd repeat, not a reduction of long runs. An UNSORTED request
+// that repeats a key remains a caller error with an unspecified sum.
 // ---------------------------------------------------------------------------------
 template <bool PUSH, bool PULL>
 __global__ __launch_bounds__(kBlock) void k_scalar(Slot* __restrict__ slots, uint64_t mask,
