@@ -55,30 +55,56 @@ constexpr int kCountShards = 32;
 constexpr int kShardStride = 16;  // in 8-byte words: one shard per 128-byte line
 constexpr int kTicketShards = 32;
 
-struct DevState {
-  unsigned long long arena_top;        // FIXED: rows handed out; VARLEN: 16-byte units handed out
-  unsigned long long special_payload;  // payload of key 2^64-1
-  unsigned long long scan_total;       // grand total of the last lens scan
-  unsigned int special_present;
-  unsigned int error;                  // sticky error bits of finished requests
-  unsigned int req_error;              // error bits of the request in flight
-  unsigned int misaligned;             // OR of (len & 3) over the lens of the current request
-  unsigned int req_flags;              // kReq* facts the workgroups of the kernel in flight have found
-  unsigned int ticket_top;             // second level of the last-workgroup ticket (ticket_last)
-  unsigned int pad0[2];
+struct alignas(32) DevState {
+  // The first 32 bytes are what a row kernel needs to know about its request (ReqFacts below):
+  // every wavefront reads them with one load.
   // "Same keys as the request that last filled the workspace" fast path of the row modes.
   // Every row-mode request has a number (epoch). cache_epoch is the request whose keys, lens,
   // row references, offsets and tile table the workspace and the key cache hold; bad_epoch ==
   // cache_epoch marks them unusable. same_epoch == e is the decision, reached once by the
   // compare kernel before anything else of request e runs, that e may reuse them.
+  unsigned long long same_epoch;
+  unsigned long long scan_total;       // grand total of the last lens scan
+  unsigned int error;                  // sticky error bits of finished requests
+  unsigned int req_error;              // error bits of the request in flight (follows `error`)
+  unsigned int misaligned;             // OR of (len & 3) over the lens of the current request
+  unsigned int req_flags;              // kReq* facts the workgroups of the kernel in flight have found
+  // 32
+  unsigned long long arena_top;        // FIXED: rows handed out; VARLEN: 16-byte units handed out
+  unsigned long long special_payload;  // payload of key 2^64-1
+  unsigned int special_present;
+  unsigned int ticket_top;             // second level of the last-workgroup ticket (ticket_last)
   unsigned long long cache_epoch;
   unsigned long long bad_epoch;
-  unsigned long long same_epoch;
+  unsigned long long pad0;
   // keys held (slot array plus the side slot) = sum of the shards
   unsigned long long count_shard[kCountShards * kShardStride];
   // first level of the last-workgroup ticket: one counter per 128-byte line
   unsigned int ticket_sub[kTicketShards * 32];
 };
+
+// The head of DevState as one load.
+struct ReqFacts {
+  unsigned long long same_epoch, scan_total;
+  unsigned int error, req_error, misaligned, req_flags;
+};
+static_assert(offsetof(DevState, same_epoch) == 0 && offsetof(DevState, scan_total) == 8 &&
+                  offsetof(DevState, error) == 16 && offsetof(DevState, req_error) == 20 &&
+                  offsetof(DevState, misaligned) == 24 && offsetof(DevState, req_flags) == 28,
+              "ReqFacts mirrors the head of DevState");
+typedef unsigned int u32x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ ReqFacts load_req_facts(const DevState* st) {
+  static_assert(sizeof(ReqFacts) == 32, "ReqFacts is the first 32 bytes of DevState");
+  const u32x8 w = *reinterpret_cast<const u32x8*>(st);
+  ReqFacts f;
+  f.same_epoch = ((unsigned long long)w[1] << 32) | w[0];
+  f.scan_total = ((unsigned long long)w[3] << 32) | w[2];
+  f.error = w[4];
+  f.req_error = w[5];
+  f.misaligned = w[6];
+  f.req_flags = w[7];
+  return f;
+}
 
 // Facts about the request that workgroups report into DevState::req_flags.
 constexpr unsigned kReqMisaligned = 3u;  // OR of (len & 3)

@@ -570,10 +570,38 @@ __device__ __forceinline__ void rows_tile_fixed(const RowsParams& p, uint64_t to
 // search the global arrays instead.
 constexpr unsigned kWaveSpan = 128;
 
+// What a wavefront can ask for knowing nothing but its tile index: the tile's shortcut note (read
+// even when it turns out not to be needed, so that it is not a second round trip after the
+// decision) and the request-side values. `bound` is what the host knows of the request's
+// length; the data may be shorter.
+template <int OP, int VEC, bool STREAM, unsigned WTILE>
+__device__ __forceinline__ void rows_wave_ask(const RowsParams& p, uint64_t bound,
+                                              typename VecT<VEC>::type* x, uint64_t& aff) {
+  using V = typename VecT<VEC>::type;
+  constexpr int kIter = WTILE / (VEC * 64);
+  const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint64_t wt = (uint64_t)blockIdx.x * (kBlock / 64) + wave;
+  const uint64_t f0 = wt * WTILE;
+  const uint64_t left = bound > f0 ? bound - f0 : 0;  // 0: the tile lies past the data
+  const uint32_t nelem = (uint32_t)(left < (uint64_t)WTILE ? left : (uint64_t)WTILE) / VEC;
+  aff = kTileNotAffine;
+  if (VEC == 4 && left) aff = p.tile_aff[wt];
+  if (OP == kOpAcc) {
+#pragma unroll
+    for (int i = 0; i < kIter; ++i) {
+      const uint32_t le = (uint32_t)i * 64 + lane;
+      x[i] = VecT<VEC>::zero();
+      if (le < nelem) x[i] = vload<STREAM>(reinterpret_cast<const V*>(p.req + f0 + le * VEC));
+    }
+  }
+}
+
+// `x` and `aff` come from rows_wave_ask; x[i] is used only below `total`.
 template <int OP, int VEC, bool STREAM, unsigned WTILE>
 __device__ __forceinline__ void rows_wave_varlen(const RowsParams& p, uint64_t total,
                                                  int32_t* s_off_all, uint64_t* s_ref_all,
-                                                 bool rejected, bool same) {
+                                                 bool rejected, bool same,
+                                                 const typename VecT<VEC>::type* x, uint64_t aff) {
   using V = typename VecT<VEC>::type;
   constexpr int kIter = WTILE / (VEC * 64);  // elements per lane
   static_assert(kIter >= 1 && kIter <= 8, "wave tile out of range");
@@ -583,24 +611,6 @@ __device__ __forceinline__ void rows_wave_varlen(const RowsParams& p, uint64_t t
   if (f0 >= total) return;  // the whole wavefront leaves; nothing below synchronises workgroups
   const uint32_t tile_floats = (uint32_t)((total - f0 < (uint64_t)WTILE) ? (total - f0) : (uint64_t)WTILE);
   const uint32_t nelem = tile_floats / VEC;
-
-  // Loads whose addresses depend on nothing but the tile index go first: the tile's shortcut
-  // note (read even when it turns out not to be needed, so that it is not a second round
-  // trip after the decision) and the request-side values.
-  uint64_t aff = kTileNotAffine;
-  if (VEC == 4) {
-    aff = p.tile_aff[wt];
-    asm volatile("" ::"v"((unsigned)aff), "v"((unsigned)(aff >> 32)));  // keep the load up here
-  }
-  V x[kIter];
-  if (OP == kOpAcc) {
-#pragma unroll
-    for (int i = 0; i < kIter; ++i) {
-      const uint32_t le = (uint32_t)i * 64 + lane;
-      x[i] = VecT<VEC>::zero();
-      if (le < nelem) x[i] = vload<STREAM>(reinterpret_cast<const V*>(p.req + f0 + le * VEC));
-    }
-  }
 
   // Shortcut of a request that repeats the cached one: if the rows of this tile lie back to
   // back in the arena, the tile maps to it with one offset and neither the row table nor a
@@ -741,28 +751,40 @@ __global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
   bool rejected = false;
   bool scalar = p.force_scalar != 0;
   uint64_t total = p.total;
-  // a request served from the cached references creates nothing and cannot have been refused
-  const bool same = cache_same(p.st, p.tag);
-  if (same) p.ignore_new = 1;
+  // What the device knows about the request: one load, one wait per wavefront.
+  const ReqFacts facts = load_req_facts(p.st);
   if (VARLEN) {
-    const unsigned err = same ? 0u : p.st->req_error;
+    // the grid covers the room in the caller's buffer, which may be more than the data
+    const uint64_t f0 = ((uint64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6)) * kTileVar;
+    if (f0 >= p.total) return;
+    // the loads that need no facts are on their way before the facts are looked at
+    f32x4 x4[kTileVar / 256];
+    uint64_t aff = kTileNotAffine;
+    if (!scalar) rows_wave_ask<OP, 4, STREAM, kTileVar>(p, p.total, x4, aff);
+    // a request served from the cached references creates nothing and cannot have been refused
+    const bool same = facts.same_epoch == p.tag.epoch;
+    if (same) p.ignore_new = 1;
+    const unsigned err = same ? 0u : facts.req_error;
     if (err & (kDevErrBadLen | kDevErrSizeMismatch)) return;
     rejected = (err & kDevErrLenChanged) != 0;
-    scalar = scalar || (p.st->misaligned != 0);
+    scalar = scalar || (facts.misaligned != 0);
     if (p.total_on_device) {
-      total = p.st->scan_total;
+      total = facts.scan_total;
       if (total > p.total) {  // the response does not fit the caller's buffer: write nothing
         if (blockIdx.x == 0 && threadIdx.x == 0) atomicOr(&p.st->error, kDevErrNoRoom);
         return;
       }
     }
-    // the grid may have been sized for the room in the caller's buffer, not for the data
     if (scalar) {
-      rows_wave_varlen<OP, 1, STREAM, kTileVar>(p, total, s_off, s_ref, rejected, same);
+      float x1[kTileVar / 64];
+      uint64_t none;
+      rows_wave_ask<OP, 1, STREAM, kTileVar>(p, total, x1, none);
+      rows_wave_varlen<OP, 1, STREAM, kTileVar>(p, total, s_off, s_ref, rejected, same, x1, none);
     } else {
-      rows_wave_varlen<OP, 4, STREAM, kTileVar>(p, total, s_off, s_ref, rejected, same);
+      rows_wave_varlen<OP, 4, STREAM, kTileVar>(p, total, s_off, s_ref, rejected, same, x4, aff);
     }
   } else {
+    if (facts.same_epoch == p.tag.epoch) p.ignore_new = 1;
     if (scalar) {
       rows_tile_fixed<OP, 1, STREAM, kTileFixed>(p, total);
     } else {
