@@ -28,6 +28,17 @@ constexpr uint64_t kLenMask = (1ull << kLenBits) - 1;
 // lie in the arena back to back, in request order and without padding, the whole tile maps to
 // the arena with one offset: the arena position (in floats) of the tile's first float.
 constexpr uint64_t kTileNotAffine = ~0ull;
+// The note a var-len row kernel leaves per tile for requests that repeat its request: where in
+// the arena the tile's floats lie when they form one or two unbroken pieces.
+//   first  = arena offset (floats) that the tile's float 0 maps to, or kTileNotAffine
+//   second = 0 for one piece; else (arena offset that float 0 would map to by the second
+//            piece's distance + kTileNoteBias) << kTileSplitBits | index of the first float
+//            of the second piece
+struct alignas(16) TileNote {
+  uint64_t first, second;
+};
+constexpr int kTileSplitBits = 10;
+constexpr int64_t kTileNoteBias = 1 << kTileSplitBits;  // keeps the second distance non-negative
 
 // sticky device-side error bits (DevState::error)
 constexpr unsigned kDevErrLenChanged = 1u;  // var-len push: stored length differs

@@ -118,7 +118,7 @@ struct pskv_table {
 
   GrowBuf ws;         // per-request workspace (row references, offsets)
   GrowBuf tiles;      // VARLEN: first key of every request-side tile
-  GrowBuf tiles_aff;  // VARLEN: arena offset of the tiles whose rows lie back to back
+  GrowBuf tiles_aff;  // VARLEN: one TileNote per tile
   char* small_in = nullptr;   // pinned, kSmallBytes: small host-resident requests, read in place
   char* small_out = nullptr;  // pinned, kSmallBytes: their responses, written in place
   GrowBuf stage;      // device copies of host-resident request buffers
@@ -530,7 +530,7 @@ int grow_tile_tables(pskv_table* t, uint64_t floats, uint64_t* ntiles_cap) {
   *ntiles_cap = (floats + kTileVar - 1) / kTileVar;
   int rc = grow(t, &t->tiles, (*ntiles_cap + 1) * sizeof(uint32_t));
   if (rc) return rc;
-  return grow(t, &t->tiles_aff, (*ntiles_cap + 1) * sizeof(uint64_t));
+  return grow(t, &t->tiles_aff, (*ntiles_cap + 1) * sizeof(TileNote));
 }
 
 // The kernels of a var-len request that work key by key: one workgroup per kBlock*items keys,
@@ -558,7 +558,7 @@ int make_tile_tables(pskv_table* t, const int32_t* lens_out, const unsigned long
               ntiles_cap, (uint64_t)kTileVar, (const DevState*)t->st, tag);
   PSKV_HIP(hipGetLastError());
   p->tile_key = tk;
-  p->tile_aff = static_cast<uint64_t*>(t->tiles_aff.ptr);
+  p->tile_aff = static_cast<TileNote*>(t->tiles_aff.ptr);
   return PSKV_OK;
 }
 
@@ -624,7 +624,7 @@ int run_varlen(pskv_table* t, Request& r) {
     t->cache_nvals = r.nvals;
     if (r.nvals) {
       p.tile_key = push_tile_key;
-      p.tile_aff = static_cast<uint64_t*>(t->tiles_aff.ptr);
+      p.tile_aff = static_cast<TileNote*>(t->tiles_aff.ptr);
       p.req = const_cast<float*>(r.vals);
       p.arena = t->arena;
       p.total = r.nvals;

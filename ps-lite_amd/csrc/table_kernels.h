@@ -10,6 +10,10 @@
 #include "device_common.h"
 #include "scan.h"
 
+#ifndef PSKV_ROWS_INLINE
+#define PSKV_ROWS_INLINE __forceinline__
+#endif
+
 namespace pskv {
 
 // ---------------------------------------------------------------------------------
@@ -442,7 +446,7 @@ struct RowsParams {
   const uint64_t* ref;       // n row references from the lookup kernel
   const uint64_t* off;       // VARLEN: n+1 request-side row offsets in floats
   const uint32_t* tile_key;  // VARLEN: ntiles+1 entries
-  uint64_t* tile_aff;        // VARLEN: ntiles entries (kTileNotAffine or the tile's arena offset)
+  TileNote* tile_aff;        // VARLEN: one note per tile
   DevState* st;
   uint64_t n;
   uint64_t total;         // floats in req
@@ -576,7 +580,7 @@ constexpr unsigned kWaveSpan = 128;
 // length; the data may be shorter.
 template <int OP, int VEC, bool STREAM, unsigned WTILE>
 __device__ __forceinline__ void rows_wave_ask(const RowsParams& p, uint64_t bound,
-                                              typename VecT<VEC>::type* x, uint64_t& aff) {
+                                              typename VecT<VEC>::type* x, TileNote& aff) {
   using V = typename VecT<VEC>::type;
   constexpr int kIter = WTILE / (VEC * 64);
   const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -584,8 +588,13 @@ __device__ __forceinline__ void rows_wave_ask(const RowsParams& p, uint64_t boun
   const uint64_t f0 = wt * WTILE;
   const uint64_t left = bound > f0 ? bound - f0 : 0;  // 0: the tile lies past the data
   const uint32_t nelem = (uint32_t)(left < (uint64_t)WTILE ? left : (uint64_t)WTILE) / VEC;
-  aff = kTileNotAffine;
-  if (VEC == 4 && left) aff = p.tile_aff[wt];
+  aff.first = kTileNotAffine;
+  aff.second = 0;
+  if (VEC == 4 && left) {
+    const u64x2 w = *reinterpret_cast<const u64x2*>(&p.tile_aff[wt]);  // one 128-bit load
+    aff.first = w.x;
+    aff.second = w.y;
+  }
   if (OP == kOpAcc) {
 #pragma unroll
     for (int i = 0; i < kIter; ++i) {
@@ -596,12 +605,56 @@ __device__ __forceinline__ void rows_wave_ask(const RowsParams& p, uint64_t boun
   }
 }
 
-// `x` and `aff` come from rows_wave_ask; x[i] is used only below `total`.
+// Shortcut of a request that repeats the cached one: if the rows of this tile lie in the arena
+// as one or two unbroken pieces (two: the tile straddles the rows of two workgroups of the
+// lookup that created them), the note the row kernel of the cached request left maps every
+// float with an offset and neither the row table nor a search is needed. Returns false when the
+// tile has to take the general way. Wavefront-uniform.
+template <int OP, bool STREAM, unsigned WTILE>
+__device__ __forceinline__ bool rows_wave_affine(const RowsParams& p, uint64_t total,
+                                                 const f32x4* x, const TileNote& aff) {
+  using V = f32x4;
+  constexpr int VEC = 4;
+  constexpr int kIter = WTILE / (VEC * 64);
+  static_assert(WTILE < (1u << kTileSplitBits), "the split index does not fit the note");
+  if (aff.first == kTileNotAffine) return false;
+  const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint64_t wt = (uint64_t)blockIdx.x * (kBlock / 64) + wave;
+  const uint64_t f0 = wt * WTILE;
+  if (f0 >= total) return true;
+  const uint32_t nelem = (uint32_t)((total - f0 < (uint64_t)WTILE) ? (total - f0) : (uint64_t)WTILE) / VEC;
+  // rows start on multiples of four floats here, so no 128-bit element straddles the split
+  const uint32_t split = aff.second ? (uint32_t)(aff.second & ((1u << kTileSplitBits) - 1)) : ~0u;
+  const int64_t first = (int64_t)aff.first;
+  const int64_t second = (int64_t)(aff.second >> kTileSplitBits) - kTileNoteBias;  // may be negative
+  V y[kIter];
+  V* dst[kIter];
+#pragma unroll
+  for (int i = 0; i < kIter; ++i) {
+    const uint32_t le = (uint32_t)i * 64 + lane;
+    dst[i] = reinterpret_cast<V*>(p.arena + ((le * VEC >= split ? second : first) + (int64_t)(le * VEC)));
+    y[i] = VecT<VEC>::zero();
+    if (le < nelem) y[i] = vload<STREAM>(dst[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < kIter; ++i) {
+    const uint32_t le = (uint32_t)i * 64 + lane;
+    if (le >= nelem) continue;
+    if (OP == kOpAcc) {
+      vstore<STREAM>(y[i] + x[i], dst[i]);
+    } else {
+      vstore<STREAM>(y[i], reinterpret_cast<V*>(p.req + f0 + le * VEC));
+    }
+  }
+  return true;
+}
+
+// `x` comes from rows_wave_ask; x[i] is used only below `total`.
 template <int OP, int VEC, bool STREAM, unsigned WTILE>
-__device__ __forceinline__ void rows_wave_varlen(const RowsParams& p, uint64_t total,
+__device__ PSKV_ROWS_INLINE void rows_wave_varlen(const RowsParams& p, uint64_t total,
                                                  int32_t* s_off_all, uint64_t* s_ref_all,
                                                  bool rejected, bool same,
-                                                 const typename VecT<VEC>::type* x, uint64_t aff) {
+                                                 const typename VecT<VEC>::type* x) {
   using V = typename VecT<VEC>::type;
   constexpr int kIter = WTILE / (VEC * 64);  // elements per lane
   static_assert(kIter >= 1 && kIter <= 8, "wave tile out of range");
@@ -611,34 +664,6 @@ __device__ __forceinline__ void rows_wave_varlen(const RowsParams& p, uint64_t t
   if (f0 >= total) return;  // the whole wavefront leaves; nothing below synchronises workgroups
   const uint32_t tile_floats = (uint32_t)((total - f0 < (uint64_t)WTILE) ? (total - f0) : (uint64_t)WTILE);
   const uint32_t nelem = tile_floats / VEC;
-
-  // Shortcut of a request that repeats the cached one: if the rows of this tile lie back to
-  // back in the arena, the tile maps to it with one offset and neither the row table nor a
-  // search is needed (wavefront-uniform branch). The table was written by the row kernel of
-  // the cached request, below.
-  if (VEC == 4 && same) {
-    if (aff != kTileNotAffine) {
-      V* base = reinterpret_cast<V*>(p.arena + aff);
-      V y[kIter];
-#pragma unroll
-      for (int i = 0; i < kIter; ++i) {
-        const uint32_t le = (uint32_t)i * 64 + lane;
-        y[i] = VecT<VEC>::zero();
-        if (le < nelem) y[i] = vload<STREAM>(base + le);
-      }
-#pragma unroll
-      for (int i = 0; i < kIter; ++i) {
-        const uint32_t le = (uint32_t)i * 64 + lane;
-        if (le >= nelem) continue;
-        if (OP == kOpAcc) {
-          vstore<STREAM>(y[i] + x[i], base + le);
-        } else {
-          vstore<STREAM>(y[i], reinterpret_cast<V*>(p.req + f0 + le * VEC));
-        }
-      }
-      return;
-    }
-  }
 
   const uint64_t j_lo = p.tile_key[wt];
   const uint32_t span = (uint32_t)((uint64_t)p.tile_key[wt + 1] - j_lo + 1);
@@ -656,23 +681,57 @@ __device__ __forceinline__ void rows_wave_varlen(const RowsParams& p, uint64_t t
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
   if (!same) {
-    // Leave a note for requests that repeat this one: the tile is "affine" when every row
-    // with floats in it sits at the same distance from its place in the request, i.e. the
-    // rows lie back to back, in request order, without padding between them.
-    uint64_t note = kTileNotAffine;
+    // Leave a note for requests that repeat this one. Every row with floats in the tile has a
+    // distance between its place in the arena and its place in the request; the tile is one
+    // piece when all distances are equal (the rows lie back to back, in request order, without
+    // padding between them) and two pieces when they change once.
+    TileNote note = {kTileNotAffine, 0};
     if (VEC == 4 && staged) {
-      const uint64_t r0 = s_ref[0];
-      const int64_t d0 = (int64_t)(((r0 & ~kRefNew) >> kLenBits) << 2) - (int64_t)s_off[0];
-      bool bad = r0 == kRefAbsent;
-      for (uint32_t s = lane; s < span; s += 64) {
-        const bool has_floats = s_off[s + 1] > s_off[s] && s_off[s] < (int32_t)tile_floats;
-        if (has_floats) {
+      bool absent = false;
+      int64_t d[(kWaveSpan + 63) / 64];
+      bool has[(kWaveSpan + 63) / 64];
+#pragma unroll
+      for (uint32_t it = 0; it < (kWaveSpan + 63) / 64; ++it) {
+        const uint32_t s = it * 64 + lane;
+        has[it] = s < span && s_off[s + 1] > s_off[s] && s_off[s] < (int32_t)tile_floats;
+        d[it] = 0;
+        if (has[it]) {
           const uint64_t r = s_ref[s];
-          const int64_t d = (int64_t)(((r & ~kRefNew) >> kLenBits) << 2) - (int64_t)s_off[s];
-          bad |= r == kRefAbsent || d != d0;
+          absent |= r == kRefAbsent;
+          d[it] = (int64_t)(((r & ~kRefNew) >> kLenBits) << 2) - (int64_t)s_off[s];
         }
       }
-      if (__ballot(bad) == 0ull) note = (uint64_t)d0;
+      // the first row with floats, its distance, and the first row whose distance differs
+      uint32_t s0 = ~0u, s1 = ~0u;
+#pragma unroll
+      for (uint32_t it = 0; it < (kWaveSpan + 63) / 64; ++it) {
+        const uint64_t m = __ballot(has[it]);
+        if (s0 == ~0u && m) s0 = it * 64 + (uint32_t)__builtin_ctzll(m);
+      }
+      if (s0 != ~0u && __ballot(absent) == 0ull) {
+        const uint64_t r0 = s_ref[s0];
+        const int64_t d0 = (int64_t)(((r0 & ~kRefNew) >> kLenBits) << 2) - (int64_t)s_off[s0];
+#pragma unroll
+        for (uint32_t it = 0; it < (kWaveSpan + 63) / 64; ++it) {
+          const uint64_t m = __ballot(has[it] && d[it] != d0);
+          if (s1 == ~0u && m) s1 = it * 64 + (uint32_t)__builtin_ctzll(m);
+        }
+        if (s1 == ~0u) {
+          note.first = (uint64_t)d0;
+        } else {
+          const uint64_t r1 = s_ref[s1];
+          const int32_t at = s_off[s1];  // > 0: row s0 comes first and has floats in the tile
+          const int64_t d1 = (int64_t)(((r1 & ~kRefNew) >> kLenBits) << 2) - (int64_t)at;
+          bool other = false;
+#pragma unroll
+          for (uint32_t it = 0; it < (kWaveSpan + 63) / 64; ++it)
+            other |= has[it] && it * 64 + lane > s1 && d[it] != d1;
+          if (__ballot(other) == 0ull && at > 0) {
+            note.first = (uint64_t)d0;
+            note.second = ((uint64_t)(d1 + kTileNoteBias) << kTileSplitBits) | (uint64_t)(uint32_t)at;
+          }
+        }
+      }
     }
     if (lane == 0) p.tile_aff[wt] = note;
   }
@@ -759,7 +818,7 @@ __global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
     if (f0 >= p.total) return;
     // the loads that need no facts are on their way before the facts are looked at
     f32x4 x4[kTileVar / 256];
-    uint64_t aff = kTileNotAffine;
+    TileNote aff = {kTileNotAffine, 0};
     if (!scalar) rows_wave_ask<OP, 4, STREAM, kTileVar>(p, p.total, x4, aff);
     // a request served from the cached references creates nothing and cannot have been refused
     const bool same = facts.same_epoch == p.tag.epoch;
@@ -777,11 +836,15 @@ __global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
     }
     if (scalar) {
       float x1[kTileVar / 64];
-      uint64_t none;
+      TileNote none;
       rows_wave_ask<OP, 1, STREAM, kTileVar>(p, total, x1, none);
-      rows_wave_varlen<OP, 1, STREAM, kTileVar>(p, total, s_off, s_ref, rejected, same, x1, none);
+      rows_wave_varlen<OP, 1, STREAM, kTileVar>(p, total, s_off, s_ref, rejected, same, x1);
     } else {
-      rows_wave_varlen<OP, 4, STREAM, kTileVar>(p, total, s_off, s_ref, rejected, same, x4, aff);
+      if (same && rows_wave_affine<OP, STREAM, kTileVar>(p, total, x4, aff)) return;
+#ifdef PSKV_EXP_NOGENERAL
+      if (same) return;  // timing experiment only: tiles without a note are skipped
+#endif
+      rows_wave_varlen<OP, 4, STREAM, kTileVar>(p, total, s_off, s_ref, rejected, same, x4);
     }
   } else {
     if (facts.same_epoch == p.tag.epoch) p.ignore_new = 1;
