@@ -50,7 +50,7 @@ SAMPLE_EVERY = 4  # MI355X HBM3E, published
 TRAFFIC = {
     ("push_scalar", 250000): 60.1e6, ("pull_scalar", 250000): 35.5e6,
     ("rows_acc_fixed", 268435456): 3.0 * 2**30, ("rows_gather_fixed", 268435456): 2.0 * 2**30,
-    ("rows_acc_varlen", 6192336): 76.4e6, ("rows_gather_varlen", 6192336): 50.9e6,
+    ("rows_acc_varlen", 6192336): 76.1e6, ("rows_gather_varlen", 6192336): 50.6e6,
 }
 
 
