@@ -10,10 +10,6 @@
 #include "device_common.h"
 #include "scan.h"
 
-#ifndef PSKV_ROWS_INLINE
-#define PSKV_ROWS_INLINE __forceinline__
-#endif
-
 namespace pskv {
 
 // ---------------------------------------------------------------------------------
@@ -651,7 +647,7 @@ __device__ __forceinline__ bool rows_wave_affine(const RowsParams& p, uint64_t t
 
 // `x` comes from rows_wave_ask; x[i] is used only below `total`.
 template <int OP, int VEC, bool STREAM, unsigned WTILE>
-__device__ PSKV_ROWS_INLINE void rows_wave_varlen(const RowsParams& p, uint64_t total,
+__device__ __forceinline__ void rows_wave_varlen(const RowsParams& p, uint64_t total,
                                                  int32_t* s_off_all, uint64_t* s_ref_all,
                                                  bool rejected, bool same,
                                                  const typename VecT<VEC>::type* x) {
@@ -841,9 +837,6 @@ __global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
       rows_wave_varlen<OP, 1, STREAM, kTileVar>(p, total, s_off, s_ref, rejected, same, x1);
     } else {
       if (same && rows_wave_affine<OP, STREAM, kTileVar>(p, total, x4, aff)) return;
-#ifdef PSKV_EXP_NOGENERAL
-      if (same) return;  // timing experiment only: tiles without a note are skipped
-#endif
       rows_wave_varlen<OP, 4, STREAM, kTileVar>(p, total, s_off, s_ref, rejected, same, x4);
     }
   } else {
