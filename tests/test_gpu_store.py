@@ -591,6 +591,63 @@ def test_varlen_pull_without_host_round_trip(capi, orc, dev):
     _check_dump(t, o, "after async pulls")
 
 
+@pytest.mark.parametrize("memkind", ["device", "host"])
+@pytest.mark.parametrize("nkeys,row", [(40, 24), (3000, 8), (9000, 72)])
+def test_varlen_tiles_in_two_arena_pieces(capi, orc, dev, memkind, nkeys, row):
+    """A request that repeats the cached one maps a 256-float tile through the note its predecessor
+    left: one arena piece, or two. Here the upper half of the keys is created first and the lower
+    half second, so in a request over all keys the tile around the middle lies in two pieces and
+    the second piece sits BELOW the first in the arena (a negative distance); further pieces come
+    from the lookup's workgroups. Pushes and pulls that repeat that request must give the
+    oracle's sums; then a changed length in the middle must end the shortcut."""
+    import torch
+    announce("varlen_two_pieces", memkind, nkeys, row)
+    rng = np.random.default_rng(nkeys + row)
+    keys = unique_keys(rng, nkeys)
+    lens = np.full(nkeys, row, np.int32)
+    lens[rng.integers(0, nkeys, size=nkeys // 10)] = 0      # rows without floats in between
+    lens[rng.integers(0, nkeys, size=nkeys // 10)] = 4 * row
+    half = nkeys // 2
+    t = capi.Table(capi.MODE_VARLEN, initial_capacity=64)
+    o = orc.Store(orc.MODE_VARLEN)
+
+    def push(k, l):
+        v = rng.integers(-8, 8, size=int(l.sum())).astype(np.float32)
+        if memkind == "device":
+            t.push(to_dev(k, dev), to_dev(v, dev), to_dev(l, dev))
+        else:
+            t.push(k, v, l)
+        o.push(k, v, l)
+
+    def pull_and_check(k, what):
+        want, want_lens = o.pull(k)
+        got = np.full(want.size, 7.0, np.float32)
+        got_lens = np.full(k.size, -1, np.int32)
+        if memkind == "device":
+            out = torch.full((want.size,), 7.0, dtype=torch.float32, device=dev)
+            out_lens = torch.full((k.size,), -1, dtype=torch.int32, device=dev)
+            t.pull(to_dev(k, dev), out, out_lens)
+            t.sync()
+            got, got_lens = from_dev(out), from_dev(out_lens)
+        else:
+            t.pull(k, got, got_lens)
+        assert np.array_equal(got_lens, want_lens), what
+        assert_bits_equal(got, want, what)
+
+    push(keys[half:], lens[half:])
+    push(keys[:half], lens[:half])
+    for rep in range(4):          # the first writes the notes, the others use them
+        push(keys, lens)
+        pull_and_check(keys, "repeat %d" % rep)
+    pull_and_check(keys, "pull again")
+    sub = keys[half - 5:half + 5]
+    push(sub, lens[half - 5:half + 5])
+    for rep in range(2):
+        push(keys, lens)
+        pull_and_check(keys, "after another request %d" % rep)
+    _check_dump(t, o, "two pieces")
+
+
 @pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
 def test_duplicate_keys_do_no_harm(capi, dev, mode):
     """Keys of a request must be unique (kv_app.h:17). A request that repeats a key is a caller error:
