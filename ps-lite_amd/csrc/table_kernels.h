@@ -809,6 +809,12 @@ __global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
   // What the device knows about the request: one load, one wait per wavefront.
   const ReqFacts facts = load_req_facts(p.st);
   if (VARLEN) {
+    // every argument the common path uses, asked for at once (the compiler otherwise fetches them
+    // group by group where they are first used, one wait each)
+    asm volatile("" ::"s"(p.req), "s"(p.arena), "s"(p.tile_aff), "s"(p.total),
+                 "s"(p.force_scalar), "s"(p.total_on_device), "s"(p.tag.epoch));
+  }
+  if (VARLEN) {
     // the grid covers the room in the caller's buffer, which may be more than the data
     const uint64_t f0 = ((uint64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6)) * kTileVar;
     if (f0 >= p.total) return;
