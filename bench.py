@@ -107,8 +107,10 @@ def kernel_stats(tables, kernel):
 def roofline(alg_bytes_per_launch, launches, total_ms, traffic=None, samples=None):
     """`achieved` is algorithmic bytes over the AVERAGE launch duration; the median and the
     minimum over the launches are given beside it."""
-    avg_s = total_ms / launches * 1e-3 if launches else float("nan")
-    achieved = alg_bytes_per_launch / avg_s / 1e9 if launches else 0.0
+    if not launches:
+        raise RuntimeError("no timed launch of the kernel: its events were switched off")
+    avg_s = total_ms / launches * 1e-3
+    achieved = alg_bytes_per_launch / avg_s / 1e9
     r = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
          "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
          "launches": launches, "avg_us": round(avg_s * 1e6, 2),
@@ -312,8 +314,10 @@ def measure_dense(capi, dev, steps, warmup, nk=64, k=4194304):
     assert torch.equal(out[idx], ref), "dense sums differ from sequential float adds"
     # plain copies of the same 1 GiB: the known-size launch that memory-traffic counters are
     # scaled by, and the copy ceiling of this GPU next to the accumulate kernel
+    t.prof_enable(True)  # the last timed step may have left the events off
     for _ in range(3):
         t.copy_probe(out, vals)
+    t.sync()
     cp = kernel_stats([t], capi.KERNEL_COPY)
     t.prof_enable(False)
     t.close()
@@ -688,7 +692,7 @@ def main():
         extra["own_streams"] = res["own_streams"]
     if extra:
         line["extra"] = extra
-    print(json.dumps(line), flush=True)
+    print(json.dumps(line, allow_nan=False), flush=True)  # strict JSON: a NaN would be a bug
 
 
 if __name__ == "__main__":
