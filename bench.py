@@ -93,6 +93,12 @@ def to_dev(a, dev):
     return torch.from_numpy(a).to(dev)
 
 
+def sampled(j, steps):
+    """Whether timed step j (0-based) is one whose launches carry events: every SAMPLE_EVERY-th,
+    and no more than a quarter of a short run (but the first step always)."""
+    return j >= 0 and j % SAMPLE_EVERY == 0 and j // SAMPLE_EVERY < max(1, steps // SAMPLE_EVERY)
+
+
 def kernel_stats(tables, kernel):
     """(launches, summed ms, per-launch ms) of one kernel over several tables."""
     n, ms, samples = 0, 0.0, []
@@ -160,7 +166,7 @@ def run_sparse_lr(args, capi, dev):
         if sample:
             j = i - args.warmup
             for s in range(S):
-                tables[s].prof_enable(j >= 0 and j % SAMPLE_EVERY == 0 and s == (j // SAMPLE_EVERY) % S)
+                tables[s].prof_enable(sampled(j, args.steps) and s == (j // SAMPLE_EVERY) % S)
         dk, dv = d_batches[i]
         kp, vp, op = dk.data_ptr(), dv.data_ptr(), out.data_ptr()
         pos, _, used = capi.slice_keys(dk, rb, re, nvals=n)
@@ -298,7 +304,7 @@ def measure_dense(capi, dev, steps, warmup, nk=64, k=4194304):
     t.prof_reset()
     t0 = time.perf_counter()
     for i in range(steps):
-        t.prof_enable(i % SAMPLE_EVERY == 0)
+        t.prof_enable(sampled(i, steps))
         t.push(keys, vals)
         t.pull(keys, out)
     t.sync()
@@ -419,7 +425,7 @@ def run_varlen(args, capi, dev):
         # kernel durations are sampled inside the timed steps: in every SAMPLE_EVERY-th step the
         # launches of one table, taken in turn, carry their own events
         for s in range(S):
-            tables[s].prof_enable(i % SAMPLE_EVERY == 0 and s == (i // SAMPLE_EVERY) % S)
+            tables[s].prof_enable(sampled(i, args.steps) and s == (i // SAMPLE_EVERY) % S)
         step()
     drain()
     dt = time.perf_counter() - t0
