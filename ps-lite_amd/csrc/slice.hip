@@ -16,17 +16,12 @@ namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-// One wavefront per search target: a 64-ary lower_bound. Each round the 64 lanes probe
-// evenly spaced keys of the remaining interval, a ballot counts how many are below
-// the target (the probes are sorted, so the votes are a prefix of ones) and the
-// interval shrinks 64-fold: ceil(log64 n) dependent loads instead of ceil(log2 n).
-__global__ __launch_bounds__(kBlock) void k_bounds(const uint64_t* __restrict__ keys, uint64_t n,
-                                                  const uint64_t* __restrict__ targets,
-                                                  uint64_t ntargets, uint64_t* __restrict__ lb) {
-  const uint64_t w = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
-  const unsigned lane = threadIdx.x & 63;
-  if (w >= ntargets) return;  // whole wavefronts leave together
-  const uint64_t target = targets[w];
+// A 64-ary lower_bound by one wavefront. Each round the 64 lanes probe evenly spaced keys of
+// the remaining interval, a ballot counts how many are below the target (the probes are
+// sorted, so the votes are a prefix of ones) and the interval shrinks 64-fold:
+// ceil(log64 n) dependent loads instead of ceil(log2 n). Every lane returns the answer.
+__device__ __forceinline__ uint64_t wave_lower_bound(const uint64_t* __restrict__ keys, uint64_t n,
+                                                     uint64_t target, unsigned lane) {
   uint64_t lo = 0, hi = n;  // the answer lies in [lo, hi]; keys[lo..hi) are undecided
   while (hi > lo) {
     const uint64_t len = hi - lo;
@@ -45,6 +40,17 @@ __global__ __launch_bounds__(kBlock) void k_bounds(const uint64_t* __restrict__ 
     hi = cap < hi ? cap : hi;
     lo = new_lo < hi ? new_lo : hi;
   }
+  return lo;
+}
+
+// One wavefront per search target.
+__global__ __launch_bounds__(kBlock) void k_bounds(const uint64_t* __restrict__ keys, uint64_t n,
+                                                  const uint64_t* __restrict__ targets,
+                                                  uint64_t ntargets, uint64_t* __restrict__ lb) {
+  const uint64_t w = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
+  const unsigned lane = threadIdx.x & 63;
+  if (w >= ntargets) return;  // whole wavefronts leave together
+  const uint64_t lo = wave_lower_bound(keys, n, targets[w], lane);
   if (lane == 0) lb[w] = lo;
 }
 
@@ -66,6 +72,38 @@ __global__ void k_bounds_chain(const uint64_t* __restrict__ lb, uint64_t S,
   pos_host[0] = p;
   for (uint64_t i = 0; i < S; ++i) {
     const uint64_t e = lb[i + 1];
+    p = e > p ? e : p;
+    pos[i + 1] = p;
+    pos_host[i + 1] = p;
+  }
+}
+
+// Both of the above in one launch when the boundaries are few (the stock case: one per server):
+// one workgroup of up to 16 wavefronts, each searching one or two boundaries, then the chain.
+// The boundaries travel with the launch: no read across the host link before the search.
+constexpr unsigned kFusedWaves = 16;
+constexpr unsigned kFusedTargets = 2 * kFusedWaves;
+struct FusedTargets {
+  uint64_t v[kFusedTargets];
+};
+__global__ __launch_bounds__(kFusedWaves * 64) void k_bounds_fused(
+    const uint64_t* __restrict__ keys, uint64_t n, FusedTargets targets, uint64_t S,
+    uint64_t* __restrict__ pos, uint64_t* __restrict__ pos_host, unsigned long long* __restrict__ sums) {
+  __shared__ uint64_t s_lb[kFusedTargets];
+  const unsigned lane = threadIdx.x & 63, waves = blockDim.x >> 6;
+  for (unsigned w = threadIdx.x >> 6; w <= S; w += waves) {  // whole wavefronts
+    const uint64_t lo = wave_lower_bound(keys, n, targets.v[w], lane);
+    if (lane == 0) s_lb[w] = lo;
+  }
+  __syncthreads();
+  if (sums)
+    for (uint64_t i = threadIdx.x; i < S; i += blockDim.x) sums[i] = 0ull;
+  if (threadIdx.x != 0) return;
+  uint64_t p = s_lb[0];
+  pos[0] = p;
+  pos_host[0] = p;
+  for (uint64_t i = 0; i < S; ++i) {
+    const uint64_t e = s_lb[i + 1];
     p = e > p ? e : p;
     pos[i + 1] = p;
     pos_host[i + 1] = p;
@@ -332,10 +370,19 @@ int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, 
     }
     h_targets[0] = range_begin[0];
     for (size_t i = 0; i < S; ++i) h_targets[i + 1] = range_end[i];
-    rc = launch_bounds_search(d_keys, n, h_targets, S + 1, d_lb, c->stream);
-    if (rc) return rc;
-    k_bounds_chain<<<dim3(1), dim3(64), 0, c->stream>>>(d_lb, S, d_pos, h_pos, do_sums ? d_sums : nullptr);
-    PSKV_HIP(hipGetLastError());
+    if (S + 1 <= kFusedTargets) {  // one launch for the boundaries when they are few
+      FusedTargets ft = {};
+      for (size_t i = 0; i <= S; ++i) ft.v[i] = h_targets[i];
+      const unsigned waves = (unsigned)std::min<size_t>(S + 1, kFusedWaves);
+      k_bounds_fused<<<dim3(1), dim3(waves * 64), 0, c->stream>>>(d_keys, n, ft, S, d_pos, h_pos,
+                                                                 do_sums ? d_sums : nullptr);
+      PSKV_HIP(hipGetLastError());
+    } else {
+      rc = launch_bounds_search(d_keys, n, h_targets, S + 1, d_lb, c->stream);
+      if (rc) return rc;
+      k_bounds_chain<<<dim3(1), dim3(64), 0, c->stream>>>(d_lb, S, d_pos, h_pos, do_sums ? d_sums : nullptr);
+      PSKV_HIP(hipGetLastError());
+    }
     if (do_sums) {
       uint64_t per = n / S / (kBlock * 8) + 1;
       if (per > 1024) per = 1024;
