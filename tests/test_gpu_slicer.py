@@ -26,7 +26,7 @@ def _compare(capi, orc, keys, rb, re, lens, nvals, dev, memkind):
 
 
 @pytest.mark.parametrize("memkind", ["device", "host"])
-@pytest.mark.parametrize("n,S", [(0, 4), (1, 1), (63, 3), (64, 4), (65, 16), (4096, 7), (4097, 64),
+@pytest.mark.parametrize("n,S", [(0, 4), (1, 1), (63, 3), (64, 4), (65, 16), (4096, 7), (4097, 64), (5000, 31), (5000, 32),
                                  (100000, 4), (262145, 16), (1000003, 1), (2000000, 16)])
 def test_slice_uniform(capi, orc, dev, memkind, n, S):
     announce("slice_uniform", memkind, n, S)
