@@ -78,3 +78,13 @@ def test_product_never_touches_the_oracle():
                     assert "pskv_oracle" not in text and "liboracle" not in text, os.path.join(dirpath, f)
                     if f != "build.py":
                         assert "oracle" not in text.lower() or f == "build.py", os.path.join(dirpath, f)
+
+
+def test_bench_measures_one_gpu_only():
+    """A table lives on one device; asked for more GPUs the benchmark says so and stops."""
+    import sys
+    p = subprocess.run([sys.executable, os.path.join(REPO, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert p.returncode != 0
+    assert "ONE GPU" in (p.stdout + p.stderr)
+    assert not p.stdout.strip().startswith("{")  # no result line
