@@ -11,7 +11,8 @@
  *                           (kv_app.h:440-463); install with
  *                           KVServer::set_request_handle (kv_app.h:417-420).
  *
- * Include either the real library ("ps/ps.h") or "pskv/ps_min.h" BEFORE this header;
+ * Include the real library ("ps/ps.h") BEFORE this header (the tests of this repository
+ * include their in-process stand-in, tests/include/pskv/ps_min.h, instead);
  * it only uses names both provide (ps::KVPairs, ps::KVMeta, ps::KVServer,
  * ps::KVWorker, ps::Range, ps::SArray, dmlc::Error).
  *

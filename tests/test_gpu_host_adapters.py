@@ -9,13 +9,13 @@ from conftest import REPO, announce
 
 pytestmark = pytest.mark.gpu
 
-BIN = os.path.join(REPO, "ps-lite_amd", "host", "test_kv_app_gpu")
+BIN = os.path.join(REPO, "tests", "test_kv_app_gpu")
 
 
 @pytest.mark.parametrize("num_servers", [1, 2, 4])
 def test_kv_app_through_adapters(num_servers):
     announce("kv_app_through_adapters", num_servers)
-    assert os.path.exists(BIN), "build() compiles ps-lite_amd/host/test_kv_app_gpu"
+    assert os.path.exists(BIN), "build() compiles tests/test_kv_app_gpu"
     r = subprocess.run([BIN, str(num_servers)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
                        text=True, timeout=100)
     print(r.stdout)
