@@ -139,6 +139,29 @@ int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, 
                size_t nvals, const uint64_t* range_begin, const uint64_t* range_end, size_t S,
                uint64_t* pos, uint64_t* val_pos, uint8_t* used, int memkind);
 
+/* pskv_slice for callers that cannot allocate. It has no counterpart in the reference: it is
+ * for code that may not call hipMalloc (under HIP graph capture, in tight serving loops, in
+ * harnesses that forbid it). It allocates nothing and waits for nothing: the kernels are
+ * enqueued on `stream` (a hipStream_t, NULL = the null stream) and their working memory (the
+ * lower bounds of the searches and the per-slice sums of lens) is a fixed array inside the
+ * library's code object, which every GPU that loads the library holds until the process ends
+ * (about 16 KiB); that bounds S by PSKV_SLICE_NOALLOC_MAX_RANGES.
+ * keys/lens are device memory on `device`; range_begin/range_end are host arrays, read before
+ * the call returns; pos[S+1], val_pos[S+1], used[S] and status[1] are DEVICE memory, valid once
+ * the stream has run the call. *status receives what pskv_slice would have returned for the
+ * data-dependent outcomes (PSKV_OK, PSKV_EUNCOVERED_KEY, PSKV_ESIZE_MISMATCH); on a non-zero
+ * status val_pos is unspecified. What the host can decide alone (null arguments, no range or
+ * too many, a gap between ranges) is returned at once and nothing is enqueued.
+ * All calls on one GPU share the one array: calls that overlap in time on a GPU (different
+ * streams, or several threads) race; put them on one stream or order them with events.
+ * The first call on a device looks the array's address up in the runtime: make it outside any
+ * graph capture (a call with n = 0 will do). */
+#define PSKV_SLICE_NOALLOC_MAX_RANGES 1024
+int pskv_slice_noalloc(int device, void* stream, const uint64_t* keys, size_t n, const int32_t* lens,
+                       size_t nlens, size_t nvals, const uint64_t* range_begin,
+                       const uint64_t* range_end, size_t S, uint64_t* pos, uint64_t* val_pos,
+                       uint8_t* used, int32_t* status);
+
 /* Postoffice::GetServerKeyRanges (src/postoffice.cc:169-180) for num_servers
  * servers; host arrays of num_servers entries each. */
 int pskv_server_ranges(uint64_t num_servers, uint64_t* range_begin, uint64_t* range_end);

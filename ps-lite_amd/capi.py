@@ -25,6 +25,7 @@ MODE_SCALAR = 0
 MODE_FIXED = 1
 MODE_VARLEN = 2
 MAX_VARLEN_ROW = (1 << 28) - 1
+SLICE_NOALLOC_MAX_RANGES = 1024
 KERNEL_PUSH_SCALAR, KERNEL_PULL_SCALAR, KERNEL_ROWS_ACC, KERNEL_ROWS_GATHER, KERNEL_LOOKUP, \
     KERNEL_REHASH, KERNEL_COPY = range(7)
 
@@ -37,7 +38,7 @@ ERROR_NAMES = {
 # every symbol include/pskv/capi.h declares
 SYMBOLS = [
     "pskv_table_create", "pskv_table_destroy", "pskv_push", "pskv_pull", "pskv_pushpull",
-    "pskv_sync", "pskv_size", "pskv_dump", "pskv_slice", "pskv_server_ranges",
+    "pskv_sync", "pskv_size", "pskv_dump", "pskv_slice", "pskv_slice_noalloc", "pskv_server_ranges",
     "pskv_assemble_pull", "pskv_prof_enable", "pskv_prof_reset", "pskv_prof_read", "pskv_prof_samples",
     "pskv_copy_probe", "pskv_host_alloc", "pskv_host_free", "pskv_host_trim", "pskv_last_error",
     "pskv_version",
@@ -86,6 +87,7 @@ def load():
     lib.pskv_size.argtypes = [vp, ctypes.POINTER(u64), ctypes.POINTER(u64)]
     lib.pskv_dump.argtypes = [vp, vp, vp, sz, vp, sz, ctypes.POINTER(sz), ctypes.POINTER(sz)]
     lib.pskv_slice.argtypes = [i32, vp, sz, vp, sz, sz, vp, vp, sz, vp, vp, vp, i32]
+    lib.pskv_slice_noalloc.argtypes = [i32, vp, vp, sz, vp, sz, sz, vp, vp, sz, vp, vp, vp, vp]
     lib.pskv_server_ranges.argtypes = [u64, vp, vp]
     lib.pskv_assemble_pull.argtypes = [i32, vp, sz, sz, vp, vp, vp, vp, vp, vp, sz, vp,
                                        ctypes.POINTER(sz), i32]
@@ -269,6 +271,19 @@ def slice_keys(keys, range_begin, range_end, lens=None, nvals=0, device=0):
                              pos.ctypes.data, val_pos.ctypes.data, used.ctypes.data,
                              _memkind(k1, k2)))
     return pos, val_pos, used[:S]
+
+
+def slice_keys_noalloc(keys, range_begin, range_end, pos, val_pos, used, status, lens=None, nvals=0,
+                       device=0, stream=None):
+    """pskv_slice_noalloc: device tensors in (keys int64, lens int32 or None) and out (pos and
+    val_pos int64 of S+1, used uint8 of S, status int32 of 1); asynchronous on `stream`."""
+    kp, n, _ = _buf(keys, np.uint64, "int64")
+    lp, nl, _ = _buf(lens, np.int32, "int32")
+    rb = np.ascontiguousarray(range_begin, dtype=np.uint64)
+    re = np.ascontiguousarray(range_end, dtype=np.uint64)
+    _check(load().pskv_slice_noalloc(device, stream, kp, n, lp, nl, nvals, rb.ctypes.data,
+                                     re.ctypes.data, rb.size, pos.data_ptr(), val_pos.data_ptr(),
+                                     used.data_ptr(), status.data_ptr()))
 
 
 def assemble_pull(req_keys, responses, out, out_lens=None, device=0):

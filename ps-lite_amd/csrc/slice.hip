@@ -58,8 +58,8 @@ __global__ __launch_bounds__(kBlock) void k_bounds(const uint64_t* __restrict__ 
 // boundary is searched in the suffix that starts at the previous one, which for
 // sorted keys is max(previous, lower_bound over the whole array).
 // One wavefront. `pos` is device memory (read by the lens sums), `pos_host` pinned host
-// memory the caller reads after the stream wait; `sums` (may be null) is cleared for
-// the kernel that follows.
+// memory the caller reads after the stream wait (may be null); `sums` (may be null) is
+// cleared for the kernel that follows.
 __global__ void k_bounds_chain(const uint64_t* __restrict__ lb, uint64_t S,
                                uint64_t* __restrict__ pos, uint64_t* __restrict__ pos_host,
                                unsigned long long* __restrict__ sums) {
@@ -69,12 +69,12 @@ __global__ void k_bounds_chain(const uint64_t* __restrict__ lb, uint64_t S,
   if (threadIdx.x != 0) return;
   uint64_t p = lb[0];
   pos[0] = p;
-  pos_host[0] = p;
+  if (pos_host) pos_host[0] = p;
   for (uint64_t i = 0; i < S; ++i) {
     const uint64_t e = lb[i + 1];
     p = e > p ? e : p;
     pos[i + 1] = p;
-    pos_host[i + 1] = p;
+    if (pos_host) pos_host[i + 1] = p;
   }
 }
 
@@ -101,12 +101,77 @@ __global__ __launch_bounds__(kFusedWaves * 64) void k_bounds_fused(
   if (threadIdx.x != 0) return;
   uint64_t p = s_lb[0];
   pos[0] = p;
-  pos_host[0] = p;
+  if (pos_host) pos_host[0] = p;
   for (uint64_t i = 0; i < S; ++i) {
     const uint64_t e = s_lb[i + 1];
     p = e > p ? e : p;
     pos[i + 1] = p;
-    pos_host[i + 1] = p;
+    if (pos_host) pos_host[i + 1] = p;
+  }
+}
+
+// ---- the slicer for callers that cannot allocate ------------------------------------------
+// Working memory of pskv_slice_noalloc: the lower bounds of the boundary searches followed by
+// the per-slice sums of lens. It lives in the code object, so every GPU that loads the library
+// holds its own copy until the process ends; host code reaches it through the address that
+// hipGetSymbolAddress returns on that GPU, never through this name.
+constexpr size_t kNoAllocMaxRanges = PSKV_SLICE_NOALLOC_MAX_RANGES;
+constexpr size_t kNoAllocLb = kNoAllocMaxRanges + 1;            // words [0, kNoAllocLb): lower bounds
+constexpr size_t kNoAllocWords = kNoAllocLb + kNoAllocMaxRanges;  // then kNoAllocMaxRanges sums
+static __device__ __align__(256) unsigned long long scratch[kNoAllocWords];
+
+// Up to kFusedTargets searches whose targets travel with the launch; the answers go to lb[].
+__global__ __launch_bounds__(kFusedWaves * 64) void k_bounds_args(const uint64_t* __restrict__ keys,
+                                                                 uint64_t n, FusedTargets targets,
+                                                                 unsigned count,
+                                                                 unsigned long long* __restrict__ lb) {
+  const unsigned lane = threadIdx.x & 63, waves = blockDim.x >> 6;
+  for (unsigned w = threadIdx.x >> 6; w < count; w += waves) {  // whole wavefronts
+    const uint64_t lo = wave_lower_bound(keys, n, targets.v[w], lane);
+    if (lane == 0) lb[w] = lo;
+  }
+}
+
+// What pskv_slice does on the host once the positions and the per-slice sums are known
+// (kv_app.h:540-571), by one thread, with the outputs in device memory: the `first` flags,
+// the coverage check, the value offsets and their checks. `late_error` is a status the host
+// already knows but which the reference raises only after the coverage check.
+__global__ void k_noalloc_finish(const uint64_t* __restrict__ pos,
+                                 const unsigned long long* __restrict__ sums, uint64_t S, uint64_t n,
+                                 uint64_t nvals, uint64_t k, int has_lens, int late_error,
+                                 uint64_t* __restrict__ val_pos, uint8_t* __restrict__ used,
+                                 int32_t* __restrict__ status) {
+  for (uint64_t i = threadIdx.x; i <= S; i += blockDim.x) val_pos[i] = 0;
+  for (uint64_t i = threadIdx.x; i < S; i += blockDim.x) used[i] = pos[i + 1] != pos[i];  // kv_app.h:540
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  if (pos[S] != n) {  // kv_app.h:542
+    *status = PSKV_EUNCOVERED_KEY;
+    return;
+  }
+  *status = PSKV_OK;
+  if (n == 0) return;  // kv_app.h:543
+  if (late_error) {    // kv_app.h:549,551
+    *status = late_error;
+    return;
+  }
+  if (!has_lens) {
+    for (uint64_t i = 0; i <= S; ++i) val_pos[i] = pos[i] * k;  // kv_app.h:569
+    return;
+  }
+  uint64_t val_begin = 0, val_end = 0;  // kv_app.h:563-567 with the CHECKs of sarray.h:249
+  for (uint64_t i = 0; i < S; ++i) {
+    val_pos[i] = val_begin;
+    if (pos[i + 1] != pos[i]) {
+      val_end += sums[i];
+      if (val_end < val_begin || val_end > nvals) {
+        val_pos[i + 1] = val_end;
+        *status = PSKV_ESIZE_MISMATCH;
+        return;
+      }
+      val_begin = val_end;
+    }
+    val_pos[i + 1] = val_end;
   }
 }
 
@@ -429,6 +494,100 @@ int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, 
     }
     val_pos[i + 1] = val_end;
   }
+  return PSKV_OK;
+}
+
+namespace {
+// Device address of `scratch` on every GPU this process has used the entry point on.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+unsigned long long* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// Called with `device` current. The first call on a device asks the runtime where that
+// device's copy of the array lives; later calls read the table.
+int noalloc_scratch(int device, unsigned long long** out) {
+  if (device < 0 || device >= kMaxDevices) return set_error(PSKV_EINVAL, "device %d out of range", device);
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (!g_scratch_ptr[device]) {
+    void* p = nullptr;
+    PSKV_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return set_error(PSKV_EHIP, "no device address for the slicer's working memory");
+    g_scratch_ptr[device] = static_cast<unsigned long long*>(p);
+  }
+  *out = g_scratch_ptr[device];
+  return PSKV_OK;
+}
+}  // namespace
+
+int pskv_slice_noalloc(int device, void* stream, const uint64_t* keys, size_t n, const int32_t* lens,
+                       size_t nlens, size_t nvals, const uint64_t* range_begin,
+                       const uint64_t* range_end, size_t S, uint64_t* pos, uint64_t* val_pos,
+                       uint8_t* used, int32_t* status) {
+  clear_error();
+  if (!pos || !val_pos || !status || (S && (!used || !range_begin || !range_end)))
+    return set_error(PSKV_EINVAL, "null argument");
+  if (n && !keys) return set_error(PSKV_EINVAL, "null keys");
+  if (S == 0) return set_error(PSKV_EINVAL, "pskv_slice_noalloc needs at least one range");
+  if (S > kNoAllocMaxRanges)
+    return set_error(PSKV_EINVAL, "pskv_slice_noalloc serves at most %zu ranges, %zu were given",
+                     kNoAllocMaxRanges, S);
+  for (size_t i = 1; i < S; ++i) {  // kv_app.h:533
+    if (range_end[i - 1] != range_begin[i])
+      return set_error(PSKV_ERANGE_GAP, "ranges[%zu].end != ranges[%zu].begin", i - 1, i);
+  }
+  DeviceGuard guard(device);
+  if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", device);
+  unsigned long long* ws = nullptr;
+  int rc = noalloc_scratch(device, &ws);
+  if (rc) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  unsigned long long* d_lb = ws;
+  unsigned long long* d_sums = ws + kNoAllocLb;
+
+  const bool has_lens = lens != nullptr && nlens != 0;
+  const bool do_sums = has_lens && nlens == n && n != 0;
+  int late_error = PSKV_OK;
+  uint64_t k = 0;
+  if (n) {
+    if (!has_lens) {
+      k = nvals / n;  // kv_app.h:548-549
+      if (k * n != nvals) late_error = PSKV_ESIZE_MISMATCH;
+    } else if (nlens != n) {  // kv_app.h:551
+      late_error = PSKV_ESIZE_MISMATCH;
+    }
+  }
+  if (S + 1 <= kFusedTargets) {  // searches, chain and the clearing of the sums in one launch
+    FusedTargets ft = {};
+    ft.v[0] = range_begin[0];
+    for (size_t i = 0; i < S; ++i) ft.v[i + 1] = range_end[i];
+    const unsigned waves = (unsigned)std::min<size_t>(S + 1, kFusedWaves);
+    k_bounds_fused<<<dim3(1), dim3(waves * 64), 0, st>>>(keys, n, ft, S, pos, (uint64_t*)nullptr, d_sums);
+    PSKV_HIP(hipGetLastError());
+  } else {
+    for (size_t first = 0; first <= S; first += kFusedTargets) {
+      const size_t count = std::min<size_t>(S + 1 - first, kFusedTargets);
+      FusedTargets ft = {};
+      for (size_t j = 0; j < count; ++j) {
+        const size_t i = first + j;
+        ft.v[j] = i == 0 ? range_begin[0] : range_end[i - 1];
+      }
+      const unsigned waves = (unsigned)std::min<size_t>(count, kFusedWaves);
+      k_bounds_args<<<dim3(1), dim3(waves * 64), 0, st>>>(keys, n, ft, (unsigned)count, d_lb + first);
+      PSKV_HIP(hipGetLastError());
+    }
+    k_bounds_chain<<<dim3(1), dim3(64), 0, st>>>(reinterpret_cast<const uint64_t*>(d_lb), S, pos,
+                                                (uint64_t*)nullptr, d_sums);
+    PSKV_HIP(hipGetLastError());
+  }
+  if (do_sums) {
+    uint64_t per = n / S / (kBlock * 8) + 1;
+    if (per > 1024) per = 1024;
+    k_segment_sums<<<dim3((unsigned)per, (unsigned)S), dim3(kBlock), 0, st>>>(lens, pos, d_sums);
+    PSKV_HIP(hipGetLastError());
+  }
+  k_noalloc_finish<<<dim3(1), dim3(256), 0, st>>>(pos, d_sums, S, n, nvals, k, has_lens ? 1 : 0,
+                                                   late_error, val_pos, used, status);
+  PSKV_HIP(hipGetLastError());
   return PSKV_OK;
 }
 
