@@ -21,9 +21,12 @@
  *    before the call. Calls with PSKV_MEM_HOST buffers return when done.
  *  - Keys within one request must be unique (ps-lite requires sorted unique
  *    keys, include/ps/kv_app.h:17); requests on one table are applied in call
- *    order. A request that repeats a key: the row modes answer PSKV_EINVAL;
- *    PSKV_MODE_SCALAR gives the result of the reference's loop
- *    (kv_app.h:451-459) when the keys are sorted, an unspecified sum otherwise. A table must not be used from two threads at once (the reference
+ *    order. A SORTED request that repeats a key: the row modes refuse it as a whole with
+ *    PSKV_EINVAL (no stored value changes; PSKV_MODE_FIXED may leave the keys it named as
+ *    zero rows, as a pull of them would), PSKV_MODE_SCALAR gives the result of the
+ *    reference's loop (kv_app.h:451-459). An unsorted request that repeats a key has an
+ *    unspecified result in every mode (no memory other than its keys' values is touched).
+ *    A table must not be used from two threads at once (the reference
  *    runs the handle on one Customer thread, src/customer.cc:49-63).
  *    pskv_slice is re-entrant.
  *

@@ -15,6 +15,10 @@ namespace pskv {
 // directly is served from one side slot kept in DevState.
 constexpr uint64_t kEmptyKey = ~0ull;
 
+// A launch serves up to kMaxBatch tables at once: blockIdx.y selects the table, blockIdx.x is the
+// workgroup's number among those that serve it.
+constexpr int kMaxBatch = 16;
+
 // Row reference handed from the lookup kernel to the row kernels.
 //   FIXED : low bits = row index
 //   VARLEN: bits [28,63) = arena offset in 16-byte units, bits [0,28) = row length in floats
@@ -87,7 +91,9 @@ struct alignas(32) DevState {
   unsigned int ticket_top;             // second level of the last-workgroup ticket (ticket_last)
   unsigned long long cache_epoch;
   unsigned long long bad_epoch;
-  unsigned long long pad0;
+  // FIXED: the request with this number was refused (it repeats a key): its row kernels change
+  // no stored value and leave the rows it created as zero rows
+  unsigned long long refused_epoch;
   // keys held (slot array plus the side slot) = sum of the shards
   unsigned long long count_shard[kCountShards * kShardStride];
   // first level of the last-workgroup ticket: one counter per 128-byte line
@@ -121,6 +127,7 @@ __device__ __forceinline__ ReqFacts load_req_facts(const DevState* st) {
 constexpr unsigned kReqMisaligned = 3u;  // OR of (len & 3)
 constexpr unsigned kReqBadLen = 4u;      // a length negative or above the maximum
 constexpr unsigned kReqDiffer = 8u;      // a key or length differs from the cached request
+constexpr unsigned kReqDuplicate = 16u;  // a key equals its left neighbour (requests are sorted)
 
 // Counters of the table as they are after request `seq`, written by the device into pinned
 // host memory so that the host can bound the counters without waiting for the stream.
@@ -154,9 +161,10 @@ __device__ __forceinline__ void raise_error(DevState* st, unsigned bit, unsigned
   st->bad_epoch = epoch;
 }
 
-// Finds the workgroup of a grid that finishes last. Thread 0 of EVERY workgroup calls it once,
-// after the writes the last workgroup is to see; it returns true in exactly one of them,
-// and that thread then sees those writes.
+// Finds the workgroup that finishes last among the `nblk` workgroups that serve one table in a
+// launch (workgroups blockIdx.x = 0 .. nblk-1 of the table's row of the grid). Thread 0 of EVERY
+// one of them calls it once, after the writes the last workgroup is to see; it returns true in
+// exactly one of them, and that thread then sees those writes.
 // What the callers hand to the last workgroup must have been written with device-scope
 // atomics (atomicOr, publish_u64 below): those are performed at the memory side, past the
 // per-XCD L2, so all a workgroup has to do before its ticket is wait for its own

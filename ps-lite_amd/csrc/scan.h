@@ -80,8 +80,8 @@ __device__ __forceinline__ void scan_spine(unsigned long long* part, uint64_t np
 // sign-extended 64-bit values modulo 2^64 (what `size_t val_end += int l` does in the
 // reference, kv_app.h:565), and the kReq* facts it found. The workgroup's total goes to
 // part[blockIdx.x], its facts to DevState::req_flags (one atomic per workgroup at most).
-// Returns true in every thread of the workgroup that finishes last.
-// `red`/`fred` hold kBlock/64 words each.
+// Returns true in every thread of the workgroup that finishes last of the `nblk` that scan this
+// table's request. `red`/`fred` hold kBlock/64 words each.
 __device__ __forceinline__ bool scan_pass1_block(unsigned long long s, unsigned flags,
                                                  unsigned long long* __restrict__ part,
                                                  DevState* st, unsigned long long* red,
@@ -112,8 +112,9 @@ __device__ __forceinline__ unsigned scan_pass1_last(unsigned long long* part, De
     st->scan_total = *carry_s;
     st->error |= st->req_error;
     const bool bad_len = (flags & kReqBadLen) != 0u;
-    st->req_error = bad_len ? kDevErrBadLen : 0u;
-    if (bad_len) st->bad_epoch = epoch;
+    const bool dup = (flags & kReqDuplicate) != 0u;
+    st->req_error = (bad_len ? kDevErrBadLen : 0u) | (dup ? kDevErrDuplicate : 0u);
+    if (bad_len || dup) st->bad_epoch = epoch;
     st->misaligned = flags & kReqMisaligned;
   }
   return flags;
@@ -160,7 +161,8 @@ __device__ __forceinline__ void scan_pass2_offsets(const unsigned long long (&v)
   }
 }
 
-inline int scan_items(uint64_t n) { return n >= kScanLargeKeys ? kScanItemsLarge : 1; }
+// `n_largest`: the longest key list among the tables a launch serves; all of them use one split.
+inline int scan_items(uint64_t n_largest) { return n_largest >= kScanLargeKeys ? kScanItemsLarge : 1; }
 inline uint64_t scan_num_parts(uint64_t n) {
   const uint64_t chunk = (uint64_t)kBlock * scan_items(n);
   return (n + chunk - 1) / chunk;

@@ -149,6 +149,14 @@ constexpr uint64_t kLookupLargeKeys = 1u << 20;
 // every thread claims slots for its keys, then the workgroup takes the rows of all
 // created keys from the arena with ONE atomic add and a workgroup-wide scan hands them
 // out in request order, so rows of neighbouring keys are neighbours in the arena.
+// FIXED: request `tag` repeats a key. Reported by the next wait; the request's row kernels
+// change no stored value.
+__device__ __forceinline__ void refuse_fixed(DevState* st, const ReqTag& tag) {
+  atomicOr(&st->error, kDevErrDuplicate);
+  st->bad_epoch = tag.epoch;
+  st->refused_epoch = tag.epoch;
+}
+
 template <int kLookupItems>
 __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slots, uint64_t mask,
                                                         DevState* st,
@@ -182,12 +190,17 @@ __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slot
       if (i < n) {
         const uint64_t key = keys[i];
         if (cache_keys) cache_keys[i] = key;
-        p[j] = find_or_insert(slots, mask, st, key, is_new[j], seen[j]);
+        // keys are sorted and must be unique (kv_app.h:17): a key that equals its left neighbour
+        // refuses the request, whether the key is new or has been in the table for long
+        if (i > 0 && keys[i - 1] == key) {
+          refuse_fixed(st, tag);
+        } else {
+          p[j] = find_or_insert(slots, mask, st, key, is_new[j], seen[j]);
+        }
       }
       if (p[j] && !is_new[j] && seen[j] == kPayloadUnset) {
-        // another lane of this request is creating the very same key: keys must be unique
-        atomicOr(&st->error, kDevErrDuplicate);
-        st->bad_epoch = tag.epoch;
+        // (unsorted request) another lane of this request is creating the very same key
+        refuse_fixed(st, tag);
         p[j] = nullptr;
       }
       mine += (p[j] && is_new[j]) ? 1u : 0u;
@@ -242,14 +255,16 @@ __global__ __launch_bounds__(kBlock) void k_var_push_begin(
   for (int j = 0; j < kItems; ++j) {
     const bool in = base + j < n;
     l[j] = in ? lens[base + j] : 0;
-    k[j] = ck[j] = 0;
+    k[j] = in ? keys[base + j] : 0;
+    ck[j] = k[j];
     cl[j] = l[j];
     if (in && tag.try_cache) {
-      k[j] = keys[base + j];
       ck[j] = cache_keys[base + j];
       cl[j] = cache_lens[base + j];
     }
   }
+  // the key in front of this thread's first one (its neighbour has asked for that line already)
+  const uint64_t left = (base > 0 && base < n) ? keys[base - 1] : 0;
   unsigned long long s = 0;
   unsigned flags = 0;
 #pragma unroll
@@ -258,6 +273,10 @@ __global__ __launch_bounds__(kBlock) void k_var_push_begin(
     flags |= (unsigned)l[j] & kReqMisaligned;
     flags |= (l[j] < 0 || (unsigned)l[j] > max_len) ? kReqBadLen : 0u;
     flags |= (k[j] != ck[j] || l[j] != cl[j]) ? kReqDiffer : 0u;
+    // keys are sorted and must be unique (kv_app.h:17): a key that equals its left neighbour
+    // refuses the request before anything of it is applied
+    const bool has_left = base + j < n && base + j > 0;
+    flags |= (has_left && k[j] == (j ? k[j - 1] : left)) ? kReqDuplicate : 0u;
   }
   if (!scan_pass1_block(s, flags, part, st, red, fred, &s_last)) return;
   flags = scan_pass1_last(part, st, tag.epoch, red, &carry_s);
@@ -285,8 +304,9 @@ __global__ __launch_bounds__(kBlock) void k_var_push_lookup(
     if (snap && blockIdx.x == 0 && threadIdx.x < 64) publish_snapshot(st, snap, snap_seq);
     return;
   }
-  // the request is refused as a whole when its lens are invalid or do not add up to vals.size()
-  if (st->req_error & (kDevErrBadLen | kDevErrSizeMismatch)) return;
+  // the request is refused as a whole when its lens are invalid or do not add up to vals.size(),
+  // or when it repeats a key
+  if (st->req_error & (kDevErrBadLen | kDevErrSizeMismatch | kDevErrDuplicate)) return;
   if (st->scan_total != nvals) {
     if (blockIdx.x == 0 && threadIdx.x == 0) raise_error(st, kDevErrSizeMismatch, tag.epoch);
     return;
@@ -487,6 +507,8 @@ __device__ __forceinline__ void vstore(V v, V* p) {
 // follows from a division (one compare when a row is at least a tile long).
 template <int OP, int VEC, bool STREAM, unsigned TILE>
 __device__ __forceinline__ void rows_tile_fixed(const RowsParams& p, uint64_t total) {
+  // a refused push (it repeats a key) changes no stored value; rows it created stay, as zero rows
+  const bool rejected = OP == kOpAcc && p.st->refused_epoch == p.tag.epoch;
   using V = typename VecT<VEC>::type;
   constexpr int kIter = TILE / (VEC * kBlock);      // elements per thread
   constexpr int kGroup = kIter < 4 ? kIter : 4;     // loads issued back to back
@@ -552,8 +574,12 @@ __device__ __forceinline__ void rows_tile_fixed(const RowsParams& p, uint64_t to
     for (int u = 0; u < kGroup; ++u) {
       if (!live[u]) continue;
       if (OP == kOpAcc) {
-        // a created row is a zero row first (0.0f + v), kv_app.h:454
-        vstore<STREAM>(y[u] + x[g + u], dst[u]);
+        if (rejected) {
+          if (fresh[u]) vstore<STREAM>(VecT<VEC>::zero(), dst[u]);
+        } else {
+          // a created row is a zero row first (0.0f + v), kv_app.h:454
+          vstore<STREAM>(y[u] + x[g + u], dst[u]);
+        }
       } else {
         vstore<STREAM>(y[u], reinterpret_cast<V*>(p.req + f0 + lf[u]));
         if (fresh[u]) vstore<STREAM>(VecT<VEC>::zero(), dst[u]);  // pull created the row: zeros
@@ -826,7 +852,7 @@ __global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
     const bool same = facts.same_epoch == p.tag.epoch;
     if (same) p.ignore_new = 1;
     const unsigned err = same ? 0u : facts.req_error;
-    if (err & (kDevErrBadLen | kDevErrSizeMismatch)) return;
+    if (err & (kDevErrBadLen | kDevErrSizeMismatch | kDevErrDuplicate)) return;
     rejected = (err & kDevErrLenChanged) != 0;
     scalar = scalar || (facts.misaligned != 0);
     if (p.total_on_device) {

@@ -126,31 +126,33 @@ def _rank_to_key(r):
     return ((r.astype(np.uint64) * np.uint64(0x9E3779B97F4A7C15)) >> np.uint64(1)).astype(np.uint64)
 
 
-@pytest.mark.parametrize("scale", [8, 1])
-def test_config4_zipf(capi, orc, dev, scale):
+@pytest.mark.parametrize("scale,model", [(8, "oracle"), (1, "integers"), (1, "oracle")])
+def test_config4_zipf(capi, orc, dev, scale, model):
     """8 worker pushes of Zipf(1.1)-popular keys from a 100M-key universe, then a pull of Zipf keys
-    of which many are absent. scale=8 is compared with the oracle float for float; scale=1 (4M keys
-    per push, 16M pulled) uses small-integer values, whose sums are exact in any order, against numpy."""
+    of which many are absent. With model "oracle" the values are N(0,1) and everything pulled is
+    compared with the oracle float for float: at one eighth of the size (where the whole store is
+    dumped and compared as well) and at the full size (4M keys per push, 16M pulled). Model
+    "integers" is a second, independent check at full size: small-integer values, whose sums are
+    exact in any order, against numpy."""
     import torch
-    announce("config4", scale)
+    announce("config4", scale, model)
     universe, n_push, n_pull, workers = 100000000 // scale, 4000000 // scale, 16000000 // scale, 8
     t = capi.Table(capi.MODE_SCALAR, initial_capacity=1 << 20)
-    o = orc.Store(orc.MODE_SCALAR) if scale > 1 else None
+    o = orc.Store(orc.MODE_SCALAR) if model == "oracle" else None
     pushed_ranks, pushed_vals = [], []
     for w in range(workers):
         rng = np.random.default_rng(0x21F + w)
         ranks = _zipf_unique(rng, n_push, universe)
         keys = np.sort(_rank_to_key(ranks))
-        vals = rng.standard_normal(n_push).astype(np.float32) if scale > 1 else \
+        vals = rng.standard_normal(n_push).astype(np.float32) if o else \
             rng.integers(-500, 500, size=n_push).astype(np.float32)
         assert np.all(np.diff(keys.astype(np.int64 if keys.max() < 2 ** 63 else np.uint64)) != 0)
         t.push(to_dev(keys, dev), to_dev(vals, dev))
         t.sync()
         if o:
             o.push(keys, vals)
-        else:
-            pushed_ranks.append(keys)
-            pushed_vals.append(vals)
+        pushed_ranks.append(keys)
+        pushed_vals.append(vals)
     rng = np.random.default_rng(0x9011)
     probe = np.sort(_rank_to_key(_zipf_unique(rng, n_pull, universe)))
     dk = to_dev(probe, dev)
@@ -161,10 +163,20 @@ def test_config4_zipf(capi, orc, dev, scale):
     if o:
         assert_bits_equal(got, o.pull(probe)[0], "config4")
         assert t.size() == o.size()
-        gk, _, gv = t.dump()
-        ok, _, ov = o.dump()
-        assert np.array_equal(gk, ok)
-        assert_bits_equal(gv, ov, "config4 dump")
+        if scale > 1:
+            gk, _, gv = t.dump()
+            ok, _, ov = o.dump()
+            assert np.array_equal(gk, ok)
+            assert_bits_equal(gv, ov, "config4 dump")
+        else:
+            # every key ever pushed, pulled back: the whole store float for float without the
+            # host-side sort of a dump
+            everything = np.unique(np.concatenate(pushed_ranks))
+            out_all = torch.empty(everything.size, dtype=torch.float32, device=dev)
+            t.pull(to_dev(everything, dev), out_all)
+            t.sync()
+            assert_bits_equal(from_dev(out_all), o.pull(everything)[0], "config4 all pushed keys")
+            assert t.size() == o.size()
     else:
         allk = np.concatenate(pushed_ranks)
         allv = np.concatenate(pushed_vals).astype(np.int64)

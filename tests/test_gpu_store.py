@@ -675,7 +675,9 @@ def test_duplicate_keys_do_no_harm(capi, dev, mode):
     except capi.PskvError as e:
         reported = e.code == capi.EINVAL
     assert reported
-    assert t.size()[0] == 4
+    # the refused request changed no value; FIXED has created the keys it named as zero rows (as a
+    # pull of them would), VARLEN has created nothing
+    assert t.size()[0] == (4 if mode == "fixed" else 0)
     # the table is still usable
     uniq = np.unique(keys)
     t.push(uniq, np.ones(uniq.size * 8, np.float32), np.full(uniq.size, 8, np.int32) if mode == "varlen" else None)
@@ -862,3 +864,116 @@ def test_scalar_long_probe_chains(capi, orc, dev):
             t.pull(probe, got)
             assert_bits_equal(got, o.pull(probe)[0], "rep %d" % rep)
     _check_dump(t, o, "long probes")
+
+
+def _row_push(t, dev, memkind, keys, vals, lens):
+    """A push through host or device buffers; returns the status the caller gets to see (device
+    buffers: at the next sync)."""
+    try:
+        if memkind == "device":
+            t.push(to_dev(keys, dev), to_dev(vals, dev), None if lens is None else to_dev(lens, dev))
+            t.sync()
+        else:
+            t.push(keys, vals, lens)
+    except Exception as e:  # capi.PskvError
+        return e.code
+    return 0
+
+
+@pytest.mark.parametrize("memkind", ["device", "host"])
+@pytest.mark.parametrize("mode", ["fixed", "varlen"])
+def test_sorted_repeats_refuse_row_requests(capi, orc, dev, mode, memkind):
+    """Keys of a request are sorted and unique (kv_app.h:17). In the row modes a sorted request that
+    repeats a key is refused as a whole with PSKV_EINVAL, whether the key is new or already stored and
+    wherever in the request the repeat sits: no stored value changes. (A FIXED request may leave
+    keys it named as zero rows, as a pull of them would.)"""
+    announce("sorted_repeats_refused", mode, memkind)
+    rng = np.random.default_rng(91)
+    m = capi.MODE_FIXED if mode == "fixed" else capi.MODE_VARLEN
+    om = orc.MODE_FIXED if mode == "fixed" else orc.MODE_VARLEN
+    k = 8
+    t = capi.Table(m, initial_capacity=16)
+    o = orc.Store(om)
+
+    def lens_for(n):
+        return None if mode == "fixed" else np.full(n, k, np.int32)
+
+    base = unique_keys(rng, 700)
+    vals = rng.normal(0, 1, size=base.size * k).astype(np.float32)
+    assert _row_push(t, dev, memkind, base, vals, lens_for(base.size)) == 0
+    o.push(base, vals, lens_for(base.size))
+    _check_dump(t, o, "before")
+
+    def refused(keys):
+        v = np.ones(keys.size * k, np.float32)
+        assert _row_push(t, dev, memkind, keys, v, lens_for(keys.size)) == capi.EINVAL
+        if mode == "fixed":
+            o.pull(np.unique(keys))  # a FIXED pull creates absent keys as zero rows
+        _check_dump(t, o, "after a refused request")
+
+    # the very key the table already holds, twice
+    refused(np.array([base[9], base[9]], np.uint64))
+    # a repeat of a stored key one workgroup apart (positions 255 and 256), among stored keys
+    refused(np.concatenate([base[:256], base[255:600]]))
+    # a repeat of a NEW key, at the wavefront boundary 63/64 and at the end of the request
+    fresh = unique_keys(rng, 300)
+    fresh = np.setdiff1d(fresh, base)[:200]
+    refused(np.concatenate([fresh[:64], fresh[63:150], fresh[149:150]]))
+    # a long run
+    refused(np.sort(np.concatenate([base[:5], np.full(300, base[3], np.uint64)])))
+    # the table still serves good requests, and they see the values of before
+    more = rng.normal(0, 1, size=base.size * k).astype(np.float32)
+    assert _row_push(t, dev, memkind, base, more, lens_for(base.size)) == 0
+    o.push(base, more, lens_for(base.size))
+    _check_dump(t, o, "after")
+    if mode == "fixed":
+        # a FIXED pull creates keys too, so it refuses repeats as well
+        dup = np.array([base[1], base[2], base[2]], np.uint64)
+        with pytest.raises(capi.PskvError) as e:
+            t.pull(dup, np.zeros(dup.size * k, np.float32))
+        assert e.value.code == capi.EINVAL
+        _check_dump(t, o, "after a refused pull")
+
+
+@pytest.mark.parametrize("memkind", ["device", "host"])
+@pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
+def test_pushpull_with_too_small_a_buffer_applies_its_push_once(capi, orc, dev, mode, memkind):
+    """A push+pull whose response does not fit answers PSKV_ESIZE_MISMATCH with the needed size; its
+    push half has been applied (exactly once), so the caller repeats only the pull. This is what the
+    second attempt of GpuKVHandle relies on."""
+    import torch
+    announce("pushpull_too_small", mode, memkind)
+    rng = np.random.default_rng(17)
+    m = {"scalar": capi.MODE_SCALAR, "fixed": capi.MODE_FIXED, "varlen": capi.MODE_VARLEN}[mode]
+    om = {"scalar": orc.MODE_SCALAR, "fixed": orc.MODE_FIXED, "varlen": orc.MODE_VARLEN}[mode]
+    t = capi.Table(m, initial_capacity=16)
+    o = orc.Store(om)
+    n = 3000
+    keys = unique_keys(rng, n)
+    lens = rng.choice(np.array([0, 4, 8, 12], np.int32), size=n).astype(np.int32) if mode == "varlen" else None
+    nvals = {"scalar": n, "fixed": 4 * n, "varlen": int(lens.sum()) if lens is not None else 0}[mode]
+
+    def as_mem(a):
+        if a is None:
+            return None
+        return to_dev(a, dev) if memkind == "device" else a
+
+    for rep in range(3):
+        vals = rng.normal(0, 1, size=nvals).astype(np.float32)
+        want, want_lens = o.pushpull(keys, vals, lens)
+        small_np = np.zeros(max(nvals // 2, 1), np.float32)
+        small = as_mem(small_np)
+        out_lens = as_mem(np.zeros(n, np.int32)) if mode == "varlen" else None
+        with pytest.raises(capi.PskvError) as e:
+            t.pushpull(as_mem(keys), as_mem(vals), small, as_mem(lens), out_lens)
+        assert e.value.code == capi.ESIZE_MISMATCH
+        assert t.last_out_nvals == nvals
+        t.sync()
+        got = as_mem(np.zeros(nvals, np.float32))
+        got_lens = as_mem(np.zeros(n, np.int32)) if mode == "varlen" else None
+        assert t.pull(as_mem(keys), got, got_lens) == nvals
+        t.sync()
+        assert_bits_equal(from_dev(got) if memkind == "device" else got, want, "pull after refused pushpull %d" % rep)
+        if mode == "varlen":
+            assert np.array_equal(from_dev(got_lens) if memkind == "device" else got_lens, want_lens)
+    _check_dump(t, o, "pushpull too small")

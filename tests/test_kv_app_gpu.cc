@@ -138,6 +138,29 @@ static void RunVarLen() {
   EXPECT(out.size() == total);
   EXPECT(out_lens == lens);
   for (size_t i = 0; i < out.size() && i < total; ++i) EXPECT(out[i] == 4 * vals[i]);
+  // push and pull in one request: the push is applied once, then read back (kv_app.h:453-458)
+  std::vector<float> both;
+  std::vector<int> both_lens = lens;
+  kv.Wait(kv.PushPull(keys, vals, &both, &both_lens));
+  EXPECT(both.size() == total);
+  EXPECT(both_lens == lens);
+  for (size_t i = 0; i < both.size() && i < total; ++i) EXPECT(both[i] == 5 * vals[i]);
+  // a small pull, then a larger one again: the handle sizes its response buffer from the last
+  // response and must ask a second time when that guess is too small
+  std::vector<Key> few(keys.begin(), keys.begin() + 10);
+  std::vector<float> few_out;
+  std::vector<int> few_lens;
+  kv.Wait(kv.Pull(few, &few_out, &few_lens));
+  size_t few_total = 0;
+  for (int i = 0; i < 10; ++i) few_total += lens[i];
+  EXPECT(few_out.size() == few_total);
+  for (size_t i = 0; i < few_out.size() && i < few_total; ++i) EXPECT(few_out[i] == 5 * vals[i]);
+  std::vector<float> again;
+  std::vector<int> again_lens;
+  kv.Wait(kv.Pull(keys, &again, &again_lens));
+  EXPECT(again.size() == total);
+  EXPECT(again_lens == lens);
+  for (size_t i = 0; i < again.size() && i < total; ++i) EXPECT(again[i] == 5 * vals[i]);
 }
 
 static void RunFailures(int num_servers) {
