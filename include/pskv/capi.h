@@ -114,6 +114,39 @@ int pskv_pushpull(pskv_table* t, const uint64_t* keys, size_t n, const float* va
                   const int32_t* lens, size_t nlens, float* out, size_t out_cap,
                   int32_t* out_lens, size_t* out_nvals, int memkind);
 
+/* One process, several logical servers on one GPU. KVWorker::Send turns a sliced request into
+ * one message per server range (kv_app.h:590-612); when the tables of those ranges live in one
+ * process on one GPU, the three calls below serve all of them with ONE launch per step of the
+ * pipeline instead of one per table (a launch over 1/S of a request leaves most of the GPU
+ * idle). pos[S+1] and val_pos[S+1] are HOST arrays, exactly what pskv_slice returns: slice s
+ * holds keys [pos[s], pos[s+1]) and vals [val_pos[s], val_pos[s+1]) (and lens [pos[s],
+ * pos[s+1]) in PSKV_MODE_VARLEN) and goes to tables[s]; a slice without keys is skipped, as
+ * Send skips it (`first == false`, kv_app.h:581-595). The result is what S calls of pskv_push /
+ * pskv_pull would give. The tables must share a device, a mode and a STREAM: create the first,
+ * then pass pskv_table_stream(first) as pskv_opts.stream of the others. keys/vals/lens/out/
+ * out_lens are device memory (PSKV_MEM_DEVICE is the only memkind accepted) and the calls are
+ * asynchronous like the single-table ones. Everything the host can check is checked for all
+ * slices before anything is enqueued; device-detected errors are reported per table by
+ * pskv_sync / pskv_sync_multi. More than 16 slices with keys are served 16 at a time. */
+void* pskv_table_stream(pskv_table* t);
+int pskv_push_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, const uint64_t* pos,
+                    const float* vals, const uint64_t* val_pos, const int32_t* lens, int memkind);
+/* Slice s answers into out[out_pos[s] .. out_pos[s+1]) (room, not necessarily all used) and, in
+ * PSKV_MODE_VARLEN, out_lens[pos[s] .. pos[s+1]). out_pos == NULL means out_pos[s] = pos[s] * k
+ * (SCALAR: k = 1, FIXED: the row length); PSKV_MODE_VARLEN needs out_pos. A SCALAR/FIXED slice
+ * whose room is too small fails the call with PSKV_ESIZE_MISMATCH before anything is enqueued.
+ * out_nvals (host array of S, may be NULL) receives the floats each slice answered; in
+ * PSKV_MODE_VARLEN a non-NULL out_nvals makes the call wait for the device (and a slice that
+ * does not fit fails it with PSKV_ESIZE_MISMATCH, the needed sizes in out_nvals), with NULL it
+ * stays asynchronous and a slice that does not fit writes nothing and is reported by the next
+ * sync, as in pskv_pull. */
+int pskv_pull_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, const uint64_t* pos,
+                    float* out, const uint64_t* out_pos, int32_t* out_lens, uint64_t* out_nvals,
+                    int memkind);
+/* pskv_sync for all tables of a group with one wait: returns the first deferred error (every
+ * table's error state is cleared). */
+int pskv_sync_multi(pskv_table* const* tables, size_t S);
+
 /* Waits for everything enqueued on the table and reports a deferred device-side
  * error (PSKV_ELEN_CHANGED) of an earlier asynchronous push, once. */
 int pskv_sync(pskv_table* t);

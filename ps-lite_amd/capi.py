@@ -38,7 +38,7 @@ ERROR_NAMES = {
 # every symbol include/pskv/capi.h declares
 SYMBOLS = [
     "pskv_table_create", "pskv_table_destroy", "pskv_push", "pskv_pull", "pskv_pushpull",
-    "pskv_sync", "pskv_size", "pskv_dump", "pskv_slice", "pskv_slice_noalloc", "pskv_server_ranges",
+    "pskv_sync", "pskv_table_stream", "pskv_push_multi", "pskv_pull_multi", "pskv_sync_multi", "pskv_size", "pskv_dump", "pskv_slice", "pskv_slice_noalloc", "pskv_server_ranges",
     "pskv_assemble_pull", "pskv_prof_enable", "pskv_prof_reset", "pskv_prof_read", "pskv_prof_samples",
     "pskv_copy_probe", "pskv_host_alloc", "pskv_host_free", "pskv_host_trim", "pskv_last_error",
     "pskv_version",
@@ -84,6 +84,11 @@ def load():
     lib.pskv_pull.argtypes = [vp, vp, sz, vp, sz, vp, ctypes.POINTER(sz), i32]
     lib.pskv_pushpull.argtypes = [vp, vp, sz, vp, sz, vp, sz, vp, sz, vp, ctypes.POINTER(sz), i32]
     lib.pskv_sync.argtypes = [vp]
+    lib.pskv_table_stream.argtypes = [vp]
+    lib.pskv_table_stream.restype = vp
+    lib.pskv_push_multi.argtypes = [vp, sz, vp, vp, vp, vp, vp, i32]
+    lib.pskv_pull_multi.argtypes = [vp, sz, vp, vp, vp, vp, vp, vp, i32]
+    lib.pskv_sync_multi.argtypes = [vp, sz]
     lib.pskv_size.argtypes = [vp, ctypes.POINTER(u64), ctypes.POINTER(u64)]
     lib.pskv_dump.argtypes = [vp, vp, vp, sz, vp, sz, ctypes.POINTER(sz), ctypes.POINTER(sz)]
     lib.pskv_slice.argtypes = [i32, vp, sz, vp, sz, sz, vp, vp, sz, vp, vp, vp, i32]
@@ -247,6 +252,80 @@ class Table:
         assert dst.is_cuda and src.is_cuda
         nbytes = src.numel() * src.element_size()
         _check(self._lib.pskv_copy_probe(self._h, dst.data_ptr(), src.data_ptr(), nbytes))
+
+
+class Group:
+    """Several tables of one process on one GPU that share a stream, so that one launch per
+    pipeline step serves all key ranges of a sliced request (pskv_push_multi / pskv_pull_multi)."""
+
+    def __init__(self, S, mode=MODE_SCALAR, device=0, initial_capacity=0, row_len=0, arena_floats=0,
+                 max_load=0.0, stream=None):
+        self.tables = []
+        for s in range(S):
+            t = Table(mode, device, initial_capacity, row_len, arena_floats, max_load, stream)
+            if stream is None:
+                stream = load().pskv_table_stream(t._h)
+            self.tables.append(t)
+        self.S = S
+        self.mode = mode
+        self._arr = (ctypes.c_void_p * max(S, 1))(*[t._h for t in self.tables])
+        self._lib = load()
+
+    def close(self):
+        # the first table owns the stream the others run on: it goes last
+        for t in reversed(self.tables):
+            t.close()
+        self.tables = []
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def push_raw(self, keys_ptr, pos, vals_ptr, val_pos, lens_ptr=None):
+        """pos / val_pos: numpy uint64 arrays of S+1 entries as pskv_slice returns them."""
+        pos = np.ascontiguousarray(pos, dtype=np.uint64)
+        val_pos = np.ascontiguousarray(val_pos, dtype=np.uint64)
+        _check(self._lib.pskv_push_multi(self._arr, self.S, keys_ptr, pos.ctypes.data, vals_ptr,
+                                         val_pos.ctypes.data, lens_ptr, MEM_DEVICE))
+
+    def pull_raw(self, keys_ptr, pos, out_ptr, out_pos=None, out_lens_ptr=None, want_sizes=False):
+        """Returns the per-slice response sizes (numpy uint64) when want_sizes, else None."""
+        pos = np.ascontiguousarray(pos, dtype=np.uint64)
+        op = None
+        if out_pos is not None:
+            out_pos = np.ascontiguousarray(out_pos, dtype=np.uint64)
+            op = out_pos.ctypes.data
+        sizes = np.zeros(max(self.S, 1), np.uint64) if want_sizes else None
+        rc = self._lib.pskv_pull_multi(self._arr, self.S, keys_ptr, pos.ctypes.data, out_ptr, op,
+                                       out_lens_ptr, sizes.ctypes.data if want_sizes else None, MEM_DEVICE)
+        self.last_sizes = sizes
+        _check(rc)
+        return sizes[:self.S] if want_sizes else None
+
+    def push(self, keys, pos, vals, val_pos, lens=None):
+        _memkind(MEM_DEVICE)
+        self.push_raw(keys.data_ptr() if keys.numel() else None, pos,
+                      vals.data_ptr() if vals.numel() else None, val_pos,
+                      None if lens is None else (lens.data_ptr() if lens.numel() else None))
+
+    def pull(self, keys, pos, out, out_pos=None, out_lens=None, want_sizes=False):
+        _memkind(MEM_DEVICE)
+        return self.pull_raw(keys.data_ptr() if keys.numel() else None, pos,
+                             out.data_ptr() if out.numel() else None, out_pos,
+                             None if out_lens is None else (out_lens.data_ptr() if out_lens.numel() else None),
+                             want_sizes)
+
+    def sync(self):
+        _check(self._lib.pskv_sync_multi(self._arr, self.S))
+
+    def size(self):
+        nk = nv = 0
+        for t in self.tables:
+            a, b = t.size()
+            nk, nv = nk + a, nv + b
+        return nk, nv
 
 
 def server_ranges(num_servers):

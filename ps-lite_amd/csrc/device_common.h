@@ -173,15 +173,15 @@ __device__ __forceinline__ void raise_error(DevState* st, unsigned bit, unsigned
 // Two levels of counters, the first spread over kTicketShards cache lines, because atomics
 // on one address are served one at a time (about 15 ns each).
 // The counters are left at zero; kernels that use it must not overlap on one table.
-__device__ __forceinline__ bool ticket_last(DevState* st) {
+__device__ __forceinline__ bool ticket_last(DevState* st, unsigned nblk) {
   // this thread's atomics and atomic stores are complete before its ticket is taken
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_s_waitcnt(0);
-  unsigned shards = gridDim.x;  // a small grid goes straight to the second level
-  if (gridDim.x > (unsigned)kTicketShards) {
+  unsigned shards = nblk;  // a small grid goes straight to the second level
+  if (nblk > (unsigned)kTicketShards) {
     shards = (unsigned)kTicketShards;
     const unsigned sub = blockIdx.x % shards;
-    const unsigned members = (gridDim.x - sub + shards - 1) / shards;  // workgroups b with b % shards == sub
+    const unsigned members = (nblk - sub + shards - 1) / shards;  // workgroups b with b % shards == sub
     unsigned* c = &st->ticket_sub[sub * 32];
     if (atomicAdd(c, 1u) != members - 1) return false;
     *c = 0;

@@ -84,13 +84,14 @@ __device__ __forceinline__ void scan_spine(unsigned long long* part, uint64_t np
 // table's request. `red`/`fred` hold kBlock/64 words each.
 __device__ __forceinline__ bool scan_pass1_block(unsigned long long s, unsigned flags,
                                                  unsigned long long* __restrict__ part,
-                                                 DevState* st, unsigned long long* red,
-                                                 unsigned* fred, unsigned* s_last) {
+                                                 DevState* st, unsigned nblk,
+                                                 unsigned long long* red, unsigned* fred,
+                                                 unsigned* s_last) {
   block_sum_or(s, flags, red, fred);
   if (threadIdx.x == 0) {
     if (flags) atomicOr(&st->req_flags, flags);
     publish_u64(&part[blockIdx.x], s);
-    *s_last = ticket_last(st) ? 1u : 0u;
+    *s_last = ticket_last(st, nblk) ? 1u : 0u;
   }
   __syncthreads();
   return *s_last != 0u;
@@ -102,10 +103,10 @@ __device__ __forceinline__ bool scan_pass1_block(unsigned long long s, unsigned 
 // one request's flags end and the next begin. Every thread of that workgroup calls it;
 // the facts collected from all workgroups are returned in thread 0.
 __device__ __forceinline__ unsigned scan_pass1_last(unsigned long long* part, DevState* st,
-                                                    unsigned long long epoch,
+                                                    unsigned nblk, unsigned long long epoch,
                                                     unsigned long long* red,
                                                     unsigned long long* carry_s) {
-  scan_spine(part, gridDim.x, red, carry_s);
+  scan_spine(part, nblk, red, carry_s);
   unsigned flags = 0;
   if (threadIdx.x == 0) {
     flags = atomicExch(&st->req_flags, 0u);
@@ -163,8 +164,8 @@ __device__ __forceinline__ void scan_pass2_offsets(const unsigned long long (&v)
 
 // `n_largest`: the longest key list among the tables a launch serves; all of them use one split.
 inline int scan_items(uint64_t n_largest) { return n_largest >= kScanLargeKeys ? kScanItemsLarge : 1; }
-inline uint64_t scan_num_parts(uint64_t n) {
-  const uint64_t chunk = (uint64_t)kBlock * scan_items(n);
+inline uint64_t scan_num_parts(uint64_t n, int items) {
+  const uint64_t chunk = (uint64_t)kBlock * items;
   return (n + chunk - 1) / chunk;
 }
 

@@ -61,7 +61,14 @@ struct StateView {
   unsigned error, req_error, special_present, pad;
 };
 
-__global__ void k_read_state(const DevState* st, StateView* out) {
+// One wavefront per table (blockIdx.x).
+struct StateBatch {
+  const DevState* st[kMaxBatch];
+  StateView* out[kMaxBatch];
+};
+__global__ void k_read_state(StateBatch sb) {
+  const DevState* st = sb.st[blockIdx.x];
+  StateView* out = sb.out[blockIdx.x];
   unsigned long long c = threadIdx.x < kCountShards ? st->count_shard[threadIdx.x * kShardStride] : 0ull;
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
@@ -75,10 +82,17 @@ __global__ void k_read_state(const DevState* st, StateView* out) {
   out->special_present = st->special_present;
 }
 
-// One wavefront, launched behind the kernel of a SCALAR request when the table is close to a
-// limit (the row modes let their lookup kernels write the record).
-__global__ void k_publish(const DevState* st, Snapshot* out, uint64_t seq) {
-  publish_snapshot(st, out, seq);
+// One wavefront per table that asked for a record (blockIdx.x), launched behind the kernel of
+// a SCALAR request when a table is close to a limit (the row modes let their lookup kernels
+// write the record).
+struct PubBatch {
+  const DevState* st[kMaxBatch];
+  Snapshot* out[kMaxBatch];
+  uint64_t seq[kMaxBatch];
+};
+__global__ void k_publish(PubBatch pb) {
+  if (!pb.out[blockIdx.x]) return;
+  publish_snapshot(pb.st[blockIdx.x], pb.out[blockIdx.x], pb.seq[blockIdx.x]);
 }
 
 }  // namespace
@@ -227,10 +241,8 @@ struct Carver {
   static size_t need(size_t count, size_t elem) { return (count * elem + 255) & ~(size_t)255; }
 };
 
-int read_state(pskv_table* t) {
-  k_read_state<<<dim3(1), dim3(64), 0, t->stream>>>(t->st, t->st_host);
-  PSKV_HIP(hipGetLastError());
-  PSKV_HIP(hipStreamSynchronize(t->stream));
+// What the host keeps of a state that k_read_state has just written (the stream is idle).
+void adopt_state(pskv_table* t) {
   const uint64_t c = t->st_host->count;
   t->count = c;
   // everything enqueued so far is complete: the bounds become exact
@@ -238,6 +250,17 @@ int read_state(pskv_table* t) {
   t->base_count = c;
   t->base_top = t->st_host->arena_top;
   t->pend_keys = t->pend_units = 0;
+}
+
+int read_state(pskv_table* t) {
+  StateBatch sb;
+  std::memset(&sb, 0, sizeof(sb));
+  sb.st[0] = t->st;
+  sb.out[0] = t->st_host;
+  k_read_state<<<dim3(1), dim3(64), 0, t->stream>>>(sb);
+  PSKV_HIP(hipGetLastError());
+  PSKV_HIP(hipStreamSynchronize(t->stream));
+  adopt_state(t);
   return PSKV_OK;
 }
 
@@ -383,6 +406,7 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
 }
 
 // ---- request pipeline ------------------------------------------------------------
+// One table's share of a request.
 struct Request {
   bool push, pull;
   const uint64_t* keys;  // device
@@ -400,50 +424,135 @@ struct Request {
   uint64_t small_out_floats;
 };
 
-int run_scalar(pskv_table* t, Request& r) {
-  r.out_nvals = r.pull ? r.n : 0;
-  if (r.n == 0) return PSKV_OK;
+// A request as the kernels see it: the shares of up to kMaxBatch tables that live on one device,
+// work in one mode and run on one stream, served by ONE launch per step of the pipeline. The
+// single-table entry points run a batch of one; pskv_push_multi / pskv_pull_multi hand over all
+// key ranges of a sliced request at once.
+struct Item {
+  pskv_table* t = nullptr;
+  Request r{};
+  TableReq d{};
   PublishReq pub;
-  int rc = reserve(t, r.n, 0, 0, &pub);
-  if (rc) return rc;
-  const dim3 grid(grid_for(r.n, kBlock, kMaxGrid)), block(kBlock);
-  const uint64_t mask = t->cap - 1;
-  if (r.push && r.pull) {
-    launch(t, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, true>, grid, block, t->slots, mask, t->st,
-           r.keys, r.vals, r.out, r.n);
-  } else if (r.push) {
-    launch(t, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, false>, grid, block, t->slots, mask, t->st,
-           r.keys, r.vals, (float*)nullptr, r.n);
-  } else {
-    launch(t, PSKV_KERNEL_PULL_SCALAR, k_scalar<false, true>, grid, block, t->slots, mask, t->st,
-           r.keys, (const float*)nullptr, r.out, r.n);
+  ReqTag tag{};
+  // var-len workspace of the request
+  int32_t* tmp_lens = nullptr;
+  uint64_t nparts = 0, tiles_cap = 0;
+};
+typedef std::vector<Item> Batch;
+
+// The table whose stream the batch runs on and whose launch statistics it is booked to.
+pskv_table* lead_of(Batch& bt) {
+  for (Item& it : bt)
+    if (it.t->prof) return it.t;
+  return bt[0].t;
+}
+
+// One launch for the whole batch: blockIdx.y selects the table, `nblk_of` says how many
+// workgroups serve each (0: none, the table sits this step out).
+template <typename F>
+int launch_batch(Batch& bt, int prof_kernel, void (*kernel)(ReqBatch), F nblk_of) {
+  ReqBatch rb;
+  std::memset(&rb, 0, sizeof(rb));
+  uint64_t gx = 0;
+  for (size_t i = 0; i < bt.size(); ++i) {
+    const uint64_t nb = nblk_of(bt[i]);
+    if (nb > 0x7fffffffull) return set_error(PSKV_EINVAL, "request too large");
+    rb.t[i] = bt[i].d;
+    rb.t[i].nblk = (uint32_t)nb;
+    gx = std::max(gx, nb);
   }
-  if (pub.snap) k_publish<<<dim3(1), dim3(64), 0, t->stream>>>(t->st, pub.snap, pub.seq);
+  if (!gx) return PSKV_OK;
+  launch(lead_of(bt), prof_kernel, kernel, dim3((unsigned)gx, (unsigned)bt.size()), dim3(kBlock), rb);
   PSKV_HIP(hipGetLastError());
   return PSKV_OK;
+}
+
+// The counter records the tables of a batch asked for (reserve), one wavefront each.
+int publish_batch(Batch& bt) {
+  PubBatch pb;
+  std::memset(&pb, 0, sizeof(pb));
+  bool any = false;
+  for (size_t i = 0; i < bt.size(); ++i) {
+    if (!bt[i].pub.snap) continue;
+    pb.st[i] = bt[i].t->st;
+    pb.out[i] = bt[i].pub.snap;
+    pb.seq[i] = bt[i].pub.seq;
+    any = true;
+  }
+  if (!any) return PSKV_OK;
+  k_publish<<<dim3((unsigned)bt.size()), dim3(64), 0, bt[0].t->stream>>>(pb);
+  PSKV_HIP(hipGetLastError());
+  return PSKV_OK;
+}
+
+// The device state of every table of the batch with one launch and one wait.
+int read_state_batch(Batch& bt) {
+  StateBatch sb;
+  std::memset(&sb, 0, sizeof(sb));
+  for (size_t i = 0; i < bt.size(); ++i) {
+    sb.st[i] = bt[i].t->st;
+    sb.out[i] = bt[i].t->st_host;
+  }
+  k_read_state<<<dim3((unsigned)bt.size()), dim3(64), 0, bt[0].t->stream>>>(sb);
+  PSKV_HIP(hipGetLastError());
+  PSKV_HIP(hipStreamSynchronize(bt[0].t->stream));
+  for (Item& it : bt) adopt_state(it.t);
+  return PSKV_OK;
+}
+
+int run_scalar(Batch& bt, bool push, bool pull) {
+  uint64_t n_largest = 0;
+  for (Item& it : bt) {
+    Request& r = it.r;
+    r.out_nvals = pull ? r.n : 0;
+    it.d = TableReq{};
+    if (r.n == 0) continue;
+    int rc = reserve(it.t, r.n, 0, 0, &it.pub);
+    if (rc) return rc;
+    it.d.slots = it.t->slots;
+    it.d.mask = it.t->cap - 1;
+    it.d.st = it.t->st;
+    it.d.keys = r.keys;
+    it.d.vals = r.vals;
+    it.d.out = r.out;
+    it.d.n = r.n;
+    n_largest = std::max(n_largest, r.n);
+  }
+  if (!n_largest) return PSKV_OK;
+  // the kernel strides over a table's keys, so a grid capped at kMaxGrid serves any request
+  const unsigned gx = grid_for(n_largest, kBlock, kMaxGrid);
+  auto nblk = [&](const Item& it) { return it.d.n ? (uint64_t)gx : 0ull; };
+  int rc;
+  if (push && pull) {
+    rc = launch_batch(bt, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, true>, nblk);
+  } else if (push) {
+    rc = launch_batch(bt, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, false>, nblk);
+  } else {
+    rc = launch_batch(bt, PSKV_KERNEL_PULL_SCALAR, k_scalar<false, true>, nblk);
+  }
+  if (rc) return rc;
+  return publish_batch(bt);
 }
 
 // Requests at least this large (4 MiB) are streamed with non-temporal accesses: between two
 // requests of a busy server they do not survive in the caches anyway.
 constexpr uint64_t kStreamFloats = 1u << 20;
 
+// The row kernel over every table of the batch whose TableReq::total is not zero.
 template <bool VARLEN>
-int launch_rows(pskv_table* t, int op, const RowsParams& p) {
-  if (p.total == 0) return PSKV_OK;
+int launch_rows(Batch& bt, int op) {
   const uint64_t tile = VARLEN ? kRowsVarPerBlock : kTileFixed;  // request-side floats per workgroup
-  const uint64_t ntiles = (p.total + tile - 1) / tile;
-  if (ntiles > 0x7fffffffull) return set_error(PSKV_EINVAL, "request too large");
-  const dim3 grid((unsigned)ntiles), block(kBlock);
-  const bool stream = p.total >= kStreamFloats;
+  uint64_t floats = 0;
+  for (const Item& it : bt) floats += it.d.total;
+  if (!floats) return PSKV_OK;
+  auto nblk = [&](const Item& it) { return (it.d.total + tile - 1) / tile; };
+  const bool stream = floats >= kStreamFloats;
   if (op == kOpAcc) {
-    if (stream) launch(t, PSKV_KERNEL_ROWS_ACC, k_rows<kOpAcc, VARLEN, true>, grid, block, p);
-    else launch(t, PSKV_KERNEL_ROWS_ACC, k_rows<kOpAcc, VARLEN, false>, grid, block, p);
-  } else {
-    if (stream) launch(t, PSKV_KERNEL_ROWS_GATHER, k_rows<kOpGather, VARLEN, true>, grid, block, p);
-    else launch(t, PSKV_KERNEL_ROWS_GATHER, k_rows<kOpGather, VARLEN, false>, grid, block, p);
+    if (stream) return launch_batch(bt, PSKV_KERNEL_ROWS_ACC, k_rows<kOpAcc, VARLEN, true>, nblk);
+    return launch_batch(bt, PSKV_KERNEL_ROWS_ACC, k_rows<kOpAcc, VARLEN, false>, nblk);
   }
-  PSKV_HIP(hipGetLastError());
-  return PSKV_OK;
+  if (stream) return launch_batch(bt, PSKV_KERNEL_ROWS_GATHER, k_rows<kOpGather, VARLEN, true>, nblk);
+  return launch_batch(bt, PSKV_KERNEL_ROWS_GATHER, k_rows<kOpGather, VARLEN, false>, nblk);
 }
 
 // Numbers a row-mode request and says whether the key cache has the right shape for it.
@@ -455,71 +564,91 @@ ReqTag next_tag(pskv_table* t, const Request& r) {
   return tag;
 }
 
-// Starts a row-mode request: numbers it and, when the key cache has the right shape, lets the
-// device compare the request with the cached one. Call after every buffer the cache lives in
-// has been grown for this request.
-int begin_row_request(pskv_table* t, const Request& r, bool with_lens, ReqTag* tag) {
-  *tag = next_tag(t, r);
-  if (tag->try_cache) {
-    k_same_keys<<<dim3((unsigned)((r.n + kBlock * 4 - 1) / (kBlock * 4))), dim3(kBlock), 0, t->stream>>>(
-        r.keys, with_lens ? r.lens : nullptr, static_cast<const uint64_t*>(t->cache_keys.ptr),
-        with_lens ? static_cast<const int32_t*>(t->cache_lens.ptr) : nullptr, r.n, t->st, *tag);
-    PSKV_HIP(hipGetLastError());
+// Starts a row-mode request on every table with keys: numbers it and, where the key cache has
+// the right shape, lets the device compare the request with the cached one. Call after every
+// buffer the cache lives in has been grown for this request.
+int begin_row_request(Batch& bt) {
+  for (Item& it : bt) {
+    if (!it.r.n) continue;
+    it.tag = next_tag(it.t, it.r);
+    it.d.tag = it.tag;
   }
-  return PSKV_OK;
+  return launch_batch(bt, -1, k_same_keys, [](const Item& it) {
+    return (it.r.n && it.tag.try_cache) ? (it.r.n + kBlock * kSameKeysItems - 1) / (kBlock * kSameKeysItems)
+                                        : 0ull;
+  });
 }
 
-int run_fixed(pskv_table* t, Request& r) {
-  const uint64_t k = t->row_len;
-  r.out_nvals = r.pull ? r.n * k : 0;
-  if (r.n == 0) return PSKV_OK;
-  PublishReq pub;
-  int rc = reserve(t, r.n, r.n, k, &pub);
-  if (rc) return rc;
-  rc = grow(t, &t->ws, Carver::need(r.n, sizeof(uint64_t)));
-  if (rc) return rc;
-  rc = grow(t, &t->cache_keys, r.n * sizeof(uint64_t));
-  if (rc) return rc;
-  Carver c(t->ws.ptr);
-  uint64_t* ref = c.take<uint64_t>(r.n);
-  uint64_t* cache_keys = static_cast<uint64_t*>(t->cache_keys.ptr);
-  ReqTag tag;
-  rc = begin_row_request(t, r, false, &tag);
-  if (rc) return rc;
-  if (r.n >= kLookupLargeKeys) {
-    launch(t, PSKV_KERNEL_LOOKUP, k_lookup_fixed<kLookupItemsLarge>,
-           dim3(grid_for(r.n, kBlock * kLookupItemsLarge, kMaxGrid)), dim3(kBlock), t->slots,
-           t->cap - 1, t->st, r.keys, r.n, ref, cache_keys, tag, pub.snap, pub.seq);
-  } else {
-    launch(t, PSKV_KERNEL_LOOKUP, k_lookup_fixed<1>, dim3(grid_for(r.n, kBlock, kMaxGrid)),
-           dim3(kBlock), t->slots, t->cap - 1, t->st, r.keys, r.n, ref, cache_keys, tag, pub.snap,
-           pub.seq);
+int run_fixed(Batch& bt, bool push, bool pull) {
+  uint64_t n_largest = 0;
+  for (Item& it : bt) {
+    pskv_table* t = it.t;
+    Request& r = it.r;
+    const uint64_t k = t->row_len;
+    r.out_nvals = pull ? r.n * k : 0;
+    it.d = TableReq{};
+    if (r.n == 0) continue;
+    int rc = reserve(t, r.n, r.n, k, &it.pub);
+    if (rc) return rc;
+    rc = grow(t, &t->ws, Carver::need(r.n, sizeof(uint64_t)));
+    if (rc) return rc;
+    rc = grow(t, &t->cache_keys, r.n * sizeof(uint64_t));
+    if (rc) return rc;
+    Carver c(t->ws.ptr);
+    TableReq& d = it.d;
+    d.slots = t->slots;
+    d.mask = t->cap - 1;
+    d.st = t->st;
+    d.keys = r.keys;
+    d.n = r.n;
+    d.arena = t->arena;
+    d.ref = c.take<uint64_t>(r.n);
+    d.cache_keys = static_cast<uint64_t*>(t->cache_keys.ptr);
+    d.snap = it.pub.snap;
+    d.snap_seq = it.pub.seq;
+    d.k = k;
+    n_largest = std::max(n_largest, r.n);
   }
-  PSKV_HIP(hipGetLastError());
-  // push and pull both create absent keys, so either leaves references for all n keys behind
-  t->cache_valid = true;
-  t->cache_n = r.n;
-  t->cache_nvals = r.n * k;
-  RowsParams p{};
-  p.arena = t->arena;
-  p.ref = ref;
-  p.st = t->st;
-  p.n = r.n;
-  p.total = r.n * k;
-  p.k = k;
-  p.tag = tag;
-  if (r.push) {
-    p.req = const_cast<float*>(r.vals);
-    p.force_scalar = ((k & 3) || (reinterpret_cast<uintptr_t>(r.vals) & 15)) ? 1u : 0u;
-    p.ignore_new = 0;
-    rc = launch_rows<false>(t, kOpAcc, p);
+  if (!n_largest) return PSKV_OK;
+  int rc = begin_row_request(bt);
+  if (rc) return rc;
+  if (n_largest >= kLookupLargeKeys) {
+    rc = launch_batch(bt, PSKV_KERNEL_LOOKUP, k_lookup_fixed<kLookupItemsLarge>, [](const Item& it) {
+      return it.r.n ? (uint64_t)grid_for(it.r.n, kBlock * kLookupItemsLarge, kMaxGrid) : 0ull;
+    });
+  } else {
+    rc = launch_batch(bt, PSKV_KERNEL_LOOKUP, k_lookup_fixed<1>, [](const Item& it) {
+      return it.r.n ? (uint64_t)grid_for(it.r.n, kBlock, kMaxGrid) : 0ull;
+    });
+  }
+  if (rc) return rc;
+  for (Item& it : bt) {
+    if (!it.r.n) continue;
+    // push and pull both create absent keys, so either leaves references for all n keys behind
+    it.t->cache_valid = true;
+    it.t->cache_n = it.r.n;
+    it.t->cache_nvals = it.r.n * it.d.k;
+  }
+  if (push) {
+    for (Item& it : bt) {
+      if (!it.r.n) continue;
+      it.d.req = const_cast<float*>(it.r.vals);
+      it.d.total = it.r.n * it.d.k;
+      it.d.force_scalar = ((it.d.k & 3) || (reinterpret_cast<uintptr_t>(it.r.vals) & 15)) ? 1u : 0u;
+      it.d.ignore_new = 0;
+    }
+    rc = launch_rows<false>(bt, kOpAcc);
     if (rc) return rc;
   }
-  if (r.pull) {
-    p.req = r.out;
-    p.force_scalar = ((k & 3) || (reinterpret_cast<uintptr_t>(r.out) & 15)) ? 1u : 0u;
-    p.ignore_new = r.push ? 1u : 0u;
-    rc = launch_rows<false>(t, kOpGather, p);
+  if (pull) {
+    for (Item& it : bt) {
+      if (!it.r.n) continue;
+      it.d.req = it.r.out;
+      it.d.total = it.r.n * it.d.k;
+      it.d.force_scalar = ((it.d.k & 3) || (reinterpret_cast<uintptr_t>(it.r.out) & 15)) ? 1u : 0u;
+      it.d.ignore_new = push ? 1u : 0u;
+    }
+    rc = launch_rows<false>(bt, kOpGather);
     if (rc) return rc;
   }
   return PSKV_OK;
@@ -534,154 +663,182 @@ int grow_tile_tables(pskv_table* t, uint64_t floats, uint64_t* ntiles_cap) {
 }
 
 // The kernels of a var-len request that work key by key: one workgroup per kBlock*items keys,
-// `items` per thread, the same split in every kernel of the request (the scan's
-// per-workgroup totals are indexed by it).
-template <typename K1, typename K4, typename... Args>
-void launch_keys(pskv_table* t, int prof_kernel, uint64_t n, K1 k1, K4 k4, Args... args) {
-  const dim3 grid((unsigned)scan_num_parts(n)), block(kBlock);
-  if (scan_items(n) == kScanItemsLarge) {
-    launch(t, prof_kernel, k4, grid, block, args...);
-  } else {
-    launch(t, prof_kernel, k1, grid, block, args...);
-  }
+// `items` per thread, the same split in every kernel of the request and for every table of the
+// batch (the scan's per-workgroup totals are indexed by it).
+int launch_keys(Batch& bt, int prof_kernel, int items, void (*k1)(ReqBatch), void (*k4)(ReqBatch)) {
+  return launch_batch(bt, prof_kernel, items == kScanItemsLarge ? k4 : k1,
+                      [](const Item& it) { return it.r.n ? it.nparts : 0ull; });
 }
 
-// Pass 2 of a pull's scan: the request-side offsets of the response and the tile table for
-// `floats` floats of room (the row kernel fills the other table).
-int make_tile_tables(pskv_table* t, const int32_t* lens_out, const unsigned long long* part,
-                     uint64_t* off, uint64_t n, uint64_t floats, RowsParams* p, const ReqTag& tag) {
-  uint64_t ntiles_cap = 0;
-  int rc = grow_tile_tables(t, floats, &ntiles_cap);
-  if (rc) return rc;
-  uint32_t* tk = static_cast<uint32_t*>(t->tiles.ptr);
-  launch_keys(t, -1, n, k_var_offsets<1>, k_var_offsets<kScanItemsLarge>, lens_out, n, part, off, tk,
-              ntiles_cap, (uint64_t)kTileVar, (const DevState*)t->st, tag);
-  PSKV_HIP(hipGetLastError());
-  p->tile_key = tk;
-  p->tile_aff = static_cast<TileNote*>(t->tiles_aff.ptr);
-  return PSKV_OK;
+// Pass 2 of a pull's scan for every table with a response: the request-side offsets of the
+// response and the tile table for Item::d.total floats of room (the row kernel fills the other
+// table).
+int make_tile_tables(Batch& bt, int items) {
+  for (Item& it : bt) {
+    if (!it.d.total) continue;
+    uint64_t ntiles_cap = 0;
+    int rc = grow_tile_tables(it.t, it.d.total, &ntiles_cap);
+    if (rc) return rc;
+    it.d.tile_key = static_cast<uint32_t*>(it.t->tiles.ptr);
+    it.d.tile_aff = static_cast<TileNote*>(it.t->tiles_aff.ptr);
+    it.d.ntiles = ntiles_cap;
+  }
+  return launch_batch(bt, -1, items == kScanItemsLarge ? k_var_offsets<kScanItemsLarge> : k_var_offsets<1>,
+                      [](const Item& it) { return (it.r.n && it.d.total) ? it.nparts : 0ull; });
 }
 
 // Launches per var-len request: a push takes three (compare + scan pass 1; scan pass 2 +
 // find-or-create + counter record; rows), a pull four (compare; stored lengths + scan pass 1;
-// scan pass 2 + tile table; rows).
-int run_varlen(pskv_table* t, Request& r) {
-  r.out_nvals = 0;
-  if (r.n == 0) return PSKV_OK;
-  if (r.n > 0xfffffffeull) return set_error(PSKV_EINVAL, "too many keys in one request");
-  const uint64_t nparts = scan_num_parts(r.n);
-  const size_t need = Carver::need(r.n, 8) + Carver::need(r.n + 1, 8) + Carver::need(nparts, 8) +
-                      Carver::need(r.n, 4);
-  // Every buffer the key cache lives in is grown BEFORE the request is compared with the
-  // cached one: a reallocation loses the cached contents and must rule the fast path out.
-  int rc = grow(t, &t->ws, need);
-  if (rc) return rc;
-  rc = grow(t, &t->cache_keys, r.n * sizeof(uint64_t));
-  if (rc) return rc;
-  rc = grow(t, &t->cache_lens, r.n * sizeof(int32_t));
-  if (rc) return rc;
-  const bool async_pull = r.pull && !r.push && !r.need_total;
-  const uint64_t tiles_for = r.push ? r.nvals : (async_pull ? r.out_cap : 0);
-  uint64_t tiles_cap = 0;
-  rc = grow_tile_tables(t, tiles_for, &tiles_cap);
-  if (rc) return rc;
-
-  Carver c(t->ws.ptr);
-  uint64_t* ref = c.take<uint64_t>(r.n);
-  uint64_t* off = c.take<uint64_t>(r.n + 1);
-  unsigned long long* part = c.take<unsigned long long>(nparts);
-  int32_t* tmp_lens = c.take<int32_t>(r.n);
-  uint64_t* cache_keys = static_cast<uint64_t*>(t->cache_keys.ptr);
-  int32_t* cache_lens = static_cast<int32_t*>(t->cache_lens.ptr);
-
-  RowsParams p{};
-  p.ref = ref;
-  p.off = off;
-  p.st = t->st;
-  p.n = r.n;
-
-  if (r.push) {
-    PublishReq pub;
-    // every key may round its row up to a 16-byte unit, every workgroup may pad its rows' start
-    rc = reserve(t, r.n, r.nvals / 4 + r.n + kArenaPadUnits * nparts, 4, &pub);
-    if (rc) return rc;
-    if (t->cache_nvals != r.nvals) t->cache_valid = false;  // same lens would mean the same total
-    const ReqTag tag = next_tag(t, r);
-    launch_keys(t, -1, r.n, k_var_push_begin<1>, k_var_push_begin<kScanItemsLarge>, r.keys, r.lens, r.n,
-                (const uint64_t*)cache_keys, (const int32_t*)cache_lens, part, t->st,
-                (unsigned)PSKV_MAX_VARLEN_ROW, tag);
-    PSKV_HIP(hipGetLastError());
-    // pass 2 also fills the tile table of the request side (tile sizes are those of nvals; a
-    // request whose lens do not add up to nvals is refused before it gets there)
-    uint32_t* push_tile_key = static_cast<uint32_t*>(t->tiles.ptr);
-    launch_keys(t, PSKV_KERNEL_LOOKUP, r.n, k_var_push_lookup<1>, k_var_push_lookup<kScanItemsLarge>,
-                t->slots, t->cap - 1, t->st, r.keys, r.lens, r.n, r.nvals,
-                (const unsigned long long*)part, off, r.nvals ? push_tile_key : (uint32_t*)nullptr,
-                tiles_cap, (uint64_t)kTileVar, ref, cache_keys, cache_lens, tag, pub.snap, pub.seq);
-    PSKV_HIP(hipGetLastError());
-    t->cache_valid = true;  // whichever way the device decided, the cache now is this request
-    t->cache_n = r.n;
-    t->cache_nvals = r.nvals;
-    if (r.nvals) {
-      p.tile_key = push_tile_key;
-      p.tile_aff = static_cast<TileNote*>(t->tiles_aff.ptr);
-      p.req = const_cast<float*>(r.vals);
-      p.arena = t->arena;
-      p.total = r.nvals;
-      p.force_scalar = (reinterpret_cast<uintptr_t>(r.vals) & 15) ? 1u : 0u;
-      p.ignore_new = 0;
-      p.tag = tag;
-      rc = launch_rows<true>(t, kOpAcc, p);
-      if (rc) return rc;
-    }
+// scan pass 2 + tile table; rows), whatever the number of tables.
+int run_varlen(Batch& bt, bool push, bool pull) {
+  uint64_t n_largest = 0;
+  for (Item& it : bt) {
+    it.r.out_nvals = 0;
+    it.d = TableReq{};
+    if (it.r.n > 0xfffffffeull) return set_error(PSKV_EINVAL, "too many keys in one request");
+    n_largest = std::max(n_largest, it.r.n);
   }
-  if (r.pull) {
-    int32_t* lens_out = r.out_lens ? r.out_lens : tmp_lens;
-    if (r.push) {
+  if (!n_largest) return PSKV_OK;
+  const int items = scan_items(n_largest);
+  const bool async_pull = pull && !push && !bt[0].r.need_total;
+  for (Item& it : bt) {
+    pskv_table* t = it.t;
+    Request& r = it.r;
+    if (!r.n) continue;
+    it.nparts = scan_num_parts(r.n, items);
+    const size_t need = Carver::need(r.n, 8) + Carver::need(r.n + 1, 8) + Carver::need(it.nparts, 8) +
+                        Carver::need(r.n, 4);
+    // Every buffer the key cache lives in is grown BEFORE the request is compared with the
+    // cached one: a reallocation loses the cached contents and must rule the fast path out.
+    int rc = grow(t, &t->ws, need);
+    if (rc) return rc;
+    rc = grow(t, &t->cache_keys, r.n * sizeof(uint64_t));
+    if (rc) return rc;
+    rc = grow(t, &t->cache_lens, r.n * sizeof(int32_t));
+    if (rc) return rc;
+    const uint64_t tiles_for = push ? r.nvals : (async_pull ? r.out_cap : 0);
+    rc = grow_tile_tables(t, tiles_for, &it.tiles_cap);
+    if (rc) return rc;
+    Carver c(t->ws.ptr);
+    TableReq& d = it.d;
+    d.ref = c.take<uint64_t>(r.n);
+    d.off = c.take<uint64_t>(r.n + 1);
+    d.part = c.take<unsigned long long>(it.nparts);
+    it.tmp_lens = c.take<int32_t>(r.n);
+    d.cache_keys = static_cast<uint64_t*>(t->cache_keys.ptr);
+    d.cache_lens = static_cast<int32_t*>(t->cache_lens.ptr);
+    d.keys = r.keys;
+    d.n = r.n;
+    d.st = t->st;
+  }
+
+  if (push) {
+    for (Item& it : bt) {
+      pskv_table* t = it.t;
+      Request& r = it.r;
+      if (!r.n) continue;
+      // every key may round its row up to a 16-byte unit, every workgroup may pad its rows' start
+      int rc = reserve(t, r.n, r.nvals / 4 + r.n + kArenaPadUnits * it.nparts, 4, &it.pub);
+      if (rc) return rc;
+      if (t->cache_nvals != r.nvals) t->cache_valid = false;  // same lens would mean the same total
+      it.tag = next_tag(t, r);
+      TableReq& d = it.d;
+      d.slots = t->slots;
+      d.mask = t->cap - 1;
+      d.arena = t->arena;
+      d.lens = r.lens;
+      d.nvals = r.nvals;
+      d.tag = it.tag;
+      d.snap = it.pub.snap;
+      d.snap_seq = it.pub.seq;
+      // pass 2 also fills the tile table of the request side (tile sizes are those of nvals; a
+      // request whose lens do not add up to nvals is refused before it gets there)
+      d.tile_key = r.nvals ? static_cast<uint32_t*>(t->tiles.ptr) : nullptr;
+      d.tile_aff = static_cast<TileNote*>(t->tiles_aff.ptr);
+      d.ntiles = it.tiles_cap;
+    }
+    int rc = launch_keys(bt, -1, items, k_var_push_begin<1>, k_var_push_begin<kScanItemsLarge>);
+    if (rc) return rc;
+    rc = launch_keys(bt, PSKV_KERNEL_LOOKUP, items, k_var_push_lookup<1>, k_var_push_lookup<kScanItemsLarge>);
+    if (rc) return rc;
+    for (Item& it : bt) {
+      if (!it.r.n) continue;
+      it.t->cache_valid = true;  // whichever way the device decided, the cache now is this request
+      it.t->cache_n = it.r.n;
+      it.t->cache_nvals = it.r.nvals;
+      it.d.req = const_cast<float*>(it.r.vals);
+      it.d.total = it.r.nvals;
+      it.d.force_scalar = (reinterpret_cast<uintptr_t>(it.r.vals) & 15) ? 1u : 0u;
+      it.d.ignore_new = 0;
+      it.d.total_on_device = 0;
+    }
+    rc = launch_rows<true>(bt, kOpAcc);
+    if (rc) return rc;
+  }
+  if (pull) {
+    int rc;
+    if (push) {
       // a refused push must not be followed by its pull half
-      rc = read_state(t);
+      rc = read_state_batch(bt);
       if (rc) return rc;
-      rc = report_device_errors(t);
-      if (rc) return rc;
+      for (Item& it : bt) {
+        rc = report_device_errors(it.t);
+        if (rc) return rc;
+      }
+    }
+    for (Item& it : bt) {
+      if (!it.r.n) continue;
+      it.d.slots = it.t->slots;
+      it.d.mask = it.t->cap - 1;
+      it.d.arena = it.t->arena;
+      it.d.out_lens = it.r.out_lens ? it.r.out_lens : it.tmp_lens;
+      it.d.total = 0;
+      it.d.snap = nullptr;
     }
     // A pull with the keys of the cached push finds every key present with the cached length
     // and reuses its references; any other pull recomputes them and so ends the cache.
-    ReqTag tag;
-    rc = begin_row_request(t, r, false, &tag);
+    rc = begin_row_request(bt);
     if (rc) return rc;
-    if (!tag.try_cache) t->cache_valid = false;
-    launch_keys(t, PSKV_KERNEL_LOOKUP, r.n, k_var_pull_lookup<1>, k_var_pull_lookup<kScanItemsLarge>,
-                (const Slot*)t->slots, t->cap - 1, t->st, r.keys, r.n, ref, lens_out,
-                (const int32_t*)cache_lens, part, tag);
-    PSKV_HIP(hipGetLastError());
-    p.tag = tag;
+    for (Item& it : bt)
+      if (it.r.n && !it.tag.try_cache) it.t->cache_valid = false;
+    rc = launch_keys(bt, PSKV_KERNEL_LOOKUP, items, k_var_pull_lookup<1>, k_var_pull_lookup<kScanItemsLarge>);
+    if (rc) return rc;
     if (async_pull) {
       // No host round trip: the grid covers the caller's buffer, the kernels take the real
       // size from the scan, and a response that does not fit is reported by the next sync.
-      if (r.out_cap) {
-        if (!r.out) return set_error(PSKV_EINVAL, "null out");
-        rc = make_tile_tables(t, lens_out, part, off, r.n, r.out_cap, &p, tag);
-        if (rc) return rc;
-        p.req = r.out;
-        p.arena = t->arena;
-        p.total = r.out_cap;
-        p.total_on_device = 1;
-        p.force_scalar = (reinterpret_cast<uintptr_t>(r.out) & 15) ? 1u : 0u;
-        p.ignore_new = 1;
-        rc = launch_rows<true>(t, kOpGather, p);
-        if (rc) return rc;
+      for (Item& it : bt) {
+        if (!it.r.n || !it.r.out_cap) continue;
+        if (!it.r.out) return set_error(PSKV_EINVAL, "null out");
+        it.d.req = it.r.out;
+        it.d.total = it.r.out_cap;
+        it.d.total_on_device = 1;
+        it.d.force_scalar = (reinterpret_cast<uintptr_t>(it.r.out) & 15) ? 1u : 0u;
+        it.d.ignore_new = 1;
       }
-      return PSKV_OK;
+      rc = make_tile_tables(bt, items);
+      if (rc) return rc;
+      return launch_rows<true>(bt, kOpGather);
     }
-    rc = read_state(t);  // the response size is data dependent
+    rc = read_state_batch(bt);  // the response sizes are data dependent
     if (rc) return rc;
-    if (t->st_host->same_epoch != tag.epoch) t->cache_valid = false;  // the pull recomputed the workspace
-    const uint64_t total = t->st_host->scan_total;
-    r.out_nvals = total;
-    if (total > r.out_cap)
-      return set_error(PSKV_ESIZE_MISMATCH, "response needs %llu floats, buffer holds %llu",
-                       (unsigned long long)total, (unsigned long long)r.out_cap);
-    if (total) {
+    int fit = PSKV_OK;
+    for (Item& it : bt) {
+      pskv_table* t = it.t;
+      Request& r = it.r;
+      if (!r.n) continue;
+      if (t->st_host->same_epoch != it.tag.epoch) t->cache_valid = false;  // the pull recomputed the workspace
+      const uint64_t total = t->st_host->scan_total;
+      r.out_nvals = total;
+      if (total > r.out_cap && !fit)
+        fit = set_error(PSKV_ESIZE_MISMATCH, "response needs %llu floats, buffer holds %llu",
+                        (unsigned long long)total, (unsigned long long)r.out_cap);
+    }
+    if (fit) return fit;
+    for (Item& it : bt) {
+      pskv_table* t = it.t;
+      Request& r = it.r;
+      const uint64_t total = r.n ? r.out_nvals : 0;
+      if (!total) continue;
       if (r.lazy_out) {
         if (r.small_out && total <= r.small_out_floats) {
           r.out = reinterpret_cast<float*>(r.small_out);
@@ -692,18 +849,26 @@ int run_varlen(pskv_table* t, Request& r) {
         }
       }
       if (!r.out) return set_error(PSKV_EINVAL, "null out");
-      rc = make_tile_tables(t, lens_out, part, off, r.n, total, &p, tag);
-      if (rc) return rc;
-      p.req = r.out;
-      p.arena = t->arena;
-      p.total = total;
-      p.force_scalar = (reinterpret_cast<uintptr_t>(r.out) & 15) ? 1u : 0u;
-      p.ignore_new = 1;
-      rc = launch_rows<true>(t, kOpGather, p);
-      if (rc) return rc;
+      it.d.req = r.out;
+      it.d.total = total;
+      it.d.total_on_device = 0;
+      it.d.force_scalar = (reinterpret_cast<uintptr_t>(r.out) & 15) ? 1u : 0u;
+      it.d.ignore_new = 1;
     }
+    rc = make_tile_tables(bt, items);
+    if (rc) return rc;
+    rc = launch_rows<true>(bt, kOpGather);
+    if (rc) return rc;
   }
   return PSKV_OK;
+}
+
+int run_batch(Batch& bt, bool push, bool pull) {
+  switch (bt[0].t->mode) {
+    case PSKV_MODE_SCALAR: return run_scalar(bt, push, pull);
+    case PSKV_MODE_FIXED: return run_fixed(bt, push, pull);
+    default: return run_varlen(bt, push, pull);
+  }
 }
 
 // Host-side checks that mirror the CHECKs of the reference and the frozen rules of
@@ -851,10 +1016,12 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
     r.out_cap = fixed_out;
   }
 
-  switch (t->mode) {
-    case PSKV_MODE_SCALAR: rc = run_scalar(t, r); break;
-    case PSKV_MODE_FIXED: rc = run_fixed(t, r); break;
-    default: rc = run_varlen(t, r); break;
+  {
+    Batch bt(1);
+    bt[0].t = t;
+    bt[0].r = r;
+    rc = run_batch(bt, push, pull);
+    r = bt[0].r;
   }
   if (out_nvals) *out_nvals = r.out_nvals;
   // Kernels of this request may still be reading the pinned request buffer, which the next
@@ -892,6 +1059,116 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
     if (pull && varlen && out_lens && n && lens_pinned) std::memcpy(out_lens, r.out_lens, n * 4);
   }
   return PSKV_OK;
+}
+
+// Tables that one launch can serve together: one device, one mode, one stream.
+int check_group(pskv_table* const* tables, size_t S) {
+  if (!tables && S) return set_error(PSKV_EINVAL, "null table list");
+  for (size_t s = 0; s < S; ++s) {
+    if (!tables[s]) return set_error(PSKV_EINVAL, "tables[%zu] is null", s);
+    if (tables[s]->device != tables[0]->device || tables[s]->mode != tables[0]->mode)
+      return set_error(PSKV_EINVAL, "tables[%zu] differs from tables[0] in device or mode", s);
+    if (tables[s]->stream != tables[0]->stream)
+      return set_error(PSKV_EINVAL,
+                       "tables[%zu] runs on a stream of its own: create the tables of a group with "
+                       "pskv_opts.stream = pskv_table_stream(first table)", s);
+    for (size_t q = 0; q < s; ++q)
+      if (tables[q] == tables[s]) return set_error(PSKV_EINVAL, "tables[%zu] is tables[%zu]", s, q);
+  }
+  return PSKV_OK;
+}
+
+// pskv_push_multi / pskv_pull_multi: slice s of the request, keys [pos[s], pos[s+1]), goes to
+// tables[s]; slices without keys are skipped as KVWorker::Send skips them (kv_app.h:590-595).
+int request_multi(pskv_table* const* tables, size_t S, bool push, const uint64_t* keys,
+                  const uint64_t* pos, const float* vals, const uint64_t* val_pos, const int32_t* lens,
+                  float* out, const uint64_t* out_pos, int32_t* out_lens, uint64_t* out_nvals,
+                  int memkind) {
+  clear_error();
+  const bool pull = !push;
+  if (memkind != PSKV_MEM_DEVICE)
+    return set_error(PSKV_EINVAL, "the multi-table entry points take device-resident buffers "
+                                  "(PSKV_MEM_DEVICE); host-resident requests go table by table");
+  if (out_nvals)
+    for (size_t s = 0; s < S; ++s) out_nvals[s] = 0;
+  if (S == 0) return PSKV_OK;
+  int rc = check_group(tables, S);
+  if (rc) return rc;
+  if (!pos) return set_error(PSKV_EINVAL, "null pos");
+  const int mode = tables[0]->mode;
+  const bool varlen = mode == PSKV_MODE_VARLEN;
+  if (pos[S] != pos[0] && !keys) return set_error(PSKV_EINVAL, "null keys");
+  if (push && !val_pos) return set_error(PSKV_EINVAL, "null val_pos");
+  if (pull && varlen && !out_pos) return set_error(PSKV_EINVAL, "a var-len pull needs out_pos");
+  // everything the host can check, for every slice, before anything is enqueued
+  std::vector<Request> reqs(S);
+  for (size_t s = 0; s < S; ++s) {
+    if (pos[s + 1] < pos[s]) return set_error(PSKV_EINVAL, "pos[%zu] > pos[%zu]", s, s + 1);
+    Request& r = reqs[s];
+    r = Request{};
+    r.push = push;
+    r.pull = pull;
+    r.n = pos[s + 1] - pos[s];
+    r.keys = keys + pos[s];
+    if (push) {
+      if (val_pos[s + 1] < val_pos[s]) return set_error(PSKV_EINVAL, "val_pos[%zu] > val_pos[%zu]", s, s + 1);
+      r.nvals = val_pos[s + 1] - val_pos[s];
+      r.vals = vals + val_pos[s];
+      r.lens = (varlen && lens) ? lens + pos[s] : nullptr;
+      if (r.nvals && !vals) return set_error(PSKV_EINVAL, "null vals");
+    }
+    if (!r.n) {
+      if (r.nvals) return set_error(PSKV_ESIZE_MISMATCH, "slice %zu has values but no keys", s);
+      continue;
+    }
+    rc = validate(tables[s], push, pull, r.n, r.nvals, r.lens, varlen && push ? r.n : 0, memkind);
+    if (rc) return rc;
+    if (pull) {
+      const uint64_t k = mode == PSKV_MODE_SCALAR ? 1 : tables[s]->row_len;
+      const uint64_t at = out_pos ? out_pos[s] : pos[s] * k;
+      if (out_pos && out_pos[s + 1] < out_pos[s])
+        return set_error(PSKV_EINVAL, "out_pos[%zu] > out_pos[%zu]", s, s + 1);
+      r.out_cap = out_pos ? out_pos[s + 1] - out_pos[s] : r.n * k;
+      r.out = out ? out + at : nullptr;
+      if (!varlen) {
+        if (r.out_cap < r.n * k)
+          return set_error(PSKV_ESIZE_MISMATCH, "slice %zu answers %llu floats, out_pos leaves room for %llu",
+                           s, (unsigned long long)(r.n * k), (unsigned long long)r.out_cap);
+        if (!r.out) return set_error(PSKV_EINVAL, "null out");
+      } else {
+        r.out_lens = out_lens ? out_lens + pos[s] : nullptr;
+        r.need_total = out_nvals != nullptr;
+      }
+    }
+  }
+  DeviceGuard guard(tables[0]->device);
+  if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", tables[0]->device);
+  Batch bt;
+  std::vector<size_t> who;
+  auto flush = [&]() -> int {
+    if (bt.empty()) return PSKV_OK;
+    const int r = run_batch(bt, push, pull);
+    for (size_t i = 0; i < bt.size(); ++i) {
+      if (out_nvals) out_nvals[who[i]] = bt[i].r.out_nvals;
+      if (r) bt[i].t->cache_valid = false;
+    }
+    bt.clear();
+    who.clear();
+    return r;
+  };
+  for (size_t s = 0; s < S; ++s) {
+    if (!reqs[s].n) continue;
+    Item it;
+    it.t = tables[s];
+    it.r = reqs[s];
+    bt.push_back(it);
+    who.push_back(s);
+    if (bt.size() == (size_t)kMaxBatch) {
+      rc = flush();
+      if (rc) return rc;
+    }
+  }
+  return flush();
 }
 
 }  // namespace
@@ -1009,6 +1286,46 @@ int pskv_pushpull(pskv_table* t, const uint64_t* keys, size_t n, const float* va
                   int32_t* out_lens, size_t* out_nvals, int memkind) {
   return request(t, true, true, keys, n, vals, nvals, lens, nlens, out, out_cap, out_lens,
                  out_nvals, memkind);
+}
+
+void* pskv_table_stream(pskv_table* t) { return t ? static_cast<void*>(t->stream) : nullptr; }
+
+int pskv_push_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, const uint64_t* pos,
+                    const float* vals, const uint64_t* val_pos, const int32_t* lens, int memkind) {
+  return request_multi(tables, S, true, keys, pos, vals, val_pos, lens, nullptr, nullptr, nullptr,
+                       nullptr, memkind);
+}
+
+int pskv_pull_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, const uint64_t* pos,
+                    float* out, const uint64_t* out_pos, int32_t* out_lens, uint64_t* out_nvals,
+                    int memkind) {
+  return request_multi(tables, S, false, keys, pos, nullptr, nullptr, nullptr, out, out_pos, out_lens,
+                       out_nvals, memkind);
+}
+
+int pskv_sync_multi(pskv_table* const* tables, size_t S) {
+  clear_error();
+  if (S == 0) return PSKV_OK;
+  int rc = check_group(tables, S);
+  if (rc) return rc;
+  DeviceGuard guard(tables[0]->device);
+  int first = PSKV_OK;
+  std::string first_text;
+  for (size_t at = 0; at < S; at += kMaxBatch) {
+    Batch bt(std::min<size_t>(S - at, kMaxBatch));
+    for (size_t i = 0; i < bt.size(); ++i) bt[i].t = tables[at + i];
+    rc = read_state_batch(bt);
+    if (rc) return rc;
+    for (Item& it : bt) {
+      rc = report_device_errors(it.t);  // every table's error bits are cleared; the first is reported
+      if (rc && !first) {
+        first = rc;
+        first_text = pskv_last_error();
+      }
+    }
+  }
+  if (first) return set_error(first, "%s", first_text.c_str());
+  return PSKV_OK;
 }
 
 int pskv_sync(pskv_table* t) {

@@ -12,6 +12,49 @@
 
 namespace pskv {
 
+// What the kernels of a request need to know about ONE table's share of it. A launch carries up
+// to kMaxBatch of these by value (blockIdx.y selects one), so that a request which the slicer
+// has cut into per-server pieces (kv_app.h:562-612) costs one launch per step and not one per
+// server; the single-table entry points launch with one of them.
+struct TableReq {
+  Slot* slots;
+  uint64_t mask;
+  DevState* st;
+  const uint64_t* keys;  // n sorted unique keys
+  const int32_t* lens;   // VARLEN push: n row lengths
+  const float* vals;     // SCALAR push: n values
+  float* out;            // SCALAR pull: n values
+  uint64_t n;
+  uint64_t nvals;        // VARLEN push: floats pushed
+  // row modes
+  float* arena;              // row storage
+  uint64_t* ref;             // n row references, written by the lookup kernel
+  uint64_t* off;             // VARLEN: n+1 request-side row offsets in floats
+  unsigned long long* part;  // VARLEN: per-workgroup totals of the lens scan
+  uint32_t* tile_key;        // VARLEN: first key of every request-side tile, ntiles+1 entries
+  TileNote* tile_aff;        // VARLEN: one note per tile
+  uint64_t ntiles;           // VARLEN: tiles of the request (push) / room in the tile table (pull)
+  uint64_t* cache_keys;      // keys (and lens) of the request whose references the workspace holds
+  int32_t* cache_lens;
+  int32_t* out_lens;         // VARLEN pull: n answered lengths
+  Snapshot* snap;            // where the kernel that creates the request's keys leaves the counters
+  uint64_t snap_seq;
+  ReqTag tag;
+  // row kernels
+  float* req;             // push: request values (read); pull: response values (written)
+  uint64_t total;         // floats in req
+  uint64_t k;             // FIXED: floats per row
+  uint32_t force_scalar;  // request buffer or k not 16-byte friendly
+  uint32_t ignore_new;    // pull half of a push+pull: rows created by the push half hold data
+  uint32_t total_on_device;  // VARLEN pull without a host round trip: the floats to move are
+                             // DevState::scan_total and `total` is the room in req
+  uint32_t nblk;          // workgroups of the launch in flight that serve this table
+};
+struct ReqBatch {
+  TableReq t[kMaxBatch];
+};
+static_assert(sizeof(ReqBatch) <= 3840, "kernel arguments are limited to 4 KiB");
+
 // ---------------------------------------------------------------------------------
 // SCALAR mode: one float per key, kept in the low word of the slot payload so that a
 // probe reads key and value with one 128-bit load.
@@ -28,11 +71,16 @@ namespace pskv {
 // that repeats a key remains a caller error with an unspecified sum.
 // ---------------------------------------------------------------------------------
 template <bool PUSH, bool PULL>
-__global__ __launch_bounds__(kBlock) void k_scalar(Slot* __restrict__ slots, uint64_t mask,
-                                                  DevState* st,
-                                                  const uint64_t* __restrict__ keys,
-                                                  const float* __restrict__ vals,
-                                                  float* __restrict__ out, uint64_t n) {
+__global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
+  const TableReq& d = b.t[blockIdx.y];
+  const uint64_t n = d.n;
+  if ((uint64_t)blockIdx.x * kBlock >= n) return;  // the grid is sized for the longest key list
+  Slot* __restrict__ slots = d.slots;
+  const uint64_t mask = d.mask;
+  DevState* st = d.st;
+  const uint64_t* __restrict__ keys = d.keys;
+  const float* __restrict__ vals = d.vals;
+  float* __restrict__ out = d.out;
   __shared__ unsigned red[kBlock / 64];
   unsigned created = 0;
   const uint64_t stride = (uint64_t)gridDim.x * kBlock;
@@ -91,35 +139,36 @@ __device__ __forceinline__ void decide_same(DevState* st, const ReqTag& tag, boo
   }
 }
 
-// Compares a request with the cached one (keys, and lens when given) and reaches the decision
-// for the whole request: the workgroup that finishes last sees whether any workgroup found a
-// difference and writes same_epoch.
-__global__ __launch_bounds__(kBlock) void k_same_keys(const uint64_t* __restrict__ keys,
-                                                     const int32_t* __restrict__ lens,
-                                                     const uint64_t* __restrict__ cache_keys,
-                                                     const int32_t* __restrict__ cache_lens,
-                                                     uint64_t n, DevState* st, ReqTag tag) {
+// Compares the keys of a request with the cached ones and reaches the decision for the whole
+// request: the workgroup that finishes last sees whether any workgroup found a difference and
+// writes same_epoch. (A var-len push, whose lens count as well, compares in k_var_push_begin.)
+constexpr int kSameKeysItems = 4;
+__global__ __launch_bounds__(kBlock) void k_same_keys(ReqBatch b) {
+  const TableReq& d = b.t[blockIdx.y];
+  if (blockIdx.x >= d.nblk) return;  // tables that have nothing to compare have no workgroups
+  const uint64_t* __restrict__ keys = d.keys;
+  const uint64_t* __restrict__ cache_keys = d.cache_keys;
+  const uint64_t n = d.n;
+  DevState* st = d.st;
+  const ReqTag tag = d.tag;
   __shared__ unsigned s_last;
-  constexpr int kItems = 4;
+  constexpr int kItems = kSameKeysItems;
   const uint64_t base = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * kItems;
   // all loads first, then the compares
-  uint64_t a[kItems], b[kItems];
-  int32_t la[kItems], lb[kItems];
+  uint64_t a[kItems], c[kItems];
 #pragma unroll
   for (int j = 0; j < kItems; ++j) {
     const bool in = base + j < n;
     a[j] = in ? keys[base + j] : 0;
-    b[j] = in ? cache_keys[base + j] : 0;
-    la[j] = in && lens ? lens[base + j] : 0;
-    lb[j] = in && lens ? cache_lens[base + j] : 0;
+    c[j] = in ? cache_keys[base + j] : 0;
   }
   bool differ = false;
 #pragma unroll
-  for (int j = 0; j < kItems; ++j) differ |= (a[j] != b[j]) | (la[j] != lb[j]);
+  for (int j = 0; j < kItems; ++j) differ |= a[j] != c[j];
   const int any = __syncthreads_or(differ ? 1 : 0);
   if (threadIdx.x == 0) {
     if (any) atomicOr(&st->req_flags, kReqDiffer);
-    s_last = ticket_last(st) ? 1u : 0u;
+    s_last = ticket_last(st, d.nblk) ? 1u : 0u;
   }
   __syncthreads();
   if (!s_last) return;
@@ -131,9 +180,9 @@ __global__ __launch_bounds__(kBlock) void k_same_keys(const uint64_t* __restrict
 // holds the counters as they are AFTER the request. Every thread of the workgroup calls it;
 // `s_last` is one word of LDS.
 __device__ __forceinline__ void publish_after_lookup(DevState* st, Snapshot* snap, uint64_t seq,
-                                                     unsigned* s_last) {
+                                                     unsigned nblk, unsigned* s_last) {
   if (!snap) return;
-  if (threadIdx.x == 0) *s_last = ticket_last(st) ? 1u : 0u;
+  if (threadIdx.x == 0) *s_last = ticket_last(st, nblk) ? 1u : 0u;
   __syncthreads();
   if (*s_last && threadIdx.x < 64) publish_snapshot(st, snap, seq);
 }
@@ -158,13 +207,20 @@ __device__ __forceinline__ void refuse_fixed(DevState* st, const ReqTag& tag) {
 }
 
 template <int kLookupItems>
-__global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slots, uint64_t mask,
-                                                        DevState* st,
-                                                        const uint64_t* __restrict__ keys,
-                                                        uint64_t n, uint64_t* __restrict__ ref,
-                                                        uint64_t* __restrict__ cache_keys,
-                                                        ReqTag tag, Snapshot* snap,
-                                                        uint64_t snap_seq) {
+__global__ __launch_bounds__(kBlock) void k_lookup_fixed(ReqBatch b) {
+  const TableReq& d = b.t[blockIdx.y];
+  const unsigned nblk = d.nblk;
+  if (blockIdx.x >= nblk) return;
+  Slot* __restrict__ slots = d.slots;
+  const uint64_t mask = d.mask;
+  DevState* st = d.st;
+  const uint64_t* __restrict__ keys = d.keys;
+  const uint64_t n = d.n;
+  uint64_t* __restrict__ ref = d.ref;
+  uint64_t* __restrict__ cache_keys = d.cache_keys;
+  const ReqTag tag = d.tag;
+  Snapshot* snap = d.snap;
+  const uint64_t snap_seq = d.snap_seq;
   if (cache_same(st, tag)) {  // the references of the cached request are this request's
     if (snap && blockIdx.x == 0 && threadIdx.x < 64) publish_snapshot(st, snap, snap_seq);
     return;
@@ -176,7 +232,7 @@ __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slot
   __shared__ unsigned s_last;
   unsigned created = 0;
   constexpr uint64_t kRound = (uint64_t)kBlock * kLookupItems;
-  for (uint64_t base = (uint64_t)blockIdx.x * kRound; base < n; base += (uint64_t)gridDim.x * kRound) {
+  for (uint64_t base = (uint64_t)blockIdx.x * kRound; base < n; base += (uint64_t)nblk * kRound) {
     uint64_t* p[kLookupItems];
     uint64_t seen[kLookupItems];
     bool is_new[kLookupItems];
@@ -229,7 +285,7 @@ __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slot
     __syncthreads();  // s_first and red are reused by the next round
   }
   block_count_add(st, created, cred);
-  publish_after_lookup(st, snap, snap_seq, &s_last);
+  publish_after_lookup(st, snap, snap_seq, nblk, &s_last);
 }
 
 // VARLEN push, first kernel: one pass over the request's keys and lens that
@@ -239,10 +295,19 @@ __global__ __launch_bounds__(kBlock) void k_lookup_fixed(Slot* __restrict__ slot
 // totals. Always launched for a push, so the decision and the scan cost no launch of their
 // own.
 template <int kItems>
-__global__ __launch_bounds__(kBlock) void k_var_push_begin(
-    const uint64_t* __restrict__ keys, const int32_t* __restrict__ lens, uint64_t n,
-    const uint64_t* __restrict__ cache_keys, const int32_t* __restrict__ cache_lens,
-    unsigned long long* __restrict__ part, DevState* st, unsigned max_len, ReqTag tag) {
+__global__ __launch_bounds__(kBlock) void k_var_push_begin(ReqBatch b) {
+  const TableReq& d = b.t[blockIdx.y];
+  const unsigned nblk = d.nblk;
+  if (blockIdx.x >= nblk) return;
+  const uint64_t* __restrict__ keys = d.keys;
+  const int32_t* __restrict__ lens = d.lens;
+  const uint64_t n = d.n;
+  const uint64_t* __restrict__ cache_keys = d.cache_keys;
+  const int32_t* __restrict__ cache_lens = d.cache_lens;
+  unsigned long long* __restrict__ part = d.part;
+  DevState* st = d.st;
+  constexpr unsigned max_len = PSKV_MAX_VARLEN_ROW;
+  const ReqTag tag = d.tag;
   __shared__ unsigned long long red[kBlock / 64];
   __shared__ unsigned fred[kBlock / 64];
   __shared__ unsigned long long carry_s;
@@ -278,8 +343,8 @@ __global__ __launch_bounds__(kBlock) void k_var_push_begin(
     const bool has_left = base + j < n && base + j > 0;
     flags |= (has_left && k[j] == (j ? k[j - 1] : left)) ? kReqDuplicate : 0u;
   }
-  if (!scan_pass1_block(s, flags, part, st, red, fred, &s_last)) return;
-  flags = scan_pass1_last(part, st, tag.epoch, red, &carry_s);
+  if (!scan_pass1_block(s, flags, part, st, nblk, red, fred, &s_last)) return;
+  flags = scan_pass1_last(part, st, nblk, tag.epoch, red, &carry_s);
   if (threadIdx.x == 0) decide_same(st, tag, (flags & kReqDiffer) != 0u);
 }
 
@@ -293,13 +358,27 @@ __global__ __launch_bounds__(kBlock) void k_var_push_begin(
 constexpr unsigned long long kArenaPadUnits = 8;  // 128 bytes in 16-byte allocation units
 
 template <int kItems>
-__global__ __launch_bounds__(kBlock) void k_var_push_lookup(
-    Slot* __restrict__ slots, uint64_t mask, DevState* st, const uint64_t* __restrict__ keys,
-    const int32_t* __restrict__ lens, uint64_t n, uint64_t nvals,
-    const unsigned long long* __restrict__ part, uint64_t* __restrict__ off,
-    uint32_t* __restrict__ tile_key, uint64_t ntiles, uint64_t tile, uint64_t* __restrict__ ref,
-    uint64_t* __restrict__ cache_keys, int32_t* __restrict__ cache_lens, ReqTag tag,
-    Snapshot* snap, uint64_t snap_seq) {
+__global__ __launch_bounds__(kBlock) void k_var_push_lookup(ReqBatch b) {
+  const TableReq& d = b.t[blockIdx.y];
+  const unsigned nblk = d.nblk;
+  if (blockIdx.x >= nblk) return;
+  Slot* __restrict__ slots = d.slots;
+  const uint64_t mask = d.mask;
+  DevState* st = d.st;
+  const uint64_t* __restrict__ keys = d.keys;
+  const int32_t* __restrict__ lens = d.lens;
+  const uint64_t n = d.n, nvals = d.nvals;
+  const unsigned long long* __restrict__ part = d.part;
+  uint64_t* __restrict__ off = d.off;
+  uint32_t* __restrict__ tile_key = d.tile_key;
+  const uint64_t ntiles = d.ntiles;
+  constexpr uint64_t tile = PSKV_TILE_VAR;
+  uint64_t* __restrict__ ref = d.ref;
+  uint64_t* __restrict__ cache_keys = d.cache_keys;
+  int32_t* __restrict__ cache_lens = d.cache_lens;
+  const ReqTag tag = d.tag;
+  Snapshot* snap = d.snap;
+  const uint64_t snap_seq = d.snap_seq;
   if (cache_same(st, tag)) {  // offsets, tile table and references of the cached request hold
     if (snap && blockIdx.x == 0 && threadIdx.x < 64) publish_snapshot(st, snap, snap_seq);
     return;
@@ -382,7 +461,7 @@ __global__ __launch_bounds__(kBlock) void k_var_push_lookup(
     ref[i] = payload | (is_new[j] ? kRefNew : 0ull);
   }
   block_count_add(st, mine, cred);
-  publish_after_lookup(st, snap, snap_seq, &s_last);
+  publish_after_lookup(st, snap, snap_seq, nblk, &s_last);
 }
 
 // VARLEN pull, first kernel: the stored length of every key (an absent key answers length 0
@@ -390,10 +469,20 @@ __global__ __launch_bounds__(kBlock) void k_var_push_lookup(
 // the cached push the answer is known without a single probe: every key is present with the
 // cached length, and the offsets of that push are the offsets of this response.
 template <int kItems>
-__global__ __launch_bounds__(kBlock) void k_var_pull_lookup(
-    const Slot* __restrict__ slots, uint64_t mask, DevState* st, const uint64_t* __restrict__ keys,
-    uint64_t n, uint64_t* __restrict__ ref, int32_t* __restrict__ out_lens,
-    const int32_t* __restrict__ cache_lens, unsigned long long* __restrict__ part, ReqTag tag) {
+__global__ __launch_bounds__(kBlock) void k_var_pull_lookup(ReqBatch b) {
+  const TableReq& d = b.t[blockIdx.y];
+  const unsigned nblk = d.nblk;
+  if (blockIdx.x >= nblk) return;
+  const Slot* __restrict__ slots = d.slots;
+  const uint64_t mask = d.mask;
+  DevState* st = d.st;
+  const uint64_t* __restrict__ keys = d.keys;
+  const uint64_t n = d.n;
+  uint64_t* __restrict__ ref = d.ref;
+  int32_t* __restrict__ out_lens = d.out_lens;
+  const int32_t* __restrict__ cache_lens = d.cache_lens;
+  unsigned long long* __restrict__ part = d.part;
+  const ReqTag tag = d.tag;
   __shared__ unsigned long long red[kBlock / 64];
   __shared__ unsigned fred[kBlock / 64];
   __shared__ unsigned long long carry_s;
@@ -422,20 +511,26 @@ __global__ __launch_bounds__(kBlock) void k_var_pull_lookup(
       bits |= l & 3u;
     }
   }
-  if (!scan_pass1_block(s, bits, part, st, red, fred, &s_last)) return;
-  scan_pass1_last(part, st, tag.epoch, red, &carry_s);
+  if (!scan_pass1_block(s, bits, part, st, nblk, red, fred, &s_last)) return;
+  scan_pass1_last(part, st, nblk, tag.epoch, red, &carry_s);
 }
 
 // VARLEN pull, second kernel: pass 2 of the scan over the answered lengths: the request-side
 // offsets of the response and its tile table. `ntiles_cap` is the room in the table; the
 // tiles in use follow from the scanned total.
 template <int kItems>
-__global__ __launch_bounds__(kBlock) void k_var_offsets(const int32_t* __restrict__ lens, uint64_t n,
-                                                       const unsigned long long* __restrict__ part,
-                                                       uint64_t* __restrict__ off,
-                                                       uint32_t* __restrict__ tile_key,
-                                                       uint64_t ntiles_cap, uint64_t tile,
-                                                       const DevState* st, ReqTag tag) {
+__global__ __launch_bounds__(kBlock) void k_var_offsets(ReqBatch b) {
+  const TableReq& d = b.t[blockIdx.y];
+  if (blockIdx.x >= d.nblk) return;
+  const int32_t* __restrict__ lens = d.out_lens;  // the lengths the lookup kernel answered
+  const uint64_t n = d.n;
+  const unsigned long long* __restrict__ part = d.part;
+  uint64_t* __restrict__ off = d.off;
+  uint32_t* __restrict__ tile_key = d.tile_key;
+  const uint64_t ntiles_cap = d.ntiles;
+  constexpr uint64_t tile = PSKV_TILE_VAR;
+  const DevState* st = d.st;
+  const ReqTag tag = d.tag;
   if (cache_same(st, tag)) return;  // offsets and tile table of the cached request hold
   __shared__ unsigned long long wsum[kBlock / 64];
   uint64_t ntiles = (st->scan_total + tile - 1) / tile;
@@ -826,7 +921,28 @@ constexpr unsigned kTileVar = PSKV_TILE_VAR;        // per wavefront; the tile t
 constexpr unsigned kRowsVarPerBlock = kTileVar * (kBlock / 64);
 
 template <int OP, bool VARLEN, bool STREAM>
-__global__ __launch_bounds__(kBlock) void k_rows(RowsParams p) {
+__global__ __launch_bounds__(kBlock) void k_rows(ReqBatch b) {
+  const TableReq& d = b.t[blockIdx.y];
+  // the grid is sized for the largest table of the launch: workgroups (VARLEN: wavefronts) past
+  // this table's floats leave before they touch anything
+  if (((uint64_t)blockIdx.x * (kBlock / 64) + (VARLEN ? (threadIdx.x >> 6) : 0u)) *
+          (VARLEN ? kTileVar : kTileFixed / (kBlock / 64)) >= d.total)
+    return;
+  RowsParams p;
+  p.req = d.req;
+  p.arena = d.arena;
+  p.ref = d.ref;
+  p.off = d.off;
+  p.tile_key = d.tile_key;
+  p.tile_aff = d.tile_aff;
+  p.st = d.st;
+  p.n = d.n;
+  p.total = d.total;
+  p.k = d.k;
+  p.force_scalar = d.force_scalar;
+  p.ignore_new = d.ignore_new;
+  p.total_on_device = d.total_on_device;
+  p.tag = d.tag;
   __shared__ int32_t s_off[VARLEN ? (kWaveSpan + 1) * (kBlock / 64) : 1];
   __shared__ uint64_t s_ref[VARLEN ? kWaveSpan * (kBlock / 64) : 1];
   bool rejected = false;
