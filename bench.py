@@ -42,20 +42,46 @@ HBM_PEAK_GBS = 8000.0
 # times its launches (for the many-table workloads: those of one table, taken in turn).
 SAMPLE_EVERY = 4  # MI355X HBM3E, published
 
-# HBM bytes per launch (read + written) of the dominant kernels at the shapes below, from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this very script, scaled by what the same
-# counters read for the 1 GiB copy kernel (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0). They are
-# measured offline (a counter run cannot be nested in a timing run) and only reported when
-# the launch shape is the default one.
-TRAFFIC = {
-    ("push_scalar", 250000): 60.1e6, ("pull_scalar", 250000): 35.5e6,
-    ("rows_acc_fixed", 268435456): 3.0 * 2**30, ("rows_gather_fixed", 268435456): 2.0 * 2**30,
-    ("rows_acc_varlen", 6192336): 76.1e6, ("rows_gather_varlen", 6192336): 50.6e6,
-}
+# HBM bytes per launch (read + written) of the dominant kernels come from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs of this very script (a counter run cannot be nested in a timing
+# run), scaled by what the same counters read for the 1 GiB copy kernel. The summaries of those
+# runs under profiles/ carry one line per kernel and launch shape,
+#   traffic_per_launch: kind=<kind> units=<keys or floats per launch> read_bytes=<r> written_bytes=<w>
+# and this script reports a figure only when it finds the line for the launch shape it ran.
+TRAFFIC_FILES = ("sparse_lr.txt", "dense.txt", "varlen.txt", "zipf.txt")
+_traffic_cache = None
+
+
+def traffic_table():
+    """{(kind, units): (bytes, 'profiles/<file>')} from the committed profile summaries."""
+    global _traffic_cache
+    if _traffic_cache is None:
+        _traffic_cache = {}
+        for name in TRAFFIC_FILES:
+            path = os.path.join(REPO, "profiles", name)
+            if not os.path.exists(path):
+                continue
+            with open(path) as f:
+                for line in f:
+                    line = line.strip()
+                    if not line.startswith("traffic_per_launch: "):
+                        continue
+                    kv = dict(item.split("=", 1) for item in line[len("traffic_per_launch: "):].split())
+                    key = (kv["kind"], int(kv["units"]))
+                    _traffic_cache.setdefault(key, (float(kv["read_bytes"]) + float(kv["written_bytes"]),
+                                                    "profiles/" + name))
+    return _traffic_cache
+
+
+TRAFFIC_SOURCES = set()
 
 
 def traffic(kind, units):
-    return TRAFFIC.get((kind, int(units)))
+    hit = traffic_table().get((kind, int(units)))
+    if hit is None:
+        return None
+    TRAFFIC_SOURCES.add(hit[1])
+    return hit[0]
 
 
 def host_info():
@@ -156,20 +182,28 @@ def run_sparse_lr(args, capi, dev):
     stream = torch.cuda.Stream()
     # sized so that the tables end the run about one third of the way to their first growth
     cap = int(n * (args.warmup + 2 * args.steps) / S * 1.1)
-    tables = [capi.Table(capi.MODE_SCALAR, initial_capacity=cap, stream=stream.cuda_stream)
-              for _ in range(S)]
+    group = capi.Group(S, capi.MODE_SCALAR, initial_capacity=cap, stream=stream.cuda_stream)
+    tables = group.tables
+    per_table = args.per_table
 
     def step(i, sample=True):
         # Kernel durations are sampled INSIDE the timed steps: in every SAMPLE_EVERY-th step the
-        # launches of one of the S tables (taken in turn) carry their own start/stop events.
-        # Events on every launch would cost more host time per step than the GPU needs for it.
+        # launches carry their own start/stop events (booked to the first table of the group; with
+        # --per-table those of one of the S tables, taken in turn). Events on every launch would
+        # cost more host time per step than the GPU needs for it.
         if sample:
             j = i - args.warmup
             for s in range(S):
-                tables[s].prof_enable(sampled(j, args.steps) and s == (j // SAMPLE_EVERY) % S)
+                tables[s].prof_enable(sampled(j, args.steps) and
+                                      s == ((j // SAMPLE_EVERY) % S if per_table else 0))
         dk, dv = d_batches[i]
         kp, vp, op = dk.data_ptr(), dv.data_ptr(), out.data_ptr()
         pos, _, used = capi.slice_keys(dk, rb, re, nvals=n)
+        if not per_table:
+            # one launch per step of the pipeline over all S key ranges
+            group.push_raw(kp, pos, vp, pos)
+            group.pull_raw(kp, pos, op)
+            return
         pos = [int(x) for x in pos]
         for s in range(S):
             if used[s]:
@@ -181,8 +215,11 @@ def run_sparse_lr(args, capi, dev):
                 tables[s].pull_raw(kp + 8 * pos[s], c, op + 4 * pos[s], c)
 
     def drain():
-        for t in tables:
-            t.sync()
+        if per_table:
+            for t in tables:
+                t.sync()
+        else:
+            group.sync()
         torch.cuda.synchronize()
 
     for i in range(args.warmup):
@@ -217,6 +254,7 @@ def run_sparse_lr(args, capi, dev):
     if args.own_streams:
         own = [capi.Table(capi.MODE_SCALAR, initial_capacity=cap) for _ in range(S)]
         shared, tables = tables, own
+        was_per_table, per_table = per_table, True  # tables with streams of their own go one by one
         for i in range(args.warmup):
             step(i, sample=False)
         drain()
@@ -228,20 +266,22 @@ def run_sparse_lr(args, capi, dev):
         assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32)), "pulled values differ"
         for t in own:
             t.close()
-        tables = shared
+        tables, per_table = shared, was_per_table
     # the slicer alone on an idle GPU: two small launches and one read-back of S+1 positions
     t_s = time.perf_counter()
     for _ in range(50):
         capi.slice_keys(d_batches[0][0], rb, re, nvals=n)
     slice_us = (time.perf_counter() - t_s) / 50 * 1e6
-    keys_per_launch = n / S
+    keys_per_launch = n / S if per_table else n
     res = {
         "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
         "dtype": "f32",
         "config": {"workload": "sparse_lr: 1M sorted unique uint64 keys/step over 4 key ranges, "
                                "push then pull, store grows by 1M keys/step", "keys_per_step": n,
                    "ranges": S, "value_len": 1, "key_dtype": "u64",
-                   "store_keys_after_timed_steps": held},
+                   "store_keys_after_timed_steps": held,
+                   "launches": "one launch per table" if per_table else
+                               "one launch over all %d key ranges (pskv_push_multi / pskv_pull_multi)" % S},
         # every pushed key is new: 8 key + 4 val in, 8 slot read, 8 key + 4 val written
         "roofline": dict(roofline(32.0 * keys_per_launch, push_n, push_ms,
                                   traffic("push_scalar", keys_per_launch), push_s),
@@ -392,13 +432,19 @@ def run_varlen(args, capi, dev):
     out_lens = torch.empty(n, dtype=torch.int32, device=dev)
     torch.cuda.synchronize()  # the raw-pointer calls below do not wait for torch's stream
     stream = torch.cuda.Stream()  # one stream for all ranges: kernels run one at a time
-    tables = [capi.Table(capi.MODE_VARLEN, initial_capacity=int(n / S * 1.2) * 4,
-                         arena_floats=int(nvals / S * 1.5) + 8 * n // S, stream=stream.cuda_stream)
-              for _ in range(S)]
+    group = capi.Group(S, capi.MODE_VARLEN, initial_capacity=int(n / S * 1.2) * 4,
+                       arena_floats=int(nvals / S * 1.5) + 8 * n // S, stream=stream.cuda_stream)
+    tables = group.tables
+    per_table = args.per_table
     kp, vp, lp, op, olp = dk.data_ptr(), dv.data_ptr(), dl.data_ptr(), out.data_ptr(), out_lens.data_ptr()
 
     def step():
         pos, vpos, used = capi.slice_keys(dk, rb, re, lens=dl, nvals=nvals)
+        if not per_table:
+            # one launch per step of the pipeline over all S key ranges
+            group.push_raw(kp, pos, vp, vpos, lp)
+            group.pull_raw(kp, pos, op, vpos, olp)
+            return
         pos, vpos = [int(x) for x in pos], [int(x) for x in vpos]
         for s in range(S):
             if used[s]:
@@ -410,8 +456,11 @@ def run_varlen(args, capi, dev):
                 tables[s].pull_raw(kp + 8 * pos[s], c, op + 4 * vpos[s], f, olp + 4 * pos[s])
 
     def drain():
-        for t in tables:
-            t.sync()
+        if per_table:
+            for t in tables:
+                t.sync()
+        else:
+            group.sync()
         torch.cuda.synchronize()
 
     step()  # creates the rows
@@ -423,9 +472,10 @@ def run_varlen(args, capi, dev):
     t0 = time.perf_counter()
     for i in range(args.steps):
         # kernel durations are sampled inside the timed steps: in every SAMPLE_EVERY-th step the
-        # launches of one table, taken in turn, carry their own events
+        # launches carry their own events (with --per-table those of one table, taken in turn)
         for s in range(S):
-            tables[s].prof_enable(sampled(i, args.steps) and s == (i // SAMPLE_EVERY) % S)
+            tables[s].prof_enable(sampled(i, args.steps) and
+                                  s == ((i // SAMPLE_EVERY) % S if per_table else 0))
         step()
     drain()
     dt = time.perf_counter() - t0
@@ -443,10 +493,10 @@ def run_varlen(args, capi, dev):
     # different ranges overlap; durations are then no longer a kernel's own, hence not the headline)
     dt_own = None
     if args.own_streams:
-        for t in tables:
-            t.close()
+        group.close()
         tables = [capi.Table(capi.MODE_VARLEN, initial_capacity=int(n / S * 1.2) * 4,
                              arena_floats=int(nvals / S * 1.5) + 8 * n // S) for _ in range(S)]
+        per_table = True  # tables with streams of their own go one by one
         step()
         for _ in range(args.warmup):
             step()
@@ -457,13 +507,14 @@ def run_varlen(args, capi, dev):
         drain()
         dt_own = time.perf_counter() - t1
         assert torch.equal(out_lens, dl), "pulled lens differ"
-    floats_per_launch = nvals / S
+    floats_per_launch = nvals / S if args.per_table else nvals
     res = {
         "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
         "dtype": "f32",
         "config": {"workload": "varlen: 2M keys, lens in {8,16,32,64,128}, 16 key ranges, push then "
-                               "pull with lens", "keys_per_step": n, "floats_per_step": nvals,
-                   "ranges": S},
+                               "pull with lens", "keys_per_step": n, "floats_per_step": nvals, "ranges": S,
+                   "launches": "one launch per table" if args.per_table else
+                               "one launch over all %d key ranges (pskv_push_multi / pskv_pull_multi)" % S},
         "gbps": (20.0 * nvals + 56.0 * n) * args.steps / dt / 1e9,
         "roofline": dict(roofline(12.0 * floats_per_launch, acc[0], acc[1],
                                   traffic("rows_acc_varlen", floats_per_launch), acc[2]),
@@ -629,6 +680,9 @@ def main():
     ap.add_argument("--keys", type=int, default=0, help="keys per step (default: the config's)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the dense-chunk side measurement")
+    ap.add_argument("--per-table", action="store_true",
+                    help="sparse_lr / varlen: serve the key ranges with one pskv_push / pskv_pull per table "
+                         "instead of one pskv_push_multi / pskv_pull_multi over all of them")
     ap.add_argument("--own-streams", action="store_true",
                     help="sparse_lr / varlen: also time the steps with one stream per table "
                          "(reported under extra.own_streams; kernels of different ranges overlap)")
@@ -692,6 +746,9 @@ def main():
         "config": res["config"], "roofline": res["roofline"], "cpu_baseline": cpu,
         "kernels": res.get("kernels"),
     }
+    line["roofline"]["traffic_source"] = (
+        "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch of this command, scaled by the 1 GiB copy "
+        "kernel; read at run time from " + ", ".join(sorted(TRAFFIC_SOURCES))) if TRAFFIC_SOURCES else None
     if "gbps" in res:
         line["gbps"] = res["gbps"]
     if "own_streams" in res:
