@@ -48,7 +48,7 @@ SAMPLE_EVERY = 4  # MI355X HBM3E, published
 # runs under profiles/ carry one line per kernel and launch shape,
 #   traffic_per_launch: kind=<kind> units=<keys or floats per launch> read_bytes=<r> written_bytes=<w>
 # and this script reports a figure only when it finds the line for the launch shape it ran.
-TRAFFIC_FILES = ("sparse_lr.txt", "dense.txt", "varlen.txt", "zipf.txt")
+TRAFFIC_FILES = ("sparse_lr.txt", "dense.txt", "varlen.txt", "zipf.txt", "sparse_repeat.txt")
 _traffic_cache = None
 
 
@@ -671,12 +671,90 @@ def cpu_zipf(orc, batches, n, budget_s=25.0):
                       "std::unordered_map store, one thread" % (done, n)}
 
 
+# ------------------------------------------------------------------------------------
+# sparse_repeat: the same key set pushed again and again (the shape of the reference's own
+# test, tests/test_kv_app.cc:27-41, at the size of a sparse model)
+# ------------------------------------------------------------------------------------
+def run_sparse_repeat(args, capi, dev):
+    """One SCALAR table; every step pushes the SAME 16M sorted unique keys with fresh values and
+    pulls them back. From the third request on the table serves the key set from its
+    request-ordered value array: a streamed comparison of the keys, then `cached[i] += v[i]`."""
+    import torch
+    n = args.keys or 16000000
+    rng = np.random.default_rng(0x5EED)
+    keys = unique_sorted_keys(rng, n, KMAX)
+    vals = rng.normal(0.0, 0.01, size=n).astype(np.float32)
+    dk, dv = to_dev(keys, dev), to_dev(vals, dev)
+    out = torch.empty(n, dtype=torch.float32, device=dev)
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=int(n * 1.1))
+    torch.cuda.synchronize()
+    kp, vp, op = dk.data_ptr(), dv.data_ptr(), out.data_ptr()
+
+    def step():
+        t.push_raw(kp, n, vp, n)
+        t.pull_raw(kp, n, op, n)
+
+    for _ in range(max(args.warmup, 3)):  # insert, record, first request served from the cache
+        step()
+    t.sync()
+    t.prof_reset()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        t.prof_enable(sampled(i, args.steps))
+        step()
+    t.sync()
+    dt = time.perf_counter() - t0
+    push = kernel_stats([t], capi.KERNEL_PUSH_SCALAR)
+    pull = kernel_stats([t], capi.KERNEL_PULL_SCALAR)
+    same = kernel_stats([t], capi.KERNEL_SAME_KEYS)
+    t.prof_enable(False)
+    # closed form: every key holds (warm-up + timed steps) sequential adds of its value
+    idx = torch.randint(0, n, (4096,), device=dev)
+    ref = torch.zeros(4096, device=dev)
+    for _ in range(max(args.warmup, 3) + args.steps):
+        ref = ref + dv[idx]
+    assert torch.equal(out[idx], ref), "sums differ from sequential float adds"
+    assert t.size()[0] == n
+    res = {
+        "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
+        "dtype": "f32",
+        "config": {"workload": "sparse_repeat: the same 16M sorted unique uint64 keys pushed (fresh values) "
+                               "and pulled every step, one table", "keys_per_step": n, "ranges": 1,
+                   "value_len": 1, "key_dtype": "u64"},
+        # 4 val in + 4 cached value read + 4 written; the keys are compared by the kernel in front
+        "roofline": dict(roofline(12.0 * n, push[0], push[1], traffic("push_scalar_cached", n), push[2]),
+                         kernel="k_scalar<push, cached key set> (cached[i] += v[i])", bytes_per_key=12),
+        "kernels": {"pull_scalar_cached": dict(roofline(8.0 * n, pull[0], pull[1],
+                                                        traffic("pull_scalar_cached", n), pull[2]),
+                                               bytes_per_key=8),
+                    "same_keys": dict(roofline(16.0 * n, same[0], same[1], traffic("same_keys", n), same[2]),
+                                      kernel="k_same_keys (request keys against cached keys), once per "
+                                             "push and once per pull", bytes_per_key=16)},
+    }
+    return res, (keys, vals, n)
+
+
+def cpu_sparse_repeat(orc, keys, vals, n, budget_s=20.0):
+    store = orc.Store(orc.MODE_SCALAR)
+    store.push(keys, vals)  # the inserting first push is not part of the GPU's timed steps either
+    done = 0
+    t0 = time.perf_counter()
+    while done < 1 or time.perf_counter() - t0 < budget_s:
+        store.push(keys, vals)
+        store.handle(False, True, keys, out_cap=n)
+        done += 1
+    dt = time.perf_counter() - t0
+    return {"value": 2.0 * n * done / dt, "unit": "keys/s", "cores": 1, "kind": "port",
+            "sample": "%d steps (push + pull of the same %d keys) on a std::unordered_map store that holds "
+                      "them already, one thread" % (done, n)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="sparse_lr", choices=["sparse_lr", "dense", "varlen", "zipf"])
+    ap.add_argument("--workload", default="sparse_lr", choices=["sparse_lr", "dense", "varlen", "zipf", "sparse_repeat"])
     ap.add_argument("--keys", type=int, default=0, help="keys per step (default: the config's)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the dense-chunk side measurement")
@@ -706,6 +784,8 @@ def main():
         if args.steps == 20:
             args.steps = 8  # the configuration has 8 worker pushes
         res, zipf_batches, zipf_n = run_zipf(args, capi, dev)
+    elif args.workload == "sparse_repeat":
+        res, repeat_inputs = run_sparse_repeat(args, capi, dev)
     else:
         res, varlen_inputs = run_varlen(args, capi, dev)
 
@@ -734,6 +814,8 @@ def main():
             extra["cpu_baseline_all_cores"] = cpu_dense_all_cores(orc)
         elif args.workload == "zipf":
             cpu = cpu_zipf(orc, zipf_batches, zipf_n)
+        elif args.workload == "sparse_repeat":
+            cpu = cpu_sparse_repeat(orc, *repeat_inputs)
         else:
             cpu = cpu_varlen(orc, *varlen_inputs)
         cpu["host"] = host_info()

@@ -68,7 +68,8 @@ extern "C" {
 #define PSKV_KERNEL_LOOKUP 4      /* key -> row lookup / insert of the row modes */
 #define PSKV_KERNEL_REHASH 5
 #define PSKV_KERNEL_COPY 6        /* the plain copy of pskv_copy_probe */
-#define PSKV_KERNEL_COUNT 7
+#define PSKV_KERNEL_SAME_KEYS 7   /* comparison of a request's keys with the cached key set */
+#define PSKV_KERNEL_COUNT 8
 
 typedef struct pskv_table pskv_table;
 

@@ -27,7 +27,7 @@ MODE_VARLEN = 2
 MAX_VARLEN_ROW = (1 << 28) - 1
 SLICE_NOALLOC_MAX_RANGES = 1024
 KERNEL_PUSH_SCALAR, KERNEL_PULL_SCALAR, KERNEL_ROWS_ACC, KERNEL_ROWS_GATHER, KERNEL_LOOKUP, \
-    KERNEL_REHASH, KERNEL_COPY = range(7)
+    KERNEL_REHASH, KERNEL_COPY, KERNEL_SAME_KEYS = range(8)
 
 ERROR_NAMES = {
     EUNCOVERED_KEY: "PSKV_EUNCOVERED_KEY", ESIZE_MISMATCH: "PSKV_ESIZE_MISMATCH",

@@ -238,6 +238,7 @@ __device__ __forceinline__ unsigned long long block_excl_scan_u64(unsigned long 
 }
 
 typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // One 128-bit read of a slot (key and payload together).
 __device__ __forceinline__ u64x2 load_slot(const Slot* p) {

@@ -14,8 +14,6 @@
 namespace pskv {
 namespace {
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
 // A 64-ary lower_bound by one wavefront. Each round the 64 lanes probe evenly spaced keys of
 // the remaining interval, a ballot counts how many are below the target (the probes are
 // sorted, so the votes are a prefix of ones) and the interval shrinks 64-fold:

@@ -4,6 +4,7 @@
 // calls in place of KVServerDefaultHandle (include/ps/kv_app.h:440-463).
 #include <algorithm>
 #include <atomic>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <string>
@@ -147,7 +148,20 @@ struct pskv_table {
   GrowBuf cache_keys, cache_lens;
   bool cache_valid = false;
   uint64_t cache_n = 0, cache_nvals = 0;
-  uint64_t epoch = 0;  // number of the last row-mode request
+  uint64_t epoch = 0;  // number of the last request that took part in this
+
+  // SCALAR: the same idea with the VALUES of the cached keys kept in request order (and the
+  // slot number of every key), so that a request which repeats the cached key set streams
+  // through `sc_vals` and touches no slot; the slots are brought up to date before anything
+  // else reads or changes them (`sc_dirty`: they may be behind).
+  GrowBuf sc_vals, sc_slots;
+  bool sc_dirty = false;
+  uint64_t sc_last_n = 0;   // keys of the previous request: a size that repeats is worth recording
+  unsigned sc_fail = 0;     // comparisons in a row that found other keys
+  unsigned sc_skip = 0;     // requests left to serve without the cache after such failures
+  unsigned long long* outcome = nullptr;  // pinned: epoch << 1 | same of the newest comparison
+  unsigned long long sc_seen = 0;         // the value of *outcome the host last looked at
+  uint64_t sc_min_keys = 0;               // requests below this size leave the cache alone; 0 = no cache
 
   bool prof = false;
   std::vector<EventPair> pending[PSKV_KERNEL_COUNT];
@@ -213,7 +227,7 @@ int grow(pskv_table* t, GrowBuf* b, size_t bytes) {
   size_t want = std::max(bytes, b->bytes + b->bytes / 2);
   want = (want + 255) & ~(size_t)255;
   if (b == &t->ws || b == &t->tiles || b == &t->tiles_aff || b == &t->cache_keys ||
-      b == &t->cache_lens)
+      b == &t->cache_lens || b == &t->sc_vals || b == &t->sc_slots)
     t->cache_valid = false;  // the contents do not survive a reallocation
   if (b->ptr) {
     // earlier requests on the stream may still read the old buffer
@@ -308,11 +322,39 @@ void adopt_snapshot(pskv_table* t) {
   t->base_top = top;
 }
 
+// SCALAR: brings the slots up to date with the values of the key cache. Enqueued before
+// anything but the kernels of a request that repeats the cached keys looks at the slots.
+int flush_scalar_cache(pskv_table* t) {
+  if (!t->sc_dirty) return PSKV_OK;
+  ReqBatch rb;
+  std::memset(&rb, 0, sizeof(rb));
+  TableReq& d = rb.t[0];
+  d.slots = t->slots;
+  d.mask = t->cap - 1;
+  d.st = t->st;
+  d.n = t->cache_n;
+  d.arena = static_cast<float*>(t->sc_vals.ptr);
+  d.tile_key = static_cast<uint32_t*>(t->sc_slots.ptr);
+  d.cache_mode = kFlushAlways;
+  d.nblk = grid_for(t->cache_n, kBlock, kMaxGrid);
+  hipLaunchKernelGGL(k_scalar_flush, dim3(d.nblk, 1), dim3(kBlock), 0, t->stream, rb);
+  PSKV_HIP(hipGetLastError());
+  t->sc_dirty = false;
+  return PSKV_OK;
+}
+
 int grow_slots(pskv_table* t, uint64_t keys_needed) {
   uint64_t want = next_pow2((uint64_t)((double)keys_needed / t->max_load) + 1);
   want = std::max(want, t->cap * 2);
   Slot* fresh = nullptr;
-  int rc = alloc_slots(want, &fresh, t->stream);
+  int rc = PSKV_OK;
+  if (t->mode == PSKV_MODE_SCALAR) {
+    // the key cache holds slot numbers of the old array, and values the old array may lack
+    rc = flush_scalar_cache(t);
+    if (rc) return rc;
+    t->cache_valid = false;
+  }
+  rc = alloc_slots(want, &fresh, t->stream);
   if (rc) return rc;
   launch(t, PSKV_KERNEL_REHASH, k_rehash, dim3(grid_for(t->cap, kBlock, kMaxGrid)), dim3(kBlock),
          (const Slot*)t->slots, t->cap, fresh, want - 1, t->st);
@@ -500,37 +542,146 @@ int read_state_batch(Batch& bt) {
   return PSKV_OK;
 }
 
+// Numbers a request that takes part in the key cache and says whether the key cache has the right shape for it.
+ReqTag next_tag(pskv_table* t, const Request& r) {
+  ReqTag tag;
+  tag.epoch = ++t->epoch;
+  tag.pad = 0;
+  tag.try_cache = (t->cache_valid && t->cache_n == r.n) ? 1u : 0u;
+  return tag;
+}
+
+// SCALAR requests of at least this many keys may use the key cache (below that a request is a
+// single short launch either way, and the cache would add two). The environment variable
+// PSKV_SCALAR_CACHE_MIN_KEYS, read when a table is created, overrides it (0 switches the cache off).
+constexpr uint64_t kScalarCacheMinKeys = 1u << 17;
+
+// How a SCALAR request of one table relates to the table's key cache.
+enum ScalarCacheUse {
+  kScPlain,   // neither uses nor fills it
+  kScRecord,  // served through the slots; leaves its keys, values and slot numbers as the new cache
+  kScTry,     // compared with the cached keys on the device: served from the cache if they match,
+              // like kScRecord otherwise
+};
+
+// Decides it from what the host knows without waiting for the device: a request whose size
+// repeats the previous one is worth recording, a request of the cached size is worth comparing,
+// and comparisons that keep finding other keys (reported by the device through a pinned word,
+// read whenever the host gets here) switch the cache off for a growing number of requests.
+ScalarCacheUse scalar_cache_use(pskv_table* t, const Request& r) {
+  const unsigned long long seen = *static_cast<volatile unsigned long long*>(t->outcome);
+  if (seen != t->sc_seen) {
+    t->sc_seen = seen;
+    if (seen & 1ull) {
+      t->sc_fail = 0;
+    } else {
+      t->sc_fail = std::min(t->sc_fail + 1u, 6u);
+      t->sc_skip = 1u << t->sc_fail;
+    }
+  }
+  ScalarCacheUse use = kScPlain;
+  const bool eligible = t->sc_min_keys && r.n >= t->sc_min_keys && t->cap < (1ull << 32);
+  if (eligible && t->sc_skip) {
+    --t->sc_skip;
+  } else if (eligible) {
+    if (t->cache_valid && t->cache_n == r.n) {
+      use = kScTry;
+    } else if (r.n == t->sc_last_n) {
+      use = kScRecord;
+    }
+  }
+  t->sc_last_n = r.n;
+  return use;
+}
+
 int run_scalar(Batch& bt, bool push, bool pull) {
   uint64_t n_largest = 0;
-  for (Item& it : bt) {
+  bool any_cache = false;
+  std::vector<ScalarCacheUse> use(bt.size(), kScPlain);
+  std::vector<char> flush_unless_same(bt.size(), 0);
+  for (size_t i = 0; i < bt.size(); ++i) {
+    Item& it = bt[i];
+    pskv_table* t = it.t;
     Request& r = it.r;
     r.out_nvals = pull ? r.n : 0;
     it.d = TableReq{};
     if (r.n == 0) continue;
-    int rc = reserve(it.t, r.n, 0, 0, &it.pub);
+    int rc = reserve(t, r.n, 0, 0, &it.pub);  // (a growth writes the cache back and drops it)
     if (rc) return rc;
-    it.d.slots = it.t->slots;
-    it.d.mask = it.t->cap - 1;
-    it.d.st = it.t->st;
-    it.d.keys = r.keys;
-    it.d.vals = r.vals;
-    it.d.out = r.out;
-    it.d.n = r.n;
+    use[i] = scalar_cache_use(t, r);
+    if (use[i] != kScTry) {
+      // the request goes through the slots, so they must be up to date; a push then makes the
+      // cached values stale, a recording replaces them
+      rc = flush_scalar_cache(t);
+      if (rc) return rc;
+      if (push || use[i] == kScRecord) t->cache_valid = false;
+    }
+    TableReq& d = it.d;
+    if (use[i] != kScPlain) {
+      // (kScTry: the buffers have the cached request's size already, nothing is reallocated)
+      rc = grow(t, &t->cache_keys, r.n * sizeof(uint64_t));
+      if (rc) return rc;
+      rc = grow(t, &t->sc_vals, r.n * sizeof(float));
+      if (rc) return rc;
+      rc = grow(t, &t->sc_slots, r.n * sizeof(uint32_t));
+      if (rc) return rc;
+      it.tag = next_tag(t, r);
+      d.tag = it.tag;
+      d.cache_keys = static_cast<uint64_t*>(t->cache_keys.ptr);
+      d.arena = static_cast<float*>(t->sc_vals.ptr);
+      d.tile_key = static_cast<uint32_t*>(t->sc_slots.ptr);
+      d.outcome = t->outcome;
+      d.cache_mode = kCacheOn;
+      any_cache = true;
+      flush_unless_same[i] = (it.tag.try_cache && t->sc_dirty) ? 1 : 0;
+    }
+    d.slots = t->slots;
+    d.mask = t->cap - 1;
+    d.st = t->st;
+    d.keys = r.keys;
+    d.vals = r.vals;
+    d.out = r.out;
+    d.n = r.n;
     n_largest = std::max(n_largest, r.n);
   }
   if (!n_largest) return PSKV_OK;
+  int rc;
+  if (any_cache) {
+    rc = launch_batch(bt, PSKV_KERNEL_SAME_KEYS, k_same_keys, [](const Item& it) {
+      return (it.d.cache_mode && it.tag.try_cache)
+                 ? (it.r.n + kBlock * kSameKeysItems - 1) / (kBlock * kSameKeysItems) : 0ull;
+    });
+    if (rc) return rc;
+    // slots that lag behind the cache are written back once the device knows that the request
+    // does NOT repeat the cached keys (cache_mode reads as kFlushUnlessSame in that kernel)
+    static_assert(kFlushUnlessSame == kCacheOn, "one descriptor serves both kernels");
+    size_t i = 0;
+    rc = launch_batch(bt, -1, k_scalar_flush, [&](const Item& it) {
+      return flush_unless_same[i++] ? (uint64_t)grid_for(it.r.n, kBlock, kMaxGrid) : 0ull;
+    });
+    if (rc) return rc;
+  }
   // the kernel strides over a table's keys, so a grid capped at kMaxGrid serves any request
   const unsigned gx = grid_for(n_largest, kBlock, kMaxGrid);
   auto nblk = [&](const Item& it) { return it.d.n ? (uint64_t)gx : 0ull; };
-  int rc;
   if (push && pull) {
-    rc = launch_batch(bt, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, true>, nblk);
+    rc = any_cache ? launch_batch(bt, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, true, true>, nblk)
+                   : launch_batch(bt, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, true, false>, nblk);
   } else if (push) {
-    rc = launch_batch(bt, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, false>, nblk);
+    rc = any_cache ? launch_batch(bt, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, false, true>, nblk)
+                   : launch_batch(bt, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, false, false>, nblk);
   } else {
-    rc = launch_batch(bt, PSKV_KERNEL_PULL_SCALAR, k_scalar<false, true>, nblk);
+    rc = any_cache ? launch_batch(bt, PSKV_KERNEL_PULL_SCALAR, k_scalar<false, true, true>, nblk)
+                   : launch_batch(bt, PSKV_KERNEL_PULL_SCALAR, k_scalar<false, true, false>, nblk);
   }
   if (rc) return rc;
+  for (size_t i = 0; i < bt.size(); ++i) {
+    if (use[i] == kScPlain || !bt[i].r.n) continue;
+    pskv_table* t = bt[i].t;
+    t->cache_valid = true;  // whichever way the device decides, the cache now stands for this request
+    t->cache_n = bt[i].r.n;
+    if (push && use[i] == kScTry) t->sc_dirty = true;  // served from the cache: the slots lag behind
+  }
   return publish_batch(bt);
 }
 
@@ -555,15 +706,6 @@ int launch_rows(Batch& bt, int op) {
   return launch_batch(bt, PSKV_KERNEL_ROWS_GATHER, k_rows<kOpGather, VARLEN, false>, nblk);
 }
 
-// Numbers a row-mode request and says whether the key cache has the right shape for it.
-ReqTag next_tag(pskv_table* t, const Request& r) {
-  ReqTag tag;
-  tag.epoch = ++t->epoch;
-  tag.pad = 0;
-  tag.try_cache = (t->cache_valid && t->cache_n == r.n) ? 1u : 0u;
-  return tag;
-}
-
 // Starts a row-mode request on every table with keys: numbers it and, where the key cache has
 // the right shape, lets the device compare the request with the cached one. Call after every
 // buffer the cache lives in has been grown for this request.
@@ -573,7 +715,7 @@ int begin_row_request(Batch& bt) {
     it.tag = next_tag(it.t, it.r);
     it.d.tag = it.tag;
   }
-  return launch_batch(bt, -1, k_same_keys, [](const Item& it) {
+  return launch_batch(bt, PSKV_KERNEL_SAME_KEYS, k_same_keys, [](const Item& it) {
     return (it.r.n && it.tag.try_cache) ? (it.r.n + kBlock * kSameKeysItems - 1) / (kBlock * kSameKeysItems)
                                         : 0ull;
   });
@@ -1197,6 +1339,8 @@ int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
   t->mode = opts->mode;
   t->max_load = opts->max_load > 0.f ? opts->max_load : 0.5f;
   t->row_len = opts->mode == PSKV_MODE_FIXED ? opts->row_len : 0;
+  t->sc_min_keys = kScalarCacheMinKeys;
+  if (const char* e = std::getenv("PSKV_SCALAR_CACHE_MIN_KEYS")) t->sc_min_keys = std::strtoull(e, nullptr, 10);
   auto fail = [&](int rc) {
     pskv_table_destroy(t);
     return rc;
@@ -1218,6 +1362,8 @@ int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
           hipSuccess ||
       hipHostMalloc(reinterpret_cast<void**>(&t->snap), sizeof(Snapshot), hipHostMallocDefault) !=
           hipSuccess ||
+      hipHostMalloc(reinterpret_cast<void**>(&t->outcome), sizeof(unsigned long long), hipHostMallocCoherent) !=
+          hipSuccess ||
       // coherent: the GPU does not cache these two, so each request sees what the host just wrote
       hipHostMalloc(reinterpret_cast<void**>(&t->small_in), kSmallBytes, hipHostMallocCoherent) !=
           hipSuccess ||
@@ -1225,6 +1371,7 @@ int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
           hipSuccess)
     return fail(set_error(PSKV_ENOMEM, "cannot allocate table state"));
   std::memset(t->snap, 0xFF, sizeof(Snapshot));  // names no request
+  *t->outcome = 0ull;
   if (t->mode != PSKV_MODE_SCALAR && opts->arena_floats) {
     t->arena_cap = (opts->arena_floats + 1023) & ~(uint64_t)1023;
     if (hipMalloc(reinterpret_cast<void**>(&t->arena), t->arena_cap * sizeof(float)) != hipSuccess)
@@ -1254,6 +1401,9 @@ int pskv_table_destroy(pskv_table* t) {
   if (t->st) (void)hipFree(t->st);
   if (t->st_host) (void)hipHostFree(t->st_host);
   if (t->snap) (void)hipHostFree(t->snap);
+  if (t->outcome) (void)hipHostFree(t->outcome);
+  if (t->sc_vals.ptr) (void)hipFree(t->sc_vals.ptr);
+  if (t->sc_slots.ptr) (void)hipFree(t->sc_slots.ptr);
   if (t->small_in) (void)hipHostFree(t->small_in);
   if (t->small_out) (void)hipHostFree(t->small_out);
   if (t->arena) (void)hipFree(t->arena);

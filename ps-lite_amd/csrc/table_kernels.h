@@ -49,7 +49,18 @@ struct TableReq {
   uint32_t total_on_device;  // VARLEN pull without a host round trip: the floats to move are
                              // DevState::scan_total and `total` is the room in req
   uint32_t nblk;          // workgroups of the launch in flight that serve this table
+  // SCALAR key cache (a request that repeats the cached sorted key set is served from a
+  // request-ordered value array): cache_keys above, the values in `arena`, the slot numbers in
+  // `tile_key`
+  unsigned long long* outcome;  // pinned host word that learns how the comparison went, or null
+  uint32_t cache_mode;          // kCache* below
+  uint32_t pad;
 };
+constexpr uint32_t kCacheOff = 0;     // SCALAR: the request neither uses nor fills the key cache
+constexpr uint32_t kCacheOn = 1;      // SCALAR: serve from the cache when the keys match, else refill it
+constexpr uint32_t kFlushUnlessSame = 1;  // k_scalar_flush: skip when the request in flight repeats the cache
+constexpr uint32_t kFlushAlways = 2;
+constexpr uint32_t kSlotSpecial = 0xffffffffu;  // cached slot number of key 2^64-1 (the side slot)
 struct ReqBatch {
   TableReq t[kMaxBatch];
 };
@@ -70,7 +81,14 @@ static_assert(sizeof(ReqBatch) <= 3840, "kernel arguments are limited to 4 KiB")
 // by element, so this is for the odd repeat, not a reduction of long runs. An UNSORTED request
 // that repeats a key remains a caller error with an unspecified sum.
 // ---------------------------------------------------------------------------------
-template <bool PUSH, bool PULL>
+// Stable key sets (the idea of the reference's unused sorted-merge helper,
+// include/ps/internal/parallel_kv_match.h:29-120: when both sides are sorted the same way no
+// lookup is needed). The CACHE variant serves a request that repeats the cached sorted key set
+// from a request-ordered value array: `cache_vals[i] += vals[i]`, fully coalesced, 12 bytes per
+// key instead of a 128-byte line per probe; the slots are brought up to date (k_scalar_flush)
+// before anything else looks at them. A request that does not repeat the cache goes the usual
+// way and leaves its keys, their values and their slot numbers behind as the new cache.
+template <bool PUSH, bool PULL, bool CACHE>
 __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
   const TableReq& d = b.t[blockIdx.y];
   const uint64_t n = d.n;
@@ -81,6 +99,30 @@ __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
   const uint64_t* __restrict__ keys = d.keys;
   const float* __restrict__ vals = d.vals;
   float* __restrict__ out = d.out;
+  const bool record = CACHE && d.cache_mode == kCacheOn;
+  if (record && cache_same(st, d.tag)) {
+    // the keys are those of the cached request: position i of the request is position i of the cache
+    float* __restrict__ cv = d.arena;
+    const bool vec = ((reinterpret_cast<uintptr_t>(vals) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock * 4;
+    for (uint64_t i = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * 4; i < n; i += stride) {
+      if (vec && i + 4 <= n) {
+        f32x4 cur = *reinterpret_cast<const f32x4*>(cv + i);
+        if (PUSH) cur = cur + __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(vals + i));
+        if (PULL) __builtin_nontemporal_store(cur, reinterpret_cast<f32x4*>(out + i));
+        if (PUSH) *reinterpret_cast<f32x4*>(cv + i) = cur;
+      } else {
+        for (uint64_t j = i; j < n && j < i + 4; ++j) {
+          float cur = cv[j];
+          if (PUSH) cur = cur + vals[j];
+          if (PULL) out[j] = cur;
+          if (PUSH) cv[j] = cur;
+        }
+      }
+    }
+    return;
+  }
+  if (record && blockIdx.x == 0 && threadIdx.x == 0) st->cache_epoch = d.tag.epoch;
   __shared__ unsigned red[kBlock / 64];
   unsigned created = 0;
   const uint64_t stride = (uint64_t)gridDim.x * kBlock;
@@ -103,6 +145,7 @@ __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
     bool is_new;
     uint64_t seen;
     uint64_t* p = find_or_insert(slots, mask, st, key, is_new, seen);
+    if (record && (!p || run)) st->bad_epoch = d.tag.epoch;  // not a request the cache can stand for
     if (!p) continue;
     // an absent key starts from Val() == 0, then `+=` (kv_app.h:454): 0.0f + v, not a copy
     float cur = is_new ? 0.0f : __uint_as_float((unsigned)seen);
@@ -116,8 +159,31 @@ __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
     }
     if (PUSH || is_new) *reinterpret_cast<float*>(p) = cur;
     created += is_new ? 1u : 0u;
+    if (record) {
+      d.cache_keys[i] = key;
+      d.arena[i] = cur;
+      d.tile_key[i] = key == kEmptyKey ? kSlotSpecial
+                                       : (uint32_t)((reinterpret_cast<Slot*>(p - 1) - slots));
+    }
   }
   block_count_add(st, created, red);
+}
+
+// Writes the cached values back to their slots. Launched before anything reads or changes the
+// slots of a table whose cache may be ahead of them: a request that does not repeat the cached
+// keys (kFlushUnlessSame: the comparison of that request has run), a growth, a dump.
+__global__ __launch_bounds__(kBlock) void k_scalar_flush(ReqBatch b) {
+  const TableReq& d = b.t[blockIdx.y];
+  if (blockIdx.x >= d.nblk) return;
+  if (d.cache_mode == kFlushUnlessSame && cache_same(d.st, d.tag)) return;
+  const uint64_t stride = (uint64_t)d.nblk * kBlock;
+  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < d.n; i += stride) {
+    const uint32_t slot = d.tile_key[i];
+    const float v = d.arena[i];
+    float* dst = slot == kSlotSpecial ? reinterpret_cast<float*>(&d.st->special_payload)
+                                      : reinterpret_cast<float*>(&d.slots[slot].payload);
+    *dst = v;
+  }
 }
 
 // ---------------------------------------------------------------------------------
@@ -129,14 +195,18 @@ __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
 // the decision is "different" (or the cache was not usable, or not even tried), the request
 // is going to refill the cache, so it becomes the cached request right here. Epochs start
 // at 1.
-__device__ __forceinline__ void decide_same(DevState* st, const ReqTag& tag, bool different) {
+__device__ __forceinline__ void decide_same(DevState* st, const ReqTag& tag, bool different,
+                                            unsigned long long* outcome = nullptr) {
   const bool usable =
       tag.try_cache && st->cache_epoch != 0ull && st->bad_epoch != st->cache_epoch;
-  if (!different && usable) {
+  const bool same = !different && usable;
+  if (same) {
     st->same_epoch = tag.epoch;
   } else {
     st->cache_epoch = tag.epoch;
   }
+  // the host reads this when it gets to it (never waits for it): epoch << 1 | same
+  if (outcome) *outcome = (tag.epoch << 1) | (same ? 1ull : 0ull);
 }
 
 // Compares the keys of a request with the cached ones and reaches the decision for the whole
@@ -172,7 +242,8 @@ __global__ __launch_bounds__(kBlock) void k_same_keys(ReqBatch b) {
   }
   __syncthreads();
   if (!s_last) return;
-  if (threadIdx.x == 0) decide_same(st, tag, (atomicExch(&st->req_flags, 0u) & kReqDiffer) != 0u);
+  if (threadIdx.x == 0)
+    decide_same(st, tag, (atomicExch(&st->req_flags, 0u) & kReqDiffer) != 0u, d.outcome);
 }
 
 // The counter record of a request, written by the kernel that creates its keys once every
@@ -571,8 +642,6 @@ struct RowsParams {
 
 constexpr int kOpAcc = 0;
 constexpr int kOpGather = 1;
-
-typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // VEC floats moved by one lane per access. STREAM selects non-temporal accesses: a
 // request far larger than the caches is read and written once per launch, and telling

@@ -194,3 +194,38 @@ def test_multi_misuse_is_a_status_code(capi, dev):
     # the other tables took their slices: only table 0 refused
     sizes = [t.size()[0] for t in gv.tables]
     assert sum(sizes) == keys.size
+
+
+def test_multi_scalar_tables_with_repeating_key_sets(capi, orc, dev, monkeypatch):
+    """SCALAR tables of a group whose requests repeat their key set: every table takes its own
+    decision (serve from its request-ordered value array, or go through the slots) inside the one
+    launch that serves them all."""
+    import torch
+    announce("multi_scalar_repeats")
+    monkeypatch.setenv("PSKV_SCALAR_CACHE_MIN_KEYS", "64")
+    rng = np.random.default_rng(77)
+    S, n = 6, 30000
+    rb, re = capi.server_ranges(S)
+    g = capi.Group(S, capi.MODE_SCALAR, initial_capacity=16)
+    o = orc.Store(orc.MODE_SCALAR)
+    a = unique_keys(rng, n, S)
+    b = a.copy()
+    # b differs from a in the keys of two ranges only: the other tables keep serving from their cache
+    lim = covered_limit(S) // S
+    for s in (1, 4):
+        m = (b >= s * lim) & (b < (s + 1) * lim)
+        b[m] = np.sort(rng.integers(s * lim, (s + 1) * lim, size=int(m.sum()), dtype=np.uint64))
+    b = np.unique(b)
+    for name in "a a a a b a a b b a".split():
+        keys = a if name == "a" else b
+        vals = rng.normal(0, 1, size=keys.size).astype(np.float32)
+        dk, dv = to_dev(keys, dev), to_dev(vals, dev)
+        pos, vpos = _slice(capi, dk, rb, re, None, keys.size)
+        g.push(dk, pos, dv, vpos)
+        o.push(keys, vals)
+        out = torch.full((keys.size,), 7.0, dtype=torch.float32, device=dev)
+        g.pull(dk, pos, out)
+        g.sync()
+        assert_bits_equal(from_dev(out), o.pull(keys)[0], "pull after push of " + name)
+    _check_dump(g, o, "multi scalar repeats")
+    g.close()

@@ -725,18 +725,27 @@ def test_scalar_sorted_repeats(capi, orc, dev, memkind, n):
     _check_dump(t, o, "sorted repeats")
 
 
-@pytest.mark.parametrize("mode", ["fixed", "varlen"])
+@pytest.fixture
+def small_scalar_cache(monkeypatch):
+    """Tables created in the test let SCALAR requests of 64 keys and more use the key cache (the
+    default is 131,072), so that short sequences of small requests go through all of its states."""
+    monkeypatch.setenv("PSKV_SCALAR_CACHE_MIN_KEYS", "64")
+
+
+@pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
 @pytest.mark.parametrize("seed", [0, 1, 2, 3])
-def test_repeated_and_alternating_key_sets(capi, orc, dev, mode, seed):
+def test_repeated_and_alternating_key_sets(capi, orc, dev, mode, seed, small_scalar_cache):
     """Requests that repeat the previous request's keys take a path that skips the hash probes; requests
     that do not must never see what that path left behind. Random sequences over a few key sets that
     are equal, differ in one key, differ in one length or differ in size, through every entry point
-    and both memory kinds, checked against the oracle after every pull."""
+    and both memory kinds, checked against the oracle after every pull. (SCALAR: the values of a
+    repeated key set live in a request-ordered array that is ahead of the slots until something else
+    needs them; a larger key set makes the table grow in the middle of that.)"""
     import torch
     announce("repeated_key_sets", mode, seed)
     rng = np.random.default_rng(1000 + seed)
     n = int(rng.integers(300, 3000))
-    k = 8
+    k = 1 if mode == "scalar" else 8
     base = unique_keys(rng, n + 50)
     sets = {}
     sets["A"] = base[:n].copy()
@@ -746,15 +755,19 @@ def test_repeated_and_alternating_key_sets(capi, orc, dev, mode, seed):
     sets["C"] = base[10:n + 10].copy()        # same size, shifted
     sets["D"] = base[: n // 2].copy()         # a different size
     lens_of = {int(key): int(l) for key, l in zip(base.tolist(), rng.choice([0, 4, 8, 12, 40], size=base.size))}
-    m = capi.MODE_FIXED if mode == "fixed" else capi.MODE_VARLEN
-    t = capi.Table(m, initial_capacity=64, row_len=k)  # small: the slot array grows during the sequence
-    o = orc.Store(orc.MODE_FIXED if mode == "fixed" else orc.MODE_VARLEN, k)
+    m = {"scalar": capi.MODE_SCALAR, "fixed": capi.MODE_FIXED, "varlen": capi.MODE_VARLEN}[mode]
+    om = {"scalar": orc.MODE_SCALAR, "fixed": orc.MODE_FIXED, "varlen": orc.MODE_VARLEN}[mode]
+    t = capi.Table(m, initial_capacity=64, row_len=k if mode == "fixed" else 0)  # small: the slot array grows during the sequence
+    o = orc.Store(om, k if mode == "fixed" else 0)
 
     def lens_for(keys):
         return np.array([lens_of[int(x)] for x in keys.tolist()], np.int32) if mode == "varlen" else None
 
     names = ["A", "A", "A", "B", "C", "D", "A"]
-    for step in range(40):
+    if mode == "scalar":
+        sets["E"] = np.union1d(base, unique_keys(rng, 6 * n))  # makes the table grow when it first comes
+        names += ["E"]
+    for step in range(60 if mode == "scalar" else 40):
         name = names[int(rng.integers(0, len(names)))]
         keys = sets[name]
         lens = lens_for(keys)
@@ -762,6 +775,8 @@ def test_repeated_and_alternating_key_sets(capi, orc, dev, mode, seed):
         op = ["push", "push", "pull", "pull_async", "pushpull"][int(rng.integers(0, 5))]
         on_dev = bool(rng.integers(0, 2))
         vals = rng.integers(-8, 8, size=nvals).astype(np.float32)
+        if mode == "scalar":
+            vals = rng.normal(0, 1, size=nvals).astype(np.float32)  # sums that depend on their order
         kk = to_dev(keys, dev) if on_dev else keys
         vv = to_dev(vals, dev) if on_dev else vals
         ll = None if lens is None else (to_dev(lens, dev) if on_dev else lens)
@@ -977,3 +992,67 @@ def test_pushpull_with_too_small_a_buffer_applies_its_push_once(capi, orc, dev, 
         if mode == "varlen":
             assert np.array_equal(from_dev(got_lens) if memkind == "device" else got_lens, want_lens)
     _check_dump(t, o, "pushpull too small")
+
+
+@pytest.mark.parametrize("memkind", ["device", "host"])
+def test_scalar_key_cache_at_its_real_size(capi, orc, dev, memkind):
+    """The stable-key-set path of SCALAR tables with its default threshold: 300,000 keys pushed again
+    and again (the third push on is served from the request-ordered value array, 128 bits per lane),
+    pulled into aligned and unaligned buffers, then other keys (which must find every slot up to date),
+    a shorter request, and the first keys again."""
+    import torch
+    announce("scalar_key_cache_large", memkind)
+    rng = np.random.default_rng(23)
+    n = 300000
+    keys = unique_keys(rng, n)
+    other = unique_keys(rng, n)
+    other[: n // 2] = keys[: n // 2]  # half of them shared with the cached set
+    other = np.unique(other)
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=16)
+    o = orc.Store(orc.MODE_SCALAR)
+
+    def mem(a):
+        return to_dev(a, dev) if memkind == "device" else a
+
+    def push(k):
+        v = rng.normal(0, 1, size=k.size).astype(np.float32)
+        t.push(mem(k), mem(v))
+        o.push(k, v)
+
+    def pull(k, shift=0):
+        want, _ = o.pull(k)
+        if memkind == "device":
+            buf = torch.full((k.size + 8,), 7.0, dtype=torch.float32, device=dev)
+            out = buf[shift:shift + k.size]
+            torch.cuda.synchronize()
+            t.pull_raw(to_dev(k, dev).data_ptr(), k.size, out.data_ptr(), k.size)
+            t.sync()
+            got = from_dev(out)
+        else:
+            buf = np.full(k.size + 8, 7.0, np.float32)
+            got = buf[shift:shift + k.size]
+            t.pull(k, got)
+        assert_bits_equal(got, want, "pull shift %d" % shift)
+
+    for _ in range(5):
+        push(keys)
+    pull(keys)
+    pull(keys, shift=1)          # a response buffer that is not 16-byte aligned
+    push(keys)
+    push(other)                  # other keys: the slots must have caught up first
+    pull(other)
+    push(keys[:200000])          # a different size
+    for _ in range(3):
+        push(keys)
+    out_np, _ = o.pushpull(keys, np.ones(n, np.float32))
+    if memkind == "device":
+        out = torch.zeros(n, dtype=torch.float32, device=dev)
+        t.pushpull(to_dev(keys, dev), to_dev(np.ones(n, np.float32), dev), out)
+        t.sync()
+        assert_bits_equal(from_dev(out), out_np, "pushpull")
+    else:
+        out = np.zeros(n, np.float32)
+        t.pushpull(keys, np.ones(n, np.float32), out)
+        assert_bits_equal(out, out_np, "pushpull")
+    t.sync()
+    _check_dump(t, o, "scalar key cache")
