@@ -94,6 +94,10 @@ struct alignas(32) DevState {
   // FIXED: the request with this number was refused (it repeats a key): its row kernels change
   // no stored value and leave the rows it created as zero rows
   unsigned long long refused_epoch;
+  // SCALAR key cache: the last request that changed cached values without touching the slots, and
+  // the value of dirty_epoch up to which the slots have been brought up to date since
+  unsigned long long dirty_epoch;
+  unsigned long long clean_epoch;
   // keys held (slot array plus the side slot) = sum of the shards
   unsigned long long count_shard[kCountShards * kShardStride];
   // first level of the last-workgroup ticket: one counter per 128-byte line

@@ -157,8 +157,16 @@ struct pskv_table {
   GrowBuf sc_vals, sc_slots;
   bool sc_dirty = false;
   uint64_t sc_last_n = 0;   // keys of the previous request: a size that repeats is worth recording
-  unsigned sc_fail = 0;     // comparisons in a row that found other keys
-  unsigned sc_skip = 0;     // requests left to serve without the cache after such failures
+  // What the comparisons of the two kinds of requests (0: pushes and push+pulls, 1: pulls) have
+  // come to lately: pushes that bring new keys every time may still leave a cache behind that the
+  // pull after each of them is served from.
+  struct ScTrack {
+    unsigned fail = 0;  // comparisons in a row that found other keys
+    unsigned skip = 0;  // requests of this kind left to run without a comparison after such failures
+    bool hit = false;   // the newest comparison of this kind found the cached keys
+  } sc_track[2];
+  static const int kScKinds = 64;
+  unsigned char sc_kind[kScKinds] = {0};  // kind of the request with number e, at e % kScKinds
   unsigned long long* outcome = nullptr;  // pinned: epoch << 1 | same of the newest comparison
   unsigned long long sc_seen = 0;         // the value of *outcome the host last looked at
   uint64_t sc_min_keys = 0;               // requests below this size leave the cache alone; 0 = no cache
@@ -567,26 +575,36 @@ enum ScalarCacheUse {
 // Decides it from what the host knows without waiting for the device: a request whose size
 // repeats the previous one is worth recording, a request of the cached size is worth comparing,
 // and comparisons that keep finding other keys (reported by the device through a pinned word,
-// read whenever the host gets here) switch the cache off for a growing number of requests.
+// read whenever the host gets here) switch the comparison off for a growing number of requests
+// of that kind.
 ScalarCacheUse scalar_cache_use(pskv_table* t, const Request& r) {
   const unsigned long long seen = *static_cast<volatile unsigned long long*>(t->outcome);
   if (seen != t->sc_seen) {
     t->sc_seen = seen;
-    if (seen & 1ull) {
-      t->sc_fail = 0;
-    } else {
-      t->sc_fail = std::min(t->sc_fail + 1u, 6u);
-      t->sc_skip = 1u << t->sc_fail;
+    const unsigned long long e = seen >> 1;
+    if (e + pskv_table::kScKinds > t->epoch) {  // (else the note of its kind has been overwritten)
+      pskv_table::ScTrack& tr = t->sc_track[t->sc_kind[e % pskv_table::kScKinds] & 1];
+      if (seen & 1ull) {
+        tr.fail = 0;
+        tr.hit = true;
+      } else {
+        tr.fail = std::min(tr.fail + 1u, 6u);
+        tr.skip = 1u << tr.fail;
+        tr.hit = false;
+      }
     }
   }
+  const int kind = r.push ? 0 : 1;
   ScalarCacheUse use = kScPlain;
-  const bool eligible = t->sc_min_keys && r.n >= t->sc_min_keys && t->cap < (1ull << 32);
-  if (eligible && t->sc_skip) {
-    --t->sc_skip;
-  } else if (eligible) {
-    if (t->cache_valid && t->cache_n == r.n) {
+  if (t->sc_min_keys && r.n >= t->sc_min_keys && t->cap < (1ull << 32)) {
+    pskv_table::ScTrack& tr = t->sc_track[kind];
+    const bool compare = tr.skip == 0;
+    if (!compare) --tr.skip;
+    if (compare && t->cache_valid && t->cache_n == r.n) {
       use = kScTry;
-    } else if (r.n == t->sc_last_n) {
+    } else if (r.n == t->sc_last_n && (compare || t->sc_track[1 - kind].hit)) {
+      // a size that repeats: worth recording when this kind of request is still being tried, or
+      // when the other kind is being served from what this one leaves behind
       use = kScRecord;
     }
   }
@@ -626,6 +644,7 @@ int run_scalar(Batch& bt, bool push, bool pull) {
       rc = grow(t, &t->sc_slots, r.n * sizeof(uint32_t));
       if (rc) return rc;
       it.tag = next_tag(t, r);
+      t->sc_kind[it.tag.epoch % pskv_table::kScKinds] = r.push ? 0 : 1;
       d.tag = it.tag;
       d.cache_keys = static_cast<uint64_t*>(t->cache_keys.ptr);
       d.arena = static_cast<float*>(t->sc_vals.ptr);
@@ -661,9 +680,14 @@ int run_scalar(Batch& bt, bool push, bool pull) {
     });
     if (rc) return rc;
   }
-  // the kernel strides over a table's keys, so a grid capped at kMaxGrid serves any request
-  const unsigned gx = grid_for(n_largest, kBlock, kMaxGrid);
-  auto nblk = [&](const Item& it) { return it.d.n ? (uint64_t)gx : 0ull; };
+  // The kernel strides over a table's keys, so a grid capped at kMaxGrid serves any request. A
+  // request that is expected to repeat the cached keys gets a quarter of the workgroups: served
+  // from the cache it moves four keys per lane (should it go through the slots after all, every
+  // lane takes four turns).
+  auto nblk = [&](const Item& it) -> uint64_t {
+    if (!it.d.n) return 0;
+    return grid_for(it.d.n, (it.d.cache_mode && it.tag.try_cache) ? kBlock * 4 : kBlock, kMaxGrid);
+  };
   if (push && pull) {
     rc = any_cache ? launch_batch(bt, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, true, true>, nblk)
                    : launch_batch(bt, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, true, false>, nblk);

@@ -92,7 +92,8 @@ template <bool PUSH, bool PULL, bool CACHE>
 __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
   const TableReq& d = b.t[blockIdx.y];
   const uint64_t n = d.n;
-  if ((uint64_t)blockIdx.x * kBlock >= n) return;  // the grid is sized for the longest key list
+  const unsigned nblk = d.nblk;  // (the grid is sized for the table with the most workgroups)
+  if (blockIdx.x >= nblk) return;
   Slot* __restrict__ slots = d.slots;
   const uint64_t mask = d.mask;
   DevState* st = d.st;
@@ -103,8 +104,9 @@ __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
   if (record && cache_same(st, d.tag)) {
     // the keys are those of the cached request: position i of the request is position i of the cache
     float* __restrict__ cv = d.arena;
+    if (PUSH && blockIdx.x == 0 && threadIdx.x == 0) st->dirty_epoch = d.tag.epoch;  // the slots fall behind
     const bool vec = ((reinterpret_cast<uintptr_t>(vals) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
-    const uint64_t stride = (uint64_t)gridDim.x * kBlock * 4;
+    const uint64_t stride = (uint64_t)nblk * kBlock * 4;
     for (uint64_t i = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * 4; i < n; i += stride) {
       if (vec && i + 4 <= n) {
         f32x4 cur = *reinterpret_cast<const f32x4*>(cv + i);
@@ -125,7 +127,7 @@ __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
   if (record && blockIdx.x == 0 && threadIdx.x == 0) st->cache_epoch = d.tag.epoch;
   __shared__ unsigned red[kBlock / 64];
   unsigned created = 0;
-  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  const uint64_t stride = (uint64_t)nblk * kBlock;
   const unsigned lane = threadIdx.x & 63;
   // whole wavefronts stay in the loop together: the shuffles below need every lane
   for (uint64_t first = (uint64_t)blockIdx.x * kBlock; first < n; first += stride) {
@@ -175,7 +177,12 @@ __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
 __global__ __launch_bounds__(kBlock) void k_scalar_flush(ReqBatch b) {
   const TableReq& d = b.t[blockIdx.y];
   if (blockIdx.x >= d.nblk) return;
+  // nothing changes these two while this kernel runs except its own last workgroup, which writes
+  // after every workgroup has read them
+  const unsigned long long dirty = d.st->dirty_epoch;
+  if (dirty <= d.st->clean_epoch) return;  // the slots are up to date
   if (d.cache_mode == kFlushUnlessSame && cache_same(d.st, d.tag)) return;
+  __shared__ unsigned s_last;
   const uint64_t stride = (uint64_t)d.nblk * kBlock;
   for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < d.n; i += stride) {
     const uint32_t slot = d.tile_key[i];
@@ -184,6 +191,9 @@ __global__ __launch_bounds__(kBlock) void k_scalar_flush(ReqBatch b) {
                                       : reinterpret_cast<float*>(&d.slots[slot].payload);
     *dst = v;
   }
+  if (threadIdx.x == 0) s_last = ticket_last(d.st, d.nblk) ? 1u : 0u;
+  __syncthreads();
+  if (s_last && threadIdx.x == 0) d.st->clean_epoch = dirty;
 }
 
 // ---------------------------------------------------------------------------------
@@ -223,14 +233,27 @@ __global__ __launch_bounds__(kBlock) void k_same_keys(ReqBatch b) {
   const ReqTag tag = d.tag;
   __shared__ unsigned s_last;
   constexpr int kItems = kSameKeysItems;
+  static_assert(kItems % 2 == 0, "two keys per 128-bit load");
   const uint64_t base = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * kItems;
-  // all loads first, then the compares
+  // all loads first, then the compares; 128 bits per load where the buffers allow it (the cached
+  // keys always do), the request side read past the caches
   uint64_t a[kItems], c[kItems];
+  const bool vec = (reinterpret_cast<uintptr_t>(keys) & 15) == 0 && base + kItems <= n;
+  if (vec) {
 #pragma unroll
-  for (int j = 0; j < kItems; ++j) {
-    const bool in = base + j < n;
-    a[j] = in ? keys[base + j] : 0;
-    c[j] = in ? cache_keys[base + j] : 0;
+    for (int j = 0; j < kItems; j += 2) {
+      const u64x2 x = __builtin_nontemporal_load(reinterpret_cast<const u64x2*>(keys + base + j));
+      const u64x2 y = *reinterpret_cast<const u64x2*>(cache_keys + base + j);
+      a[j] = x.x, a[j + 1] = x.y;
+      c[j] = y.x, c[j + 1] = y.y;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < kItems; ++j) {
+      const bool in = base + j < n;
+      a[j] = in ? keys[base + j] : 0;
+      c[j] = in ? cache_keys[base + j] : 0;
+    }
   }
   bool differ = false;
 #pragma unroll
