@@ -136,6 +136,23 @@ def kernel_stats(tables, kernel):
     return n, ms, np.concatenate(samples) if samples else np.zeros(0, np.float32)
 
 
+def pull_entries(units, pull, same, traffic_plain):
+    """The `kernels` entries of a SCALAR pull. Once a table has seen pulls come right behind pushes
+    of the same keys it serves them from its key cache: the pull kernel then only streams the cached
+    values (8 B/key) and the keys are compared by k_same_keys (16 B/key) in front of it, which
+    together are the 24 B/key of a pull that goes through the slots."""
+    cached = same[0] > 0
+    out = {"pull_scalar": dict(roofline((8.0 if cached else 24.0) * units, pull[0], pull[1],
+                                        None if cached else traffic_plain, pull[2]),
+                               bytes_per_key=8 if cached else 24,
+                               path="served from the key cache (k_same_keys in front)" if cached
+                                    else "through the slots")}
+    if cached:
+        out["same_keys"] = dict(roofline(16.0 * units, same[0], same[1], None, same[2]), bytes_per_key=16,
+                                kernel="k_same_keys (request keys against cached keys)")
+    return out
+
+
 def roofline(alg_bytes_per_launch, launches, total_ms, traffic=None, samples=None):
     """`achieved` is algorithmic bytes over the AVERAGE launch duration; the median and the
     minimum over the launches are given beside it."""
@@ -233,7 +250,8 @@ def run_sparse_lr(args, capi, dev):
     drain()
     dt = time.perf_counter() - t0
     push_n, push_ms, push_s = kernel_stats(tables, capi.KERNEL_PUSH_SCALAR)
-    pull_n, pull_ms, pull_s = kernel_stats(tables, capi.KERNEL_PULL_SCALAR)
+    pull_st = kernel_stats(tables, capi.KERNEL_PULL_SCALAR)
+    same_st = kernel_stats(tables, capi.KERNEL_SAME_KEYS)
     for t in tables:
         t.prof_enable(False)
 
@@ -267,6 +285,29 @@ def run_sparse_lr(args, capi, dev):
         for t in own:
             t.close()
         tables, per_table = shared, was_per_table
+    # The same steps once more on tables that start at the library's default size and grow
+    # (allocate twice the slots, re-insert everything) while the clock runs, as the CPU's
+    # std::unordered_map does inside its own timing.
+    growing = None
+    if not args.no_extra and not per_table:
+        main_group, main_tables = group, tables
+        group = capi.Group(S, capi.MODE_SCALAR, stream=stream.cuda_stream)
+        tables = group.tables
+        for i in range(args.warmup):
+            step(i, sample=False)
+        drain()
+        t2 = time.perf_counter()
+        for i in range(args.warmup, args.warmup + args.steps):
+            step(i, sample=False)
+        drain()
+        dt_grow = time.perf_counter() - t2
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32)), "pulled values differ"
+        growing = {"value": 2.0 * n * args.steps / dt_grow, "unit": "keys/s",
+                   "ms_per_step": dt_grow / args.steps * 1e3,
+                   "note": "same steps on tables created with the default capacity (1M keys each, %d keys "
+                           "held at the end): they grow inside the timed steps" % sum(t.size()[0] for t in tables)}
+        group.close()
+        group, tables = main_group, main_tables
     # the slicer alone on an idle GPU: two small launches and one read-back of S+1 positions
     t_s = time.perf_counter()
     for _ in range(50):
@@ -286,15 +327,15 @@ def run_sparse_lr(args, capi, dev):
         "roofline": dict(roofline(32.0 * keys_per_launch, push_n, push_ms,
                                   traffic("push_scalar", keys_per_launch), push_s),
                          kernel="k_scalar<push> (find-or-insert + add)", bytes_per_key=32),
-        "kernels": {"pull_scalar": dict(roofline(24.0 * keys_per_launch, pull_n, pull_ms,
-                                                 traffic("pull_scalar", keys_per_launch), pull_s),
-                                        bytes_per_key=24),
-                    "slicer": {"wall_us_per_call": round(slice_us, 1), "keys": n, "ranges": S}},
+        "kernels": dict(pull_entries(keys_per_launch, pull_st, same_st, traffic("pull_scalar", keys_per_launch)),
+                        slicer={"wall_us_per_call": round(slice_us, 1), "keys": n, "ranges": S}),
     }
     if dt_own is not None:
         res["own_streams"] = {"value": 2.0 * n * args.steps / dt_own, "unit": "keys/s",
                               "ms_per_step": dt_own / args.steps * 1e3,
                               "note": "same steps, one stream per table (kernels of different ranges overlap)"}
+    if growing is not None:
+        res["growing_tables"] = growing
     return res, batches[args.warmup:args.warmup + args.steps], (n, S)
 
 
@@ -318,7 +359,9 @@ def cpu_sparse_lr(orc, batches, n, S, budget_s=25.0):
     dt = time.perf_counter() - t0
     return {"value": 2.0 * n * done / dt, "unit": "keys/s", "cores": 1, "kind": "port",
             "sample": "first %d of the timed steps (slice + push + pull of %d keys each), "
-                      "std::unordered_map store per range, one thread" % (done, n)}
+                      "std::unordered_map store per range, one thread; the maps start empty and rehash as "
+                      "they grow inside this timing, whereas the GPU tables of `value` are sized up front "
+                      "(extra.growing_tables is the GPU run whose tables grow inside the timing too)" % (done, n)}
 
 
 # ------------------------------------------------------------------------------------
@@ -637,6 +680,7 @@ def run_zipf(args, capi, dev):
     dt = time.perf_counter() - t0
     push = kernel_stats([t], capi.KERNEL_PUSH_SCALAR)
     pull = kernel_stats([t], capi.KERNEL_PULL_SCALAR)
+    same = kernel_stats([t], capi.KERNEL_SAME_KEYS)
     rehash = kernel_stats([t], capi.KERNEL_REHASH)
     held = t.size()[0]
     res = {
@@ -649,8 +693,8 @@ def run_zipf(args, capi, dev):
         # between a hit (28 B/key) and an insert (32 B/key); priced as inserts
         "roofline": dict(roofline(32.0 * n, push[0], push[1], None, push[2]),
                          kernel="k_scalar<push> (find-or-insert + add)", bytes_per_key=32),
-        "kernels": {"pull_scalar": dict(roofline(24.0 * n, pull[0], pull[1], None, pull[2]), bytes_per_key=24),
-                    "rehash": {"launches": rehash[0], "total_us": round(rehash[1] * 1e3, 1)}},
+        "kernels": dict(pull_entries(n, pull, same, None),
+                        rehash={"launches": rehash[0], "total_us": round(rehash[1] * 1e3, 1)}),
     }
     return res, batches[args.warmup:], n
 
@@ -835,6 +879,8 @@ def main():
         line["gbps"] = res["gbps"]
     if "own_streams" in res:
         extra["own_streams"] = res["own_streams"]
+    if "growing_tables" in res:
+        extra["growing_tables"] = res["growing_tables"]
     if extra:
         line["extra"] = extra
     print(json.dumps(line, allow_nan=False), flush=True)  # strict JSON: a NaN would be a bug

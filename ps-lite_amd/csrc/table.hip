@@ -157,6 +157,8 @@ struct pskv_table {
   GrowBuf sc_vals, sc_slots;
   bool sc_dirty = false;
   uint64_t sc_last_n = 0;   // keys of the previous request: a size that repeats is worth recording
+  int sc_last_kind = -1;    // and its kind (0: push or push+pull, 1: pull)
+  unsigned sc_pairs = 0;    // pulls in a row (up to 2) that came right behind a push of their own size
   // What the comparisons of the two kinds of requests (0: pushes and push+pulls, 1: pulls) have
   // come to lately: pushes that bring new keys every time may still leave a cache behind that the
   // pull after each of them is served from.
@@ -577,6 +579,10 @@ enum ScalarCacheUse {
 // and comparisons that keep finding other keys (reported by the device through a pinned word,
 // read whenever the host gets here) switch the comparison off for a growing number of requests
 // of that kind.
+bool scalar_cache_eligible(const pskv_table* t, const Request& r) {
+  return t->sc_min_keys && r.n >= t->sc_min_keys && t->cap < (1ull << 32);
+}
+
 ScalarCacheUse scalar_cache_use(pskv_table* t, const Request& r) {
   const unsigned long long seen = *static_cast<volatile unsigned long long*>(t->outcome);
   if (seen != t->sc_seen) {
@@ -595,20 +601,29 @@ ScalarCacheUse scalar_cache_use(pskv_table* t, const Request& r) {
     }
   }
   const int kind = r.push ? 0 : 1;
+  // a worker that pushes gradients and pulls the weights of the same keys right away shows as a
+  // pull behind a push of its own size, whatever that size is from one step to the next
+  if (kind == 1 && t->sc_last_kind == 0)
+    t->sc_pairs = r.n == t->sc_last_n ? std::min(t->sc_pairs + 1u, 2u) : 0u;
   ScalarCacheUse use = kScPlain;
-  if (t->sc_min_keys && r.n >= t->sc_min_keys && t->cap < (1ull << 32)) {
+  if (scalar_cache_eligible(t, r)) {
     pskv_table::ScTrack& tr = t->sc_track[kind];
     const bool compare = tr.skip == 0;
     if (!compare) --tr.skip;
+    const bool size_repeats = r.n == t->sc_last_n;
     if (compare && t->cache_valid && t->cache_n == r.n) {
       use = kScTry;
-    } else if (r.n == t->sc_last_n && (compare || t->sc_track[1 - kind].hit)) {
-      // a size that repeats: worth recording when this kind of request is still being tried, or
-      // when the other kind is being served from what this one leaves behind
-      use = kScRecord;
+    } else if (kind == 0) {
+      // a push is worth recording when its size repeats (the same keys may be coming again) or
+      // when pulls have been following the pushes and are not in a spell of failed comparisons
+      const bool pulls_follow = t->sc_pairs >= 2 && t->sc_track[1].skip == 0;
+      if ((compare && size_repeats) || pulls_follow) use = kScRecord;
+    } else if (compare && size_repeats && t->sc_last_kind == 1) {
+      use = kScRecord;  // a pull behind a pull of the same size
     }
   }
   t->sc_last_n = r.n;
+  t->sc_last_kind = kind;
   return use;
 }
 
@@ -635,14 +650,19 @@ int run_scalar(Batch& bt, bool push, bool pull) {
       if (push || use[i] == kScRecord) t->cache_valid = false;
     }
     TableReq& d = it.d;
-    if (use[i] != kScPlain) {
-      // (kScTry: the buffers have the cached request's size already, nothing is reallocated)
+    if (use[i] != kScTry && scalar_cache_eligible(t, r)) {
+      // Room for this request in the cache, whether or not it is recorded: a table that sees
+      // requests of this size allocates once, on the first of them, and not in the middle of a
+      // run when the cache comes into use. (The cache has been written back above; kScTry needs
+      // nothing: the buffers have the cached request's size.)
       rc = grow(t, &t->cache_keys, r.n * sizeof(uint64_t));
       if (rc) return rc;
       rc = grow(t, &t->sc_vals, r.n * sizeof(float));
       if (rc) return rc;
       rc = grow(t, &t->sc_slots, r.n * sizeof(uint32_t));
       if (rc) return rc;
+    }
+    if (use[i] != kScPlain) {
       it.tag = next_tag(t, r);
       t->sc_kind[it.tag.epoch % pskv_table::kScKinds] = r.push ? 0 : 1;
       d.tag = it.tag;

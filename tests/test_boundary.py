@@ -89,3 +89,26 @@ def test_bench_measures_one_gpu_only():
     assert p.returncode != 0
     assert "ONE GPU" in (p.stdout + p.stderr)
     assert not p.stdout.strip().startswith("{")  # no result line
+
+
+def test_bench_reads_its_traffic_figures_from_the_profiles():
+    """roofline.traffic is not typed into bench.py: it comes from the `traffic_per_launch:` lines of the
+    rocprofv3 summaries under profiles/, for the launch shapes the default commands run."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_for_test", os.path.join(REPO, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    table = bench.traffic_table()
+    for kind, units in [("push_scalar", 1000000), ("rows_acc_fixed", 268435456), ("rows_gather_fixed", 268435456),
+                        ("rows_acc_varlen", 99077384), ("rows_gather_varlen", 99077384),
+                        ("push_scalar_cached", 16000000), ("same_keys", 16000000)]:
+        assert (kind, units) in table, (kind, units)
+        nbytes, source = table[(kind, units)]
+        assert nbytes > 0 and source.startswith("profiles/")
+        assert os.path.exists(os.path.join(REPO, source))
+    # every figure is at least the algorithmic traffic of its kernel and within 2x of it, except the
+    # random-probe kernel, which moves whole lines
+    assert 0.99 * 12 * 268435456 <= table[("rows_acc_fixed", 268435456)][0] <= 1.05 * 12 * 268435456
+    assert 0.99 * 12 * 99077384 <= table[("rows_acc_varlen", 99077384)][0] <= 1.1 * 12 * 99077384
+    assert 0.99 * 12 * 16000000 <= table[("push_scalar_cached", 16000000)][0] <= 1.05 * 12 * 16000000
+    assert bench.traffic("push_scalar", 123) is None  # another launch shape: no figure
