@@ -14,6 +14,9 @@ namespace pskv {
 int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 void clear_error();
 
+// Whether [ptr, ptr + bytes) lies inside one buffer handed out by pskv_host_alloc (pinned memory).
+bool host_pool_owns(const void* ptr, size_t bytes);
+
 #define PSKV_HIP(call)                                                                     \
   do {                                                                                     \
     hipError_t e_ = (call);                                                                \

@@ -66,6 +66,25 @@ void pskv_host_free(void* ptr) {
   p.free_by_size[it->second].push_back(ptr);
 }
 
+}  // extern "C"
+
+namespace pskv {
+// Whether [ptr, ptr + bytes) lies inside one buffer of the pinned pool: such memory needs no
+// staging, the copy engines reach it directly.
+bool host_pool_owns(const void* ptr, size_t bytes) {
+  Pool& p = pool();
+  const uintptr_t a = reinterpret_cast<uintptr_t>(ptr);
+  std::lock_guard<std::mutex> lk(p.mu);
+  for (const auto& kv : p.size_of) {  // a handful of live buffers per process
+    const uintptr_t base = reinterpret_cast<uintptr_t>(kv.first);
+    if (a >= base && a + bytes <= base + kv.second) return true;
+  }
+  return false;
+}
+}  // namespace pskv
+
+extern "C" {
+
 int pskv_host_trim(void) {
   Pool& p = pool();
   std::vector<void*> victims;

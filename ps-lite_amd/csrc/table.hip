@@ -14,6 +14,7 @@
 
 #include "host_common.h"
 #include "scan.h"
+#include "stager.h"
 #include "table_kernels.h"
 
 namespace pskv {
@@ -41,6 +42,9 @@ constexpr uint64_t kSlackBytes = 256ull << 20;  // tables up to this size trade 
 // Host-resident requests up to this size (per direction) skip the copy commands: the kernels
 // read the request from, and write the response to, pinned host memory mapped into the GPU.
 constexpr size_t kSmallBytes = 1024u << 10;
+// Host-resident buffers from this size on travel piece by piece through the ring of pinned memory
+// (stager.h), copying, transfer and kernels overlapping; smaller ones take one copy command.
+constexpr size_t kPipeBytes = 4u << 20;
 
 // A device buffer that only grows. Contents are not kept across growth.
 struct GrowBuf {
@@ -474,6 +478,13 @@ struct Request {
   bool need_total;       // VARLEN pull: the caller wants the response size back (forces a wait)
   char* small_out;       // lazy_out: pinned room the response may go to when it fits
   uint64_t small_out_floats;
+  // Large host-resident requests (row modes). pipe_in: `vals` is room in device memory that the
+  // row kernel fills itself, piece by piece, from `vals_host` while it works through the pieces
+  // that have arrived. pipe_out: the gather kernel is not launched with the request; the caller
+  // launches it piece by piece in step with the transfer of the response (gather_deferred says
+  // that it is still owed, gather_varlen which kernel it is).
+  const float* vals_host;
+  bool pipe_in, pipe_out, gather_deferred, gather_varlen;
 };
 
 // A request as the kernels see it: the shares of up to kMaxBatch tables that live on one device,
@@ -733,6 +744,27 @@ int run_scalar(Batch& bt, bool push, bool pull) {
 // requests of a busy server they do not survive in the caches anyway.
 constexpr uint64_t kStreamFloats = 1u << 20;
 
+// The row kernel over `floats` request-side floats of the batch's only table, starting at float
+// `first` (a multiple of the tile size): one piece of a request that is served as it arrives.
+template <bool VARLEN>
+int launch_rows_piece(Batch& bt, int op, uint64_t first, uint64_t floats) {
+  const uint64_t tile = VARLEN ? kRowsVarPerBlock : kTileFixed;
+  Item& it = bt[0];
+  const bool stream = it.d.total >= kStreamFloats;
+  it.d.tile_base = (uint32_t)(first / tile);
+  auto nblk = [&](const Item&) { return (floats + tile - 1) / tile; };
+  int rc;
+  if (op == kOpAcc) {
+    rc = stream ? launch_batch(bt, PSKV_KERNEL_ROWS_ACC, k_rows<kOpAcc, VARLEN, true>, nblk)
+                : launch_batch(bt, PSKV_KERNEL_ROWS_ACC, k_rows<kOpAcc, VARLEN, false>, nblk);
+  } else {
+    rc = stream ? launch_batch(bt, PSKV_KERNEL_ROWS_GATHER, k_rows<kOpGather, VARLEN, true>, nblk)
+                : launch_batch(bt, PSKV_KERNEL_ROWS_GATHER, k_rows<kOpGather, VARLEN, false>, nblk);
+  }
+  it.d.tile_base = 0;
+  return rc;
+}
+
 // The row kernel over every table of the batch whose TableReq::total is not zero.
 template <bool VARLEN>
 int launch_rows(Batch& bt, int op) {
@@ -740,6 +772,21 @@ int launch_rows(Batch& bt, int op) {
   uint64_t floats = 0;
   for (const Item& it : bt) floats += it.d.total;
   if (!floats) return PSKV_OK;
+  if (bt.size() == 1 && op == kOpAcc && bt[0].r.pipe_in) {
+    // the values are still in the caller's memory: every piece is accumulated as soon as it is here
+    Item& it = bt[0];
+    Stager* sg = Stager::get(it.t->device);
+    if (!sg) return set_error(PSKV_ENOMEM, "no pinned memory to stage the request through");
+    return sg->to_device(const_cast<float*>(it.r.vals), it.r.vals_host, it.d.total * sizeof(float),
+                         it.t->stream, [&](size_t off, size_t len) {
+                           return launch_rows_piece<VARLEN>(bt, kOpAcc, off / sizeof(float), len / sizeof(float));
+                         });
+  }
+  if (bt.size() == 1 && op == kOpGather && bt[0].r.pipe_out) {
+    bt[0].r.gather_deferred = true;  // launched piece by piece in step with the transfer to the host
+    bt[0].r.gather_varlen = VARLEN;
+    return PSKV_OK;
+  }
   auto nblk = [&](const Item& it) { return (it.d.total + tile - 1) / tile; };
   const bool stream = floats >= kStreamFloats;
   if (op == kOpAcc) {
@@ -1177,10 +1224,35 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
       if (want_out_lens) dout_lens = reinterpret_cast<int32_t*>(t->small_out);
     } else {
       dout_lens = c.take<int32_t>(want_out_lens ? n : 0);
-      if (n) PSKV_HIP(hipMemcpyAsync(dkeys, keys, n * 8, hipMemcpyHostToDevice, t->stream));
-      if (r.nvals) PSKV_HIP(hipMemcpyAsync(dvals, vals, r.nvals * 4, hipMemcpyHostToDevice, t->stream));
-      if (want_lens && n) PSKV_HIP(hipMemcpyAsync(dlens, lens, n * 4, hipMemcpyHostToDevice, t->stream));
+      Stager* sg = Stager::get(t->device);
+      auto copy_in = [&](void* dst, const void* src, size_t bytes) -> int {
+        if (!bytes) return PSKV_OK;
+        // (buffers of the pinned pool are within reach of the copy engines as they are)
+        if (sg && bytes >= kPipeBytes && !host_pool_owns(src, bytes))
+          return sg->to_device(dst, src, bytes, t->stream, nullptr);
+        PSKV_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, t->stream));
+        return PSKV_OK;
+      };
+      rc = copy_in(dkeys, keys, n * 8);
+      if (rc) return rc;
+      if (want_lens) {
+        rc = copy_in(dlens, lens, n * 4);
+        if (rc) return rc;
+      }
+      if (sg && t->mode != PSKV_MODE_SCALAR && r.nvals * 4 >= kPipeBytes && !host_pool_owns(vals, r.nvals * 4)) {
+        // the values follow piece by piece while the lookup and the row kernel are already at work
+        r.vals_host = vals;
+        r.pipe_in = true;
+      } else {
+        rc = copy_in(dvals, vals, r.nvals * 4);
+        if (rc) return rc;
+      }
     }
+    // a large response of a row mode into ordinary memory leaves piece by piece as well, each piece
+    // gathered just before it travels
+    const uint64_t out_room = varlen ? out_cap : fixed_out;
+    r.pipe_out = pull && !too_small && t->mode != PSKV_MODE_SCALAR && out_room * 4 >= kPipeBytes &&
+                 !host_pool_owns(out, out_room * 4) && Stager::get(t->device) != nullptr;
     r.keys = dkeys;
     r.vals = dvals;
     r.lens = dlens;
@@ -1202,13 +1274,11 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
     r.out_cap = fixed_out;
   }
 
-  {
-    Batch bt(1);
-    bt[0].t = t;
-    bt[0].r = r;
-    rc = run_batch(bt, push, pull);
-    r = bt[0].r;
-  }
+  Batch bt(1);
+  bt[0].t = t;
+  bt[0].r = r;
+  rc = run_batch(bt, push, pull);
+  r = bt[0].r;
   if (out_nvals) *out_nvals = r.out_nvals;
   // Kernels of this request may still be reading the pinned request buffer, which the next
   // host-resident request overwrites from the host: no early return without a wait.
@@ -1225,8 +1295,25 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
     const bool out_pinned = pull && r.out_nvals && r.out >= reinterpret_cast<float*>(t->small_out) &&
                             r.out < reinterpret_cast<float*>(t->small_out + kSmallBytes);
     const bool lens_pinned = r.out_lens == reinterpret_cast<int32_t*>(t->small_out);
-    if (pull && r.out_nvals && !out_pinned)
-      PSKV_HIP(hipMemcpyAsync(out, r.out, r.out_nvals * 4, hipMemcpyDeviceToHost, t->stream));
+    Stager* sg = Stager::get(t->device);
+    if (pull && r.out_nvals && !out_pinned) {
+      if (r.gather_deferred || (sg && r.out_nvals * 4 >= kPipeBytes && !host_pool_owns(out, r.out_nvals * 4))) {
+        // piece by piece: the gather of a piece (when it is still owed), its transfer, and the copy
+        // into the caller's buffer overlap with those of the neighbouring pieces
+        if (!sg) return set_error(PSKV_ENOMEM, "no pinned memory to stage the response through");
+        std::function<int(size_t, size_t)> gather;
+        if (r.gather_deferred) {
+          gather = [&](size_t off, size_t len) {
+            return r.gather_varlen ? launch_rows_piece<true>(bt, kOpGather, off / 4, len / 4)
+                                   : launch_rows_piece<false>(bt, kOpGather, off / 4, len / 4);
+          };
+        }
+        rc = sg->to_host(out, r.out, r.out_nvals * 4, t->stream, gather);
+        if (rc) return rc;
+      } else {
+        PSKV_HIP(hipMemcpyAsync(out, r.out, r.out_nvals * 4, hipMemcpyDeviceToHost, t->stream));
+      }
+    }
     if (pull && varlen && out_lens && n && !lens_pinned)
       PSKV_HIP(hipMemcpyAsync(out_lens, r.out_lens, n * 4, hipMemcpyDeviceToHost, t->stream));
     if (t->mode == PSKV_MODE_SCALAR) {

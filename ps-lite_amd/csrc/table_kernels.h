@@ -54,7 +54,8 @@ struct TableReq {
   // `tile_key`
   unsigned long long* outcome;  // pinned host word that learns how the comparison went, or null
   uint32_t cache_mode;          // kCache* below
-  uint32_t pad;
+  uint32_t tile_base;           // row kernels: the launch starts at this tile of the request (a large
+                                // host-resident request is served piece by piece as it arrives)
 };
 constexpr uint32_t kCacheOff = 0;     // SCALAR: the request neither uses nor fills the key cache
 constexpr uint32_t kCacheOn = 1;      // SCALAR: serve from the cache when the keys match, else refill it
@@ -660,6 +661,7 @@ struct RowsParams {
   uint32_t ignore_new;    // pull half of a push+pull: rows created by the push half hold data
   uint32_t total_on_device;  // VARLEN pull without a host round trip: the floats to move are
                              // DevState::scan_total and `total` is the room in req
+  uint32_t blk;              // the workgroup's number among those that cover the request
   ReqTag tag;
 };
 
@@ -700,7 +702,7 @@ __device__ __forceinline__ void rows_tile_fixed(const RowsParams& p, uint64_t to
   constexpr int kIter = TILE / (VEC * kBlock);      // elements per thread
   constexpr int kGroup = kIter < 4 ? kIter : 4;     // loads issued back to back
   static_assert(kIter >= 1 && kIter % kGroup == 0, "tile does not divide over the workgroup");
-  const uint64_t f0 = (uint64_t)blockIdx.x * TILE;
+  const uint64_t f0 = (uint64_t)p.blk * TILE;
   if (f0 >= total) return;
   const uint32_t tile_floats = (uint32_t)((total - f0 < (uint64_t)TILE) ? (total - f0) : (uint64_t)TILE);
   const uint32_t nelem = tile_floats / VEC;
@@ -793,7 +795,7 @@ __device__ __forceinline__ void rows_wave_ask(const RowsParams& p, uint64_t boun
   using V = typename VecT<VEC>::type;
   constexpr int kIter = WTILE / (VEC * 64);
   const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const uint64_t wt = (uint64_t)blockIdx.x * (kBlock / 64) + wave;
+  const uint64_t wt = (uint64_t)p.blk * (kBlock / 64) + wave;
   const uint64_t f0 = wt * WTILE;
   const uint64_t left = bound > f0 ? bound - f0 : 0;  // 0: the tile lies past the data
   const uint32_t nelem = (uint32_t)(left < (uint64_t)WTILE ? left : (uint64_t)WTILE) / VEC;
@@ -828,7 +830,7 @@ __device__ __forceinline__ bool rows_wave_affine(const RowsParams& p, uint64_t t
   static_assert(WTILE < (1u << kTileSplitBits), "the split index does not fit the note");
   if (aff.first == kTileNotAffine) return false;
   const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const uint64_t wt = (uint64_t)blockIdx.x * (kBlock / 64) + wave;
+  const uint64_t wt = (uint64_t)p.blk * (kBlock / 64) + wave;
   const uint64_t f0 = wt * WTILE;
   if (f0 >= total) return true;
   const uint32_t nelem = (uint32_t)((total - f0 < (uint64_t)WTILE) ? (total - f0) : (uint64_t)WTILE) / VEC;
@@ -868,7 +870,7 @@ __device__ __forceinline__ void rows_wave_varlen(const RowsParams& p, uint64_t t
   constexpr int kIter = WTILE / (VEC * 64);  // elements per lane
   static_assert(kIter >= 1 && kIter <= 8, "wave tile out of range");
   const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const uint64_t wt = (uint64_t)blockIdx.x * (kBlock / 64) + wave;
+  const uint64_t wt = (uint64_t)p.blk * (kBlock / 64) + wave;
   const uint64_t f0 = wt * WTILE;
   if (f0 >= total) return;  // the whole wavefront leaves; nothing below synchronises workgroups
   const uint32_t tile_floats = (uint32_t)((total - f0 < (uint64_t)WTILE) ? (total - f0) : (uint64_t)WTILE);
@@ -1017,7 +1019,7 @@ __global__ __launch_bounds__(kBlock) void k_rows(ReqBatch b) {
   const TableReq& d = b.t[blockIdx.y];
   // the grid is sized for the largest table of the launch: workgroups (VARLEN: wavefronts) past
   // this table's floats leave before they touch anything
-  if (((uint64_t)blockIdx.x * (kBlock / 64) + (VARLEN ? (threadIdx.x >> 6) : 0u)) *
+  if ((((uint64_t)blockIdx.x + d.tile_base) * (kBlock / 64) + (VARLEN ? (threadIdx.x >> 6) : 0u)) *
           (VARLEN ? kTileVar : kTileFixed / (kBlock / 64)) >= d.total)
     return;
   RowsParams p;
@@ -1034,6 +1036,7 @@ __global__ __launch_bounds__(kBlock) void k_rows(ReqBatch b) {
   p.force_scalar = d.force_scalar;
   p.ignore_new = d.ignore_new;
   p.total_on_device = d.total_on_device;
+  p.blk = blockIdx.x + d.tile_base;
   p.tag = d.tag;
   __shared__ int32_t s_off[VARLEN ? (kWaveSpan + 1) * (kBlock / 64) : 1];
   __shared__ uint64_t s_ref[VARLEN ? kWaveSpan * (kBlock / 64) : 1];
@@ -1050,7 +1053,7 @@ __global__ __launch_bounds__(kBlock) void k_rows(ReqBatch b) {
   }
   if (VARLEN) {
     // the grid covers the room in the caller's buffer, which may be more than the data
-    const uint64_t f0 = ((uint64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6)) * kTileVar;
+    const uint64_t f0 = ((uint64_t)p.blk * (kBlock / 64) + (threadIdx.x >> 6)) * kTileVar;
     if (f0 >= p.total) return;
     // the loads that need no facts are on their way before the facts are looked at
     f32x4 x4[kTileVar / 256];
@@ -1066,7 +1069,7 @@ __global__ __launch_bounds__(kBlock) void k_rows(ReqBatch b) {
     if (p.total_on_device) {
       total = facts.scan_total;
       if (total > p.total) {  // the response does not fit the caller's buffer: write nothing
-        if (blockIdx.x == 0 && threadIdx.x == 0) atomicOr(&p.st->error, kDevErrNoRoom);
+        if (p.blk == 0 && threadIdx.x == 0) atomicOr(&p.st->error, kDevErrNoRoom);
         return;
       }
     }

@@ -110,6 +110,34 @@ def test_config3_dense_chunks_full(capi, orc, dev):
     assert t.size() == (nk, nk * k)
 
 
+def test_config3_dense_chunks_from_host_memory(capi, orc, dev):
+    """Configuration 3 the way a ps-lite server gets it: the 1 GiB of every push sits in ordinary host
+    memory and the pull answers into host memory. 3 worker pushes and a full pull, bit for bit against
+    the oracle; the requests travel through the ring of pinned pieces, 128 pieces per GiB."""
+    import time
+    announce("config3 from host memory")
+    nk, k, workers = 64, 4194304, 3
+    keys = np.uint64(KMAX // nk) * np.arange(nk, dtype=np.uint64)
+    t = capi.Table(capi.MODE_FIXED, row_len=k, arena_floats=nk * k)
+    o = orc.Store(orc.MODE_FIXED, k)
+    secs = []
+    for w in range(workers):
+        vals = np.random.default_rng(0xD15E + w).uniform(-1, 1, size=nk * k).astype(np.float32)
+        t0 = time.perf_counter()
+        t.push(keys, vals)
+        secs.append(time.perf_counter() - t0)
+        o.push(keys, vals)
+    out = np.empty(nk * k, np.float32)
+    t0 = time.perf_counter()
+    assert t.pull(keys, out) == nk * k
+    pull_s = time.perf_counter() - t0
+    rc, want, _, _ = o.handle(False, True, keys, out_cap=nk * k)
+    assert rc == 0
+    assert_bits_equal(out, want, "config3 host")
+    print("host-resident 1 GiB push: %s GB/s, pull: %.1f GB/s" % (
+        ", ".join("%.1f" % (nk * k * 4 / s / 1e9) for s in secs), nk * k * 4 / pull_s / 1e9))
+
+
 def _zipf_unique(rng, n, universe, s=1.1):
     """n distinct ranks in [0, universe) with Zipf(s) popularity, sorted."""
     got = np.zeros(0, np.int64)

@@ -21,3 +21,15 @@ def test_kv_app_through_adapters(num_servers):
     print(r.stdout)
     assert r.returncode == 0, r.stdout
     assert "test_kv_app_gpu: ok" in r.stdout
+
+
+def test_dense_chunks_from_host_memory_through_adapters():
+    """Configuration 3 (64 keys x 4,194,304 floats, 1 GiB per request) from ordinary host memory through
+    GpuSlicer + GpuKVHandle and through the C ABI alone; the program checks the sums against their closed
+    form and prints the PCIe-inclusive rates (they are not the benchmark's `value`)."""
+    announce("dense_from_host_through_adapters")
+    assert os.path.exists(BIN), "build() compiles tests/test_kv_app_gpu"
+    r = subprocess.run([BIN, "1", "4194304"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=280)
+    print(r.stdout)
+    assert r.returncode == 0, r.stdout
+    assert "dense from host memory" in r.stdout and "test_kv_app_gpu: ok" in r.stdout

@@ -1056,3 +1056,52 @@ def test_scalar_key_cache_at_its_real_size(capi, orc, dev, memkind):
         assert_bits_equal(out, out_np, "pushpull")
     t.sync()
     _check_dump(t, o, "scalar key cache")
+
+
+@pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
+def test_large_host_requests_travel_piece_by_piece(capi, orc, dev, mode):
+    """Host-resident requests of tens of megabytes go through the ring of pinned pieces (8 MiB each):
+    copy into the ring, transfer and row kernels overlap piece by piece, in both directions. Sizes that
+    are not multiples of a piece, a row length that is not a multiple of four, push, pull and push+pull."""
+    announce("large_host_requests", mode)
+    rng = np.random.default_rng(31)
+    if mode == "scalar":
+        n, k = 3000017, 1
+        lens = None
+    elif mode == "fixed":
+        n, k = 1999, 12289  # 98 MB per request, rows that are no multiple of 16 bytes
+        lens = None
+    else:
+        n = 250001
+        lens = rng.choice(np.array([0, 8, 16, 64, 128, 300], np.int32), size=n).astype(np.int32)
+        k = 0
+    nvals = n * k if lens is None else int(lens.sum())
+    m = {"scalar": capi.MODE_SCALAR, "fixed": capi.MODE_FIXED, "varlen": capi.MODE_VARLEN}[mode]
+    om = {"scalar": orc.MODE_SCALAR, "fixed": orc.MODE_FIXED, "varlen": orc.MODE_VARLEN}[mode]
+    t = capi.Table(m, initial_capacity=16)
+    o = orc.Store(om)
+    keys = unique_keys(rng, n)
+    for rep in range(2):
+        vals = rng.normal(0, 1, size=nvals).astype(np.float32)
+        t.push(keys, vals, lens)
+        o.push(keys, vals, lens)
+    want, want_lens = o.pull(keys)
+    got = np.full(nvals, 7.0, np.float32)
+    got_lens = np.full(n, -1, np.int32) if mode == "varlen" else None
+    assert t.pull(keys, got, got_lens) == nvals
+    assert_bits_equal(got, want, "pull")
+    if mode == "varlen":
+        assert np.array_equal(got_lens, want_lens)
+    vals = rng.normal(0, 1, size=nvals).astype(np.float32)
+    want, _ = o.pushpull(keys, vals, lens)
+    got = np.full(nvals, 7.0, np.float32)
+    t.pushpull(keys, vals, got, lens, got_lens)
+    assert_bits_equal(got, want, "pushpull")
+    # a pull of half the keys plus as many absent ones (FIXED creates them as zero rows while it answers)
+    probe = np.unique(np.concatenate([keys[::2], unique_keys(rng, n // 2)]))
+    want, want_lens = o.pull(probe)
+    got = np.full(want.size, 7.0, np.float32)
+    got_lens = np.full(probe.size, -1, np.int32) if mode == "varlen" else None
+    assert t.pull(probe, got, got_lens) == want.size
+    assert_bits_equal(got, want, "pull of other keys")
+    assert t.size() == o.size()

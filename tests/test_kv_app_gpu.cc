@@ -3,7 +3,7 @@
 // worker program, the same closed forms, plus the multi-float layouts and the failure
 // cases of the data path.
 //
-//   test_kv_app_gpu [num_servers]
+//   test_kv_app_gpu [num_servers [floats per key of the dense run from host memory]]
 #include <chrono>
 #include <cmath>
 #include <cstdio>
@@ -163,6 +163,69 @@ static void RunVarLen() {
   for (size_t i = 0; i < again.size() && i < total; ++i) EXPECT(again[i] == 5 * vals[i]);
 }
 
+// Dense chunks the way a ps-lite server gets them (BASELINE configuration 3: 64 keys of 4,194,304
+// floats, 1 GiB per push): requests in ordinary host memory through the slicer and the request
+// handle, the response in pinned buffers that the worker copies out of (kv_app.h:701-708). Prints
+// the PCIe-inclusive rates; the sums are checked against their closed form.
+static void RunDenseFromHost(size_t floats_per_key) {
+  const int num = 64;
+  KVWorker<float> kv(5, 0);
+  kv.set_slicer(pskv::GpuSlicer<float>(0));
+  std::vector<Key> keys(num);
+  for (int i = 0; i < num; ++i) keys[i] = kMaxKey / num * i;
+  std::vector<float> vals(num * floats_per_key);
+  for (size_t i = 0; i < vals.size(); ++i) vals[i] = static_cast<float>(static_cast<int>(i % 251) - 125);
+  const double gib = vals.size() * sizeof(float) / 1073741824.0;
+  // the zero-copy calls (kv_app.h:243-258): Push/Pull would first copy the gigabyte into an SArray
+  SArray<Key> zkeys(keys);
+  SArray<float> zvals(vals);
+  SArray<float> out(vals.size());
+  kv.Wait(kv.ZPush(zkeys, zvals));  // creates the rows, warms the staging buffers up
+  double best_push = 1e30, best_pull = 1e30;
+  for (int r = 0; r < 3; ++r) {
+    auto t0 = std::chrono::steady_clock::now();
+    kv.Wait(kv.ZPush(zkeys, zvals));
+    auto t1 = std::chrono::steady_clock::now();
+    kv.Wait(kv.ZPull(zkeys, &out));
+    auto t2 = std::chrono::steady_clock::now();
+    best_push = std::min(best_push, std::chrono::duration<double>(t1 - t0).count());
+    best_pull = std::min(best_pull, std::chrono::duration<double>(t2 - t1).count());
+  }
+  EXPECT(out.size() == vals.size());
+  size_t bad = 0;
+  for (size_t i = 0; i < out.size() && i < vals.size(); ++i) bad += out[i] != 4 * vals[i];
+  EXPECT(bad == 0);
+  std::printf("dense from host memory, %.2f GiB per request through GpuSlicer + GpuKVHandle: push %.1f GB/s, "
+              "pull %.1f GB/s (the pull includes the worker's own copy out of the response)\n",
+              gib, gib * 1.073741824 / best_push, gib * 1.073741824 / best_pull);
+  // the C ABI alone, ordinary (pageable) buffers both ways
+  pskv_opts o = pskv_opts();
+  o.mode = PSKV_MODE_FIXED;
+  o.row_len = floats_per_key;
+  pskv_table* t = nullptr;
+  EXPECT(pskv_table_create(&t, &o) == PSKV_OK);
+  std::vector<uint64_t> k64(keys.begin(), keys.end());
+  std::vector<float> out2(vals.size());
+  EXPECT(pskv_push(t, k64.data(), num, vals.data(), vals.size(), nullptr, 0, PSKV_MEM_HOST) == PSKV_OK);
+  best_push = best_pull = 1e30;
+  size_t got = 0;
+  for (int r = 0; r < 3; ++r) {
+    auto t0 = std::chrono::steady_clock::now();
+    EXPECT(pskv_push(t, k64.data(), num, vals.data(), vals.size(), nullptr, 0, PSKV_MEM_HOST) == PSKV_OK);
+    auto t1 = std::chrono::steady_clock::now();
+    EXPECT(pskv_pull(t, k64.data(), num, out2.data(), out2.size(), nullptr, &got, PSKV_MEM_HOST) == PSKV_OK);
+    auto t2 = std::chrono::steady_clock::now();
+    best_push = std::min(best_push, std::chrono::duration<double>(t1 - t0).count());
+    best_pull = std::min(best_pull, std::chrono::duration<double>(t2 - t1).count());
+  }
+  bad = 0;
+  for (size_t i = 0; i < out2.size(); ++i) bad += out2[i] != 4 * vals[i];
+  EXPECT(bad == 0 && got == vals.size());
+  std::printf("dense from host memory, %.2f GiB per request through pskv_push / pskv_pull (ordinary buffers): "
+              "push %.1f GB/s, pull %.1f GB/s\n", gib, gib * 1.073741824 / best_push, gib * 1.073741824 / best_pull);
+  pskv_table_destroy(t);
+}
+
 static void RunFailures(int num_servers) {
   KVWorker<float> kv(0, 1);
   kv.set_slicer(pskv::GpuSlicer<float>(0));
@@ -203,6 +266,10 @@ int main(int argc, char** argv) {
     RunFixed();
     RunVarLen();
     RunFailures(num_servers);
+    if (argc > 2) {  // floats per key of the dense run from host memory (4194304 is the configuration's)
+      auto s5 = StartServers(5, num_servers, PSKV_MODE_FIXED);
+      RunDenseFromHost(static_cast<size_t>(std::atoll(argv[2])));
+    }
   } catch (const std::exception& e) {
     std::fprintf(stderr, "unexpected exception: %s\n", e.what());
     return 2;
