@@ -72,8 +72,9 @@ typedef struct pskv_meta {
   int32_t priority;
 } pskv_meta;
 
-/* Van::PackMeta (van.cc:477-514); with_data_size != 0 adds field 11 like Van::PackMetaPB
- * (van.cc:445-475). Writes at most cap bytes and always sets *size to the bytes needed
+/* Van::PackMeta (van.cc:477-514); with_data_size != 0 packs like Van::PackMetaPB
+ * (van.cc:445-475) instead: field 11 (data_size) is written and field 12 (pull) is not, as
+ * that function never sets it. Writes at most cap bytes and always sets *size to the bytes needed
  * (PBMeta::ByteSize); returns 0, or -2 (PSKV_ESIZE_MISMATCH) when cap is too small. */
 int pskv_meta_pack(const pskv_meta* m, int with_data_size, char* buf, size_t cap, size_t* size);
 

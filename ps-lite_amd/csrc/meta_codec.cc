@@ -105,8 +105,11 @@ void write_meta(Sink& s, const pskv_meta& m, bool with_data_size) {
       s.varint(static_cast<uint64_t>(static_cast<int64_t>(m.data_type[i])));
   }
   s.int32_field(10, m.customer_id);
-  if (with_data_size) s.int32_field(11, m.data_size);
-  s.bool_field(12, m.pull);
+  if (with_data_size) {
+    s.int32_field(11, m.data_size);  // Van::PackMetaPB, van.cc:445-475: data_size, and pull is NOT set
+  } else {
+    s.bool_field(12, m.pull);        // Van::PackMeta, van.cc:485
+  }
   s.int32_field(13, m.priority);
 }
 

@@ -304,11 +304,16 @@ void give_ctx(SliceCtx* c) {
   g_pool.push_back(c);
 }
 
+// A context goes back to the pool only when nothing enqueued on its stream can still touch its
+// buffers: a call that leaves early (after a failed runtime call) waits for the stream first.
 struct CtxLease {
   SliceCtx* c;
+  bool idle = true;  // nothing has been enqueued since the stream was last waited for
   explicit CtxLease(int device) : c(take_ctx(device)) {}
   ~CtxLease() {
-    if (c) give_ctx(c);
+    if (!c) return;
+    if (!idle) (void)hipStreamSynchronize(c->stream);
+    give_ctx(c);
   }
 };
 
@@ -396,6 +401,7 @@ int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, 
     CtxLease lease(device);
     SliceCtx* c = lease.c;
     if (!c) return set_error(PSKV_EHIP, "cannot create a slicer context on device %d", device);
+    lease.idle = false;
     const bool do_sums = has_lens && nlens == n;
     if (do_sums && S > 65535) return set_error(PSKV_EINVAL, "more than 65535 ranges with lens");
     // device: lb[S+1] | pos[S+1] | sums[S]      pinned: targets[S+1] | pos[S+1] | sums[S]
@@ -456,6 +462,7 @@ int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, 
       PSKV_HIP(hipGetLastError());
     }
     PSKV_HIP(hipStreamSynchronize(c->stream));
+    lease.idle = true;
     for (size_t i = 0; i <= S; ++i) pos[i] = h_pos[i];
     if (do_sums)
       for (size_t i = 0; i < S; ++i) val_pos[i + 1] = h_sums[i];  // per-slice sums for now
@@ -616,6 +623,7 @@ int pskv_assemble_pull(int device, const uint64_t* req_keys, size_t n, size_t R,
     CtxLease lease(device);
     SliceCtx* c = lease.c;
     if (!c) return set_error(PSKV_EHIP, "cannot create a context on device %d", device);
+    lease.idle = false;
     // pinned, read and written by the kernels in place:
     //   key pointers[R] | nkeys[R] | targets[2R] | lower bounds[2R] | segments[2R]
     const size_t a = pad256(R * 8), b = pad256(2 * R * 8), sg = pad256(2 * R * sizeof(Segment));
@@ -637,6 +645,7 @@ int pskv_assemble_pull(int device, const uint64_t* req_keys, size_t n, size_t R,
     rc = launch_bounds_search(req_keys, n, h_targets, 2 * R, h_lb, c->stream);
     if (rc) return rc;
     PSKV_HIP(hipStreamSynchronize(c->stream));
+    lease.idle = true;
     for (size_t r = 0; r < R; ++r) {  // kv_app.h:670-677
       const uint64_t lower = h_targets[2 * r], upper = h_targets[2 * r + 1];
       const uint64_t size = upper <= lower ? 0 : h_lb[2 * r + 1] - h_lb[2 * r];  // sarray.h:283
@@ -672,6 +681,7 @@ int pskv_assemble_pull(int device, const uint64_t* req_keys, size_t n, size_t R,
       }
       koff += resp_nkeys[r];
     }
+    lease.idle = false;
     for (size_t first = 0; first < nseg; first += 65535) {  // gridDim.y holds 65535 segments
       const size_t now = std::min<size_t>(nseg - first, 65535);
       const uint64_t per = std::min<uint64_t>(longest / (16 * kBlock) + 1, 4096);
@@ -679,6 +689,7 @@ int pskv_assemble_pull(int device, const uint64_t* req_keys, size_t n, size_t R,
       PSKV_HIP(hipGetLastError());
     }
     PSKV_HIP(hipStreamSynchronize(c->stream));
+    lease.idle = true;
     return PSKV_OK;
   }
   if (total_key != n)

@@ -71,7 +71,9 @@ def pack_like_van(cls, h, with_data_size=False):
         pb.timestamp = h["timestamp"]
     if h.get("body"):
         pb.body = h["body"]
-    pb.push, pb.pull = bool(h.get("push")), bool(h.get("pull"))
+    pb.push = bool(h.get("push"))
+    if not with_data_size:  # Van::PackMetaPB (van.cc:445-475) never calls set_pull
+        pb.pull = bool(h.get("pull"))
     pb.request, pb.simple_app = bool(h.get("request")), bool(h.get("simple_app"))
     pb.priority, pb.customer_id = h.get("priority", 0), h.get("customer_id", 0)
     pb.data_type.extend(h.get("data_type", []))

@@ -43,6 +43,8 @@ def _as_unpacked(h, with_data_size=False):
     """What Van::UnpackMeta (van.cc:516-557) makes of a header packed by Van::PackMeta."""
     u = dict(h)
     u["data_size"] = h["data_size"] if with_data_size else 0
+    if with_data_size:
+        u["pull"] = False  # Van::PackMetaPB (van.cc:445-475) never sets it, so it does not travel
     c = h["control"]
     if c is not None:
         # only the field that belongs to the command travels (van.cc:494-498)
