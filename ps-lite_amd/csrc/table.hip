@@ -500,6 +500,9 @@ struct Item {
   // var-len workspace of the request
   int32_t* tmp_lens = nullptr;
   uint64_t nparts = 0, tiles_cap = 0;
+  // SCALAR: the slots may lag behind the key cache and must be written back if the device finds
+  // that this request does not repeat the cached keys
+  bool flush_unless_same = false;
 };
 typedef std::vector<Item> Batch;
 
@@ -642,7 +645,6 @@ int run_scalar(Batch& bt, bool push, bool pull) {
   uint64_t n_largest = 0;
   bool any_cache = false;
   std::vector<ScalarCacheUse> use(bt.size(), kScPlain);
-  std::vector<char> flush_unless_same(bt.size(), 0);
   for (size_t i = 0; i < bt.size(); ++i) {
     Item& it = bt[i];
     pskv_table* t = it.t;
@@ -683,7 +685,7 @@ int run_scalar(Batch& bt, bool push, bool pull) {
       d.outcome = t->outcome;
       d.cache_mode = kCacheOn;
       any_cache = true;
-      flush_unless_same[i] = (it.tag.try_cache && t->sc_dirty) ? 1 : 0;
+      it.flush_unless_same = it.tag.try_cache && t->sc_dirty;
     }
     d.slots = t->slots;
     d.mask = t->cap - 1;
@@ -705,9 +707,8 @@ int run_scalar(Batch& bt, bool push, bool pull) {
     // slots that lag behind the cache are written back once the device knows that the request
     // does NOT repeat the cached keys (cache_mode reads as kFlushUnlessSame in that kernel)
     static_assert(kFlushUnlessSame == kCacheOn, "one descriptor serves both kernels");
-    size_t i = 0;
-    rc = launch_batch(bt, -1, k_scalar_flush, [&](const Item& it) {
-      return flush_unless_same[i++] ? (uint64_t)grid_for(it.r.n, kBlock, kMaxGrid) : 0ull;
+    rc = launch_batch(bt, -1, k_scalar_flush, [](const Item& it) {
+      return it.flush_unless_same ? (uint64_t)grid_for(it.r.n, kBlock, kMaxGrid) : 0ull;
     });
     if (rc) return rc;
   }
