@@ -136,17 +136,29 @@ def kernel_stats(tables, kernel):
     return n, ms, np.concatenate(samples) if samples else np.zeros(0, np.float32)
 
 
-def pull_entries(units, pull, same, traffic_plain):
+def pull_entries(units, pull, same, per_key, traffic_plain, traffic_per_key=None):
     """The `kernels` entries of a SCALAR pull. Once a table has seen pulls come right behind pushes
-    of the same keys it serves them from its key cache: the pull kernel then only streams the cached
-    values (8 B/key) and the keys are compared by k_same_keys (16 B/key) in front of it, which
-    together are the 24 B/key of a pull that goes through the slots."""
+    of the same keys, the pushes leave their keys and values behind in request order and such a
+    pull compares and answers in one pass over them (24 B/key, all of it streamed). A pull that
+    repeats a key set whose values have run ahead of the slots is decided as a whole first: the
+    keys are compared by k_same_keys (16 B/key) and the pull kernel streams the values (8 B/key).
+    Any other pull goes through the slots (24 B/key algorithmic, a 128-byte line per key)."""
+    out = {}
+    if per_key[0]:
+        out["pull_scalar"] = dict(roofline(24.0 * units, per_key[0], per_key[1], traffic_per_key, per_key[2]),
+                                  bytes_per_key=24,
+                                  path="compared with the keys the push left behind and answered from its "
+                                       "values, one pass")
+        if pull[0]:
+            out["pull_scalar_slots"] = dict(roofline(24.0 * units, pull[0], pull[1], traffic_plain, pull[2]),
+                                            bytes_per_key=24, path="through the slots")
+        return out
     cached = same[0] > 0
-    out = {"pull_scalar": dict(roofline((8.0 if cached else 24.0) * units, pull[0], pull[1],
-                                        None if cached else traffic_plain, pull[2]),
-                               bytes_per_key=8 if cached else 24,
-                               path="served from the key cache (k_same_keys in front)" if cached
-                                    else "through the slots")}
+    out["pull_scalar"] = dict(roofline((8.0 if cached else 24.0) * units, pull[0], pull[1],
+                                       None if cached else traffic_plain, pull[2]),
+                              bytes_per_key=8 if cached else 24,
+                              path="served from the key cache (k_same_keys in front)" if cached
+                                   else "through the slots")
     if cached:
         out["same_keys"] = dict(roofline(16.0 * units, same[0], same[1], None, same[2]), bytes_per_key=16,
                                 kernel="k_same_keys (request keys against cached keys)")
@@ -203,19 +215,27 @@ def run_sparse_lr(args, capi, dev):
     tables = group.tables
     per_table = args.per_table
 
-    def step(i, sample=True):
+    prof_on = [-1]  # the table whose launches carry events at the moment (-1: none)
+
+    def slice_step(i):
+        return capi.slice_keys(d_batches[i][0], rb, re, nvals=n)
+
+    def step(i, sliced, sample=True):
         # Kernel durations are sampled INSIDE the timed steps: in every SAMPLE_EVERY-th step the
         # launches carry their own start/stop events (booked to the first table of the group; with
         # --per-table those of one of the S tables, taken in turn). Events on every launch would
         # cost more host time per step than the GPU needs for it.
         if sample:
             j = i - args.warmup
-            for s in range(S):
-                tables[s].prof_enable(sampled(j, args.steps) and
-                                      s == ((j // SAMPLE_EVERY) % S if per_table else 0))
+            on = sampled(j, args.steps)
+            which = ((j // SAMPLE_EVERY) % S if per_table else 0) if on else -1
+            if which != prof_on[0]:
+                for s in range(S):
+                    tables[s].prof_enable(s == which)
+                prof_on[0] = which
         dk, dv = d_batches[i]
         kp, vp, op = dk.data_ptr(), dv.data_ptr(), out.data_ptr()
-        pos, _, used = capi.slice_keys(dk, rb, re, nvals=n)
+        pos, _, used = sliced
         if not per_table:
             # one launch per step of the pipeline over all S key ranges
             group.push_raw(kp, pos, vp, pos)
@@ -231,6 +251,13 @@ def run_sparse_lr(args, capi, dev):
                 c = pos[s + 1] - pos[s]
                 tables[s].pull_raw(kp + 8 * pos[s], c, op + 4 * pos[s], c)
 
+    def steps(first, last, sample=True):
+        # Every step slices its keys, pushes and pulls, in line. (Slicing the keys of coming steps
+        # ahead of time, on this thread or on a second one, was measured and gains nothing: the
+        # slicer's short kernel shares the GPU with the store's long ones either way.)
+        for i in range(first, last):
+            step(i, slice_step(i), sample)
+
     def drain():
         if per_table:
             for t in tables:
@@ -239,19 +266,18 @@ def run_sparse_lr(args, capi, dev):
             group.sync()
         torch.cuda.synchronize()
 
-    for i in range(args.warmup):
-        step(i)
+    steps(0, args.warmup)
     drain()
     for t in tables:
         t.prof_reset()
     t0 = time.perf_counter()
-    for i in range(args.warmup, args.warmup + args.steps):
-        step(i)
+    steps(args.warmup, args.warmup + args.steps)
     drain()
     dt = time.perf_counter() - t0
     push_n, push_ms, push_s = kernel_stats(tables, capi.KERNEL_PUSH_SCALAR)
     pull_st = kernel_stats(tables, capi.KERNEL_PULL_SCALAR)
     same_st = kernel_stats(tables, capi.KERNEL_SAME_KEYS)
+    per_key_st = kernel_stats(tables, capi.KERNEL_PULL_PER_KEY)
     for t in tables:
         t.prof_enable(False)
 
@@ -273,12 +299,10 @@ def run_sparse_lr(args, capi, dev):
         own = [capi.Table(capi.MODE_SCALAR, initial_capacity=cap) for _ in range(S)]
         shared, tables = tables, own
         was_per_table, per_table = per_table, True  # tables with streams of their own go one by one
-        for i in range(args.warmup):
-            step(i, sample=False)
+        steps(0, args.warmup, sample=False)
         drain()
         t1 = time.perf_counter()
-        for i in range(args.warmup, args.warmup + args.steps):
-            step(i, sample=False)
+        steps(args.warmup, args.warmup + args.steps, sample=False)
         drain()
         dt_own = time.perf_counter() - t1
         assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32)), "pulled values differ"
@@ -293,12 +317,10 @@ def run_sparse_lr(args, capi, dev):
         main_group, main_tables = group, tables
         group = capi.Group(S, capi.MODE_SCALAR, stream=stream.cuda_stream)
         tables = group.tables
-        for i in range(args.warmup):
-            step(i, sample=False)
+        steps(0, args.warmup, sample=False)
         drain()
         t2 = time.perf_counter()
-        for i in range(args.warmup, args.warmup + args.steps):
-            step(i, sample=False)
+        steps(args.warmup, args.warmup + args.steps, sample=False)
         drain()
         dt_grow = time.perf_counter() - t2
         assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32)), "pulled values differ"
@@ -327,7 +349,9 @@ def run_sparse_lr(args, capi, dev):
         "roofline": dict(roofline(32.0 * keys_per_launch, push_n, push_ms,
                                   traffic("push_scalar", keys_per_launch), push_s),
                          kernel="k_scalar<push> (find-or-insert + add)", bytes_per_key=32),
-        "kernels": dict(pull_entries(keys_per_launch, pull_st, same_st, traffic("pull_scalar", keys_per_launch)),
+        "kernels": dict(pull_entries(keys_per_launch, pull_st, same_st, per_key_st,
+                                     traffic("pull_scalar", keys_per_launch),
+                                     traffic("pull_per_key", keys_per_launch)),
                         slicer={"wall_us_per_call": round(slice_us, 1), "keys": n, "ranges": S}),
     }
     if dt_own is not None:
@@ -693,7 +717,7 @@ def run_zipf(args, capi, dev):
         # between a hit (28 B/key) and an insert (32 B/key); priced as inserts
         "roofline": dict(roofline(32.0 * n, push[0], push[1], None, push[2]),
                          kernel="k_scalar<push> (find-or-insert + add)", bytes_per_key=32),
-        "kernels": dict(pull_entries(n, pull, same, None),
+        "kernels": dict(pull_entries(n, pull, same, (0, 0.0, []), None),
                         rehash={"launches": rehash[0], "total_us": round(rehash[1] * 1e3, 1)}),
     }
     return res, batches[args.warmup:], n

@@ -69,7 +69,9 @@ extern "C" {
 #define PSKV_KERNEL_REHASH 5
 #define PSKV_KERNEL_COPY 6        /* the plain copy of pskv_copy_probe */
 #define PSKV_KERNEL_SAME_KEYS 7   /* comparison of a request's keys with the cached key set */
-#define PSKV_KERNEL_COUNT 8
+#define PSKV_KERNEL_PULL_PER_KEY 8 /* SCALAR pull right behind the push that filled the key cache: keys
+                                     compared and values answered in one pass (booked by a launch's first table) */
+#define PSKV_KERNEL_COUNT 9
 
 typedef struct pskv_table pskv_table;
 

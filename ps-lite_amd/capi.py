@@ -6,6 +6,7 @@ memory here; every computation happens inside libpskv.so.
 """
 import ctypes
 import os
+import sys
 
 import numpy as np
 
@@ -27,7 +28,7 @@ MODE_VARLEN = 2
 MAX_VARLEN_ROW = (1 << 28) - 1
 SLICE_NOALLOC_MAX_RANGES = 1024
 KERNEL_PUSH_SCALAR, KERNEL_PULL_SCALAR, KERNEL_ROWS_ACC, KERNEL_ROWS_GATHER, KERNEL_LOOKUP, \
-    KERNEL_REHASH, KERNEL_COPY, KERNEL_SAME_KEYS = range(8)
+    KERNEL_REHASH, KERNEL_COPY, KERNEL_SAME_KEYS, KERNEL_PULL_PER_KEY = range(9)
 
 ERROR_NAMES = {
     EUNCOVERED_KEY: "PSKV_EUNCOVERED_KEY", ESIZE_MISMATCH: "PSKV_ESIZE_MISMATCH",
@@ -165,6 +166,10 @@ class Table:
             self._h = ctypes.c_void_p()
 
     def __del__(self):
+        # Not while the interpreter shuts down: a stream that the caller lent (torch's, say) may be
+        # gone by then, and the process is about to give everything back anyway.
+        if sys is None or sys.is_finalizing():
+            return
         try:
             self.close()
         except Exception:
@@ -278,6 +283,10 @@ class Group:
         self.tables = []
 
     def __del__(self):
+        # Not while the interpreter shuts down: a stream that the caller lent (torch's, say) may be
+        # gone by then, and the process is about to give everything back anyway.
+        if sys is None or sys.is_finalizing():
+            return
         try:
             self.close()
         except Exception:

@@ -654,6 +654,7 @@ int run_scalar(Batch& bt, bool push, bool pull) {
     if (r.n == 0) continue;
     int rc = reserve(t, r.n, 0, 0, &it.pub);  // (a growth writes the cache back and drops it)
     if (rc) return rc;
+    const int kind_before = t->sc_last_kind;
     use[i] = scalar_cache_use(t, r);
     if (use[i] != kScTry) {
       // the request goes through the slots, so they must be up to date; a push then makes the
@@ -683,9 +684,12 @@ int run_scalar(Batch& bt, bool push, bool pull) {
       d.arena = static_cast<float*>(t->sc_vals.ptr);
       d.tile_key = static_cast<uint32_t*>(t->sc_slots.ptr);
       d.outcome = t->outcome;
-      d.cache_mode = kCacheOn;
+      // A pull right behind a push, with the slots up to date (the push went through them and
+      // recorded itself): the pull kernel compares key by key and needs no launch in front of it.
+      const bool per_key = use[i] == kScTry && !push && !t->sc_dirty && kind_before == 0;
+      d.cache_mode = per_key ? kCachePerKey : kCacheOn;
       any_cache = true;
-      it.flush_unless_same = it.tag.try_cache && t->sc_dirty;
+      it.flush_unless_same = !per_key && it.tag.try_cache && t->sc_dirty;
     }
     d.slots = t->slots;
     d.mask = t->cap - 1;
@@ -700,7 +704,7 @@ int run_scalar(Batch& bt, bool push, bool pull) {
   int rc;
   if (any_cache) {
     rc = launch_batch(bt, PSKV_KERNEL_SAME_KEYS, k_same_keys, [](const Item& it) {
-      return (it.d.cache_mode && it.tag.try_cache)
+      return (it.d.cache_mode == kCacheOn && it.tag.try_cache)
                  ? (it.r.n + kBlock * kSameKeysItems - 1) / (kBlock * kSameKeysItems) : 0ull;
     });
     if (rc) return rc;
@@ -718,7 +722,8 @@ int run_scalar(Batch& bt, bool push, bool pull) {
   // lane takes four turns).
   auto nblk = [&](const Item& it) -> uint64_t {
     if (!it.d.n) return 0;
-    return grid_for(it.d.n, (it.d.cache_mode && it.tag.try_cache) ? kBlock * 4 : kBlock, kMaxGrid);
+    const bool four = (it.d.cache_mode == kCacheOn && it.tag.try_cache) || it.d.cache_mode == kCachePerKey;
+    return grid_for(it.d.n, four ? kBlock * 4 : kBlock, kMaxGrid);
   };
   if (push && pull) {
     rc = any_cache ? launch_batch(bt, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, true, true>, nblk)
@@ -727,7 +732,8 @@ int run_scalar(Batch& bt, bool push, bool pull) {
     rc = any_cache ? launch_batch(bt, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, false, true>, nblk)
                    : launch_batch(bt, PSKV_KERNEL_PUSH_SCALAR, k_scalar<true, false, false>, nblk);
   } else {
-    rc = any_cache ? launch_batch(bt, PSKV_KERNEL_PULL_SCALAR, k_scalar<false, true, true>, nblk)
+    const int kind = bt[0].d.cache_mode == kCachePerKey ? PSKV_KERNEL_PULL_PER_KEY : PSKV_KERNEL_PULL_SCALAR;
+    rc = any_cache ? launch_batch(bt, kind, k_scalar<false, true, true>, nblk)
                    : launch_batch(bt, PSKV_KERNEL_PULL_SCALAR, k_scalar<false, true, false>, nblk);
   }
   if (rc) return rc;

@@ -59,6 +59,8 @@ struct TableReq {
 };
 constexpr uint32_t kCacheOff = 0;     // SCALAR: the request neither uses nor fills the key cache
 constexpr uint32_t kCacheOn = 1;      // SCALAR: serve from the cache when the keys match, else refill it
+constexpr uint32_t kCachePerKey = 3;  // SCALAR pull, slots up to date: every key that sits at its cached
+                                      // position is answered from the cache, the others through the slots
 constexpr uint32_t kFlushUnlessSame = 1;  // k_scalar_flush: skip when the request in flight repeats the cache
 constexpr uint32_t kFlushAlways = 2;
 constexpr uint32_t kSlotSpecial = 0xffffffffu;  // cached slot number of key 2^64-1 (the side slot)
@@ -89,6 +91,8 @@ static_assert(sizeof(ReqBatch) <= 3840, "kernel arguments are limited to 4 KiB")
 // key instead of a 128-byte line per probe; the slots are brought up to date (k_scalar_flush)
 // before anything else looks at them. A request that does not repeat the cache goes the usual
 // way and leaves its keys, their values and their slot numbers behind as the new cache.
+// A pull that comes right behind the push that filled the cache (the slots are up to date then)
+// needs no decision for the whole request: kCachePerKey compares key by key, in the same pass.
 template <bool PUSH, bool PULL, bool CACHE>
 __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
   const TableReq& d = b.t[blockIdx.y];
@@ -126,12 +130,72 @@ __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
     return;
   }
   if (record && blockIdx.x == 0 && threadIdx.x == 0) st->cache_epoch = d.tag.epoch;
+  constexpr bool kPerKey = CACHE && PULL && !PUSH;
+  bool per_key = false, differs = false;
+  if (kPerKey) {
+    // (nothing writes these two words while a pull of this kind runs)
+    per_key = d.cache_mode == kCachePerKey && st->cache_epoch != 0ull && st->bad_epoch != st->cache_epoch;
+  }
   __shared__ unsigned red[kBlock / 64];
   unsigned created = 0;
+  if (kPerKey && per_key) {
+    // Four keys per lane, 128 bits per load. The cached request had no repeats, so four keys that
+    // equal their cached neighbours are four different keys; the key behind them says whether
+    // the last of them starts a run, which goes through the slots as a whole.
+    const uint64_t* __restrict__ ck = d.cache_keys;
+    const float* __restrict__ cv = d.arena;
+    const bool kvec = (reinterpret_cast<uintptr_t>(keys) & 15) == 0;
+    const bool ovec = (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    const uint64_t stride4 = (uint64_t)nblk * kBlock * 4;
+    for (uint64_t i = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * 4; i < n; i += stride4) {
+      if (i + 4 <= n) {
+        u64x2 x0, x1;
+        if (kvec) {
+          x0 = __builtin_nontemporal_load(reinterpret_cast<const u64x2*>(keys + i));
+          x1 = __builtin_nontemporal_load(reinterpret_cast<const u64x2*>(keys + i + 2));
+        } else {
+          x0.x = keys[i], x0.y = keys[i + 1], x1.x = keys[i + 2], x1.y = keys[i + 3];
+        }
+        const u64x2 y0 = *reinterpret_cast<const u64x2*>(ck + i);
+        const u64x2 y1 = *reinterpret_cast<const u64x2*>(ck + i + 2);
+        const f32x4 v4 = *reinterpret_cast<const f32x4*>(cv + i);
+        const uint64_t behind = i + 4 < n ? keys[i + 4] : ~x1.y;
+        if (x0.x == y0.x && x0.y == y0.y && x1.x == y1.x && x1.y == y1.y && behind != x1.y) {
+          if (ovec) {
+            __builtin_nontemporal_store(v4, reinterpret_cast<f32x4*>(out + i));
+          } else {
+            out[i] = v4.x, out[i + 1] = v4.y, out[i + 2] = v4.z, out[i + 3] = v4.w;
+          }
+          continue;
+        }
+      }
+      for (uint64_t j = i; j < n && j < i + 4; ++j) {  // key by key
+        const uint64_t key = keys[j];
+        if (j > 0 && keys[j - 1] == key) continue;  // inside a run: its first key answers for it
+        const bool run = j + 1 < n && keys[j + 1] == key;
+        if (!run && ck[j] == key) {
+          out[j] = cv[j];
+          continue;
+        }
+        differs = true;
+        bool is_new;
+        uint64_t seen;
+        uint64_t* p = find_or_insert(slots, mask, st, key, is_new, seen);
+        if (!p) continue;
+        const float cur = is_new ? 0.0f : __uint_as_float((unsigned)seen);
+        out[j] = cur;
+        for (uint64_t r = j + 1; r < n && keys[r] == key; ++r) out[r] = cur;
+        if (is_new) *reinterpret_cast<float*>(p) = cur;
+        created += is_new ? 1u : 0u;
+      }
+    }
+  }
+  // every other request: one key per lane and turn through the slots
+  const uint64_t n_turns = (kPerKey && per_key) ? 0 : n;
   const uint64_t stride = (uint64_t)nblk * kBlock;
   const unsigned lane = threadIdx.x & 63;
   // whole wavefronts stay in the loop together: the shuffles below need every lane
-  for (uint64_t first = (uint64_t)blockIdx.x * kBlock; first < n; first += stride) {
+  for (uint64_t first = (uint64_t)blockIdx.x * kBlock; first < n_turns; first += stride) {
     const uint64_t i = first + threadIdx.x;
     const bool live = i < n;
     const uint64_t key = live ? keys[i] : 0;
@@ -170,6 +234,17 @@ __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
     }
   }
   block_count_add(st, created, red);
+  if (kPerKey && d.cache_mode == kCachePerKey) {
+    // tell the host, which never waits for it, whether every key sat at its cached position
+    const int any = __syncthreads_or(differs ? 1 : 0);
+    if (threadIdx.x == 0) {
+      if (any) atomicOr(&st->req_flags, kReqDiffer);
+      if (ticket_last(st, nblk)) {
+        const bool all = (atomicExch(&st->req_flags, 0u) & kReqDiffer) == 0u && per_key;
+        if (d.outcome) *d.outcome = (d.tag.epoch << 1) | (all ? 1ull : 0ull);
+      }
+    }
+  }
 }
 
 // Writes the cached values back to their slots. Launched before anything reads or changes the

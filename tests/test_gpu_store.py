@@ -1105,3 +1105,67 @@ def test_large_host_requests_travel_piece_by_piece(capi, orc, dev, mode):
     assert t.pull(probe, got, got_lens) == want.size
     assert_bits_equal(got, want, "pull of other keys")
     assert t.size() == o.size()
+
+
+@pytest.mark.parametrize("memkind", ["device", "host"])
+def test_pull_right_behind_a_push_compares_key_by_key(capi, orc, dev, memkind, small_scalar_cache):
+    """A worker that pushes gradients and pulls the weights of the same keys (tests/test_kv_app.cc:27-41)
+    shows as pulls right behind pushes of their size. Once pushes record themselves, such a pull is
+    answered from the recorded values wherever a key sits at its recorded position and through the
+    slots elsewhere: pulls of the pushed keys, of keys that differ in a few places (some absent from
+    the store, which a pull creates), of a sorted request that repeats a key, and of 2^64-1."""
+    import torch
+    announce("pull_behind_push", memkind)
+    rng = np.random.default_rng(77)
+    n = 1500
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=16)
+    o = orc.Store(orc.MODE_SCALAR)
+
+    def mem(a):
+        return to_dev(a, dev) if memkind == "device" else a
+
+    def push(k):
+        v = rng.normal(0, 1, size=k.size).astype(np.float32)
+        t.push(mem(k), mem(v))
+        o.push(k, v)
+
+    def pull(k, what):
+        want, _ = o.pull(k)
+        if memkind == "device":
+            out = torch.full((k.size,), 7.0, dtype=torch.float32, device=dev)
+            t.pull(to_dev(k, dev), out)
+            t.sync()
+            got = from_dev(out)
+        else:
+            got = np.full(k.size, 7.0, np.float32)
+            t.pull(k, got)
+        assert_bits_equal(got, want, what)
+
+    for step in range(4):  # fresh keys every step, as in a sparse model that keeps growing
+        k = unique_keys(rng, n)
+        push(k)
+        pull(k, "same keys, step %d" % step)
+    k = unique_keys(rng, n)
+    push(k)
+    other = k.copy()
+    other[10:20] = k[10:20] + np.uint64(1)  # absent keys (a pull creates them), still sorted
+    other[700] = k[701]                     # sorted repeats: k[701] twice within four keys,
+    other[703] = k[704]                     # k[704] twice across two lanes' keys
+    other[1499] = k[1498]                   # and the last key twice
+    assert np.all(other[1:] >= other[:-1])
+    pull(other, "keys that differ in a few places")
+    pull(k, "the pushed keys after all")
+    k2 = unique_keys(rng, n)
+    k2[-1] = np.uint64(2**64 - 1)
+    push(k2)
+    pull(k2, "with the largest key")
+    shifted = np.sort(np.concatenate([k2[1:], unique_keys(rng, 1)]))
+    push(k2)
+    pull(shifted, "every position holds another key")
+    for step in range(3):
+        k = unique_keys(rng, n)
+        push(k)
+        pull(k, "same keys again, step %d" % step)
+    t.sync()
+    _check_dump(t, o, "pull behind push")
+    t.close()
