@@ -144,21 +144,24 @@ def pull_entries(units, pull, same, per_key, traffic_plain, traffic_per_key=None
     keys are compared by k_same_keys (16 B/key) and the pull kernel streams the values (8 B/key).
     Any other pull goes through the slots (24 B/key algorithmic, a 128-byte line per key)."""
     out = {}
+    cached = same[0] > 0
     if per_key[0]:
         out["pull_scalar"] = dict(roofline(24.0 * units, per_key[0], per_key[1], traffic_per_key, per_key[2]),
                                   bytes_per_key=24,
                                   path="compared with the keys the push left behind and answered from its "
                                        "values, one pass")
         if pull[0]:
-            out["pull_scalar_slots"] = dict(roofline(24.0 * units, pull[0], pull[1], traffic_plain, pull[2]),
-                                            bytes_per_key=24, path="through the slots")
-        return out
-    cached = same[0] > 0
-    out["pull_scalar"] = dict(roofline((8.0 if cached else 24.0) * units, pull[0], pull[1],
-                                       None if cached else traffic_plain, pull[2]),
-                              bytes_per_key=8 if cached else 24,
-                              path="served from the key cache (k_same_keys in front)" if cached
-                                   else "through the slots")
+            out["pull_scalar_other"] = dict(roofline(24.0 * units, pull[0], pull[1], None, pull[2]),
+                                            bytes_per_key=24,
+                                            path="the other pulls of the run: through the slots" +
+                                                 (", or streamed from the key cache behind k_same_keys" if cached
+                                                  else ""))
+    else:
+        out["pull_scalar"] = dict(roofline((8.0 if cached else 24.0) * units, pull[0], pull[1],
+                                           None if cached else traffic_plain, pull[2]),
+                                  bytes_per_key=8 if cached else 24,
+                                  path="served from the key cache (k_same_keys in front)" if cached
+                                       else "through the slots")
     if cached:
         out["same_keys"] = dict(roofline(16.0 * units, same[0], same[1], None, same[2]), bytes_per_key=16,
                                 kernel="k_same_keys (request keys against cached keys)")
@@ -705,6 +708,7 @@ def run_zipf(args, capi, dev):
     push = kernel_stats([t], capi.KERNEL_PUSH_SCALAR)
     pull = kernel_stats([t], capi.KERNEL_PULL_SCALAR)
     same = kernel_stats([t], capi.KERNEL_SAME_KEYS)
+    per_key = kernel_stats([t], capi.KERNEL_PULL_PER_KEY)
     rehash = kernel_stats([t], capi.KERNEL_REHASH)
     held = t.size()[0]
     res = {
@@ -717,7 +721,7 @@ def run_zipf(args, capi, dev):
         # between a hit (28 B/key) and an insert (32 B/key); priced as inserts
         "roofline": dict(roofline(32.0 * n, push[0], push[1], None, push[2]),
                          kernel="k_scalar<push> (find-or-insert + add)", bytes_per_key=32),
-        "kernels": dict(pull_entries(n, pull, same, (0, 0.0, []), None),
+        "kernels": dict(pull_entries(n, pull, same, per_key, None),
                         rehash={"launches": rehash[0], "total_us": round(rehash[1] * 1e3, 1)}),
     }
     return res, batches[args.warmup:], n
