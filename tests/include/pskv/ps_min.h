@@ -1,8 +1,8 @@
 /*
  * A small in-process stand-in for the part of the ps-lite API that surrounds the
  * key-value data path, so that the GPU slicer and the GPU request handle can be
- * driven exactly the way a ps-lite program drives them, without a scheduler,
- * sockets or threads.
+ * driven exactly the way a ps-lite program drives them, without a scheduler or
+ * sockets.
  *
  * It keeps the names, argument meaning and failure behaviour of the interface in
  * dmlc/ps-lite (include/ps/kv_app.h, sarray.h, range.h, base.h): a program written
@@ -10,7 +10,10 @@
  * different is the inside: every worker request is sliced, handed straight to the
  * servers' request handles on the calling thread and answered before Push/Pull
  * returns, so requests are applied in program order (the reference's receive queue
- * does not promise that for equal priorities, threadsafe_pqueue.h:46-53).
+ * does not promise that for equal priorities, threadsafe_pqueue.h:46-53). Workers
+ * may run on threads of their own (tests/test_kv_app_multi_workers.cc:64-69 runs two
+ * in one process): a server then handles one request at a time, as its receive
+ * thread does (customer.cc:54-66), and a worker's requests stay in its program order.
  *
  * There is deliberately no default slicer and no default request handle here:
  * both must be installed (pskv::GpuSlicer / pskv::GpuKVHandle), so nothing in this
@@ -27,6 +30,7 @@
 #include <functional>
 #include <limits>
 #include <memory>
+#include <mutex>
 #include <sstream>
 #include <stdexcept>
 #include <string>
@@ -196,26 +200,32 @@ class Postoffice {
   }
   /* servers of one app register in creation order: the i-th created is server rank i */
   int AddServer(int app_id, void* server) {
+    std::lock_guard<std::mutex> lk(mu_);
     auto& v = servers_[app_id];
     v.push_back(server);
     return static_cast<int>(v.size()) - 1;
   }
   void RemoveServer(int app_id, void* server) {
+    std::lock_guard<std::mutex> lk(mu_);
     auto& v = servers_[app_id];
     v.erase(std::remove(v.begin(), v.end(), server), v.end());
   }
   void* server(int app_id, int rank) {
+    std::lock_guard<std::mutex> lk(mu_);
     auto it = servers_.find(app_id);
     if (it == servers_.end() || rank >= static_cast<int>(it->second.size())) return nullptr;
     return it->second[rank];
   }
   void AddWorker(int app_id, int customer_id, void* worker) {
+    std::lock_guard<std::mutex> lk(mu_);
     workers_[(static_cast<int64_t>(app_id) << 32) | static_cast<uint32_t>(customer_id)] = worker;
   }
   void RemoveWorker(int app_id, int customer_id) {
+    std::lock_guard<std::mutex> lk(mu_);
     workers_.erase((static_cast<int64_t>(app_id) << 32) | static_cast<uint32_t>(customer_id));
   }
   void* worker(int app_id, int customer_id) {
+    std::lock_guard<std::mutex> lk(mu_);
     auto it = workers_.find((static_cast<int64_t>(app_id) << 32) | static_cast<uint32_t>(customer_id));
     return it == workers_.end() ? nullptr : it->second;
   }
@@ -225,6 +235,7 @@ class Postoffice {
 
  private:
   Postoffice() {}
+  std::mutex mu_;  /* the two registries; workers may be created on threads of their own */
   int num_servers_ = 1;
   std::vector<Range> ranges_;
   std::unordered_map<int, std::vector<void*>> servers_;
@@ -252,6 +263,7 @@ class KVServer {
   void Process(const KVMeta& meta, const KVPairs<Val>& data) {
     if (data.lens.size()) PSKV_MIN_CHECK(data.lens.size() == data.keys.size(), "lens.size() == keys.size()");
     PSKV_MIN_CHECK(static_cast<bool>(request_handle_), "no request handle installed");
+    std::lock_guard<std::mutex> one_at_a_time(mu_);
     responses_ = 0;
     request_handle_(meta, data, this);
     /* a handle must answer exactly once, or the worker's Wait would hang (customer.cc:32-37) */
@@ -262,6 +274,7 @@ class KVServer {
 
  private:
   int app_id_, rank_ = 0, responses_ = 0;
+  std::mutex mu_;
   ReqHandle request_handle_;
 };
 

@@ -21,6 +21,8 @@ def test_kv_app_through_adapters(num_servers):
     print(r.stdout)
     assert r.returncode == 0, r.stdout
     assert "test_kv_app_gpu: ok" in r.stdout
+    # the two workers of tests/test_kv_app_multi_workers.cc ran, each on its own thread
+    assert "two workers, customer 0: error 0, 0" in r.stdout and "two workers, customer 1: error 0, 0" in r.stdout
 
 
 def test_dense_chunks_from_host_memory_through_adapters():

@@ -1,15 +1,18 @@
 // The reference's key-value integration test (tests/test_kv_app.cc) run against the GPU
 // slicer and the GPU request handle through the in-process ps:: surface: the same
 // worker program, the same closed forms, plus the multi-float layouts and the failure
-// cases of the data path.
+// cases of the data path, and the two-workers-in-one-process variant
+// (tests/test_kv_app_multi_workers.cc).
 //
 //   test_kv_app_gpu [num_servers [floats per key of the dense run from host memory]]
+#include <atomic>
 #include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <memory>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "pskv/ps_min.h"
@@ -17,7 +20,7 @@
 
 using namespace ps;
 
-static int g_failures = 0;
+static std::atomic<int> g_failures(0);
 #define EXPECT(cond)                                                        \
   do {                                                                      \
     if (!(cond)) {                                                          \
@@ -86,6 +89,55 @@ static void RunWorker(int app_id, int num, bool ones) {
   EXPECT(res == 0.0f && res2 == 0.0f);
   std::printf("kv_app num=%d error: %g, %g; %d pushes + 1 pull through slicer, handle and host staging: %.2f ms\n",
               num, res / repeat, res2 / (2 * repeat), repeat, push_pull_ms);
+}
+
+// tests/test_kv_app_multi_workers.cc:12-60: one of two workers of a process, each on a thread of
+// its own with its own customer id; the key sets interleave (keys offset by the customer id), so
+// every server sees requests of both workers in whatever order the threads get there, and every
+// GpuSlicer call may run next to the other worker's.
+static void RunOneOfTwoWorkers(int app_id, int customer_id) {
+  try {
+    KVWorker<float> kv(app_id, customer_id);
+    kv.set_slicer(pskv::GpuSlicer<float>(0));
+    const int num = 10000;
+    std::vector<Key> keys(num);
+    std::vector<float> vals(num);
+    unsigned seed = 7u + static_cast<unsigned>(customer_id);
+    for (int i = 0; i < num; ++i) {
+      keys[i] = kMaxKey / num * i + customer_id;
+      seed = seed * 1103515245u + 12345u;
+      vals[i] = static_cast<float>((seed >> 16) % 1000);
+    }
+    const int repeat = 50;
+    std::vector<int> ts;
+    for (int i = 0; i < repeat; ++i) {
+      ts.push_back(kv.Push(keys, vals));
+      if (i > 10) kv.Wait(ts[ts.size() - 10]);
+    }
+    for (int t : ts) kv.Wait(t);
+    std::vector<float> rets;
+    kv.Wait(kv.Pull(keys, &rets));
+    std::vector<float> outs;
+    for (int i = 0; i < repeat; ++i) kv.Wait(kv.PushPull(keys, vals, &outs));
+    float res = 0, res2 = 0;
+    for (int i = 0; i < num; ++i) {
+      res += std::fabs(rets[i] - vals[i] * repeat);
+      res2 += std::fabs(outs[i] - vals[i] * 2 * repeat);  // (the reference never adds to res2, :53-57)
+    }
+    EXPECT(rets.size() == static_cast<size_t>(num) && outs.size() == static_cast<size_t>(num));
+    EXPECT(res == 0.0f && res2 == 0.0f);
+    std::printf("kv_app two workers, customer %d: error %g, %g\n", customer_id, res / repeat, res2 / (2 * repeat));
+  } catch (const std::exception& e) {
+    std::fprintf(stderr, "worker %d: unexpected exception: %s\n", customer_id, e.what());
+    ++g_failures;
+  }
+}
+
+static void RunTwoWorkers(int app_id) {
+  std::thread t0(RunOneOfTwoWorkers, app_id, 0);
+  std::thread t1(RunOneOfTwoWorkers, app_id, 1);
+  t0.join();
+  t1.join();
 }
 
 // The example of kv_app.h:89-96: two keys with length-2 values.
@@ -266,6 +318,8 @@ int main(int argc, char** argv) {
     RunFixed();
     RunVarLen();
     RunFailures(num_servers);
+    auto s6 = StartServers(6, num_servers, PSKV_MODE_SCALAR);
+    RunTwoWorkers(6);
     if (argc > 2) {  // floats per key of the dense run from host memory (4194304 is the configuration's)
       auto s5 = StartServers(5, num_servers, PSKV_MODE_FIXED);
       RunDenseFromHost(static_cast<size_t>(std::atoll(argv[2])));
@@ -275,7 +329,7 @@ int main(int argc, char** argv) {
     return 2;
   }
   if (g_failures) {
-    std::fprintf(stderr, "%d expectation(s) failed\n", g_failures);
+    std::fprintf(stderr, "%d expectation(s) failed\n", g_failures.load());
     return 1;
   }
   std::printf("test_kv_app_gpu: ok (%d server%s)\n", num_servers, num_servers == 1 ? "" : "s");
