@@ -821,12 +821,83 @@ def cpu_sparse_repeat(orc, keys, vals, n, budget_s=20.0):
                       "them already, one thread" % (done, n)}
 
 
+# ------------------------------------------------------------------------------------
+# match: the ordered match of two sorted key sets (parallel_kv_match.h:29-120), worker side
+# ------------------------------------------------------------------------------------
+def run_match(args, capi, dev):
+    """A worker merges pulled values into its sorted local parameters: 16M destination keys, 12M source
+    keys of which 8M are among the destination's, one float per key, `dst[i] += src[j]` where the keys
+    are equal. A step is one pskv_match call (it returns when the destination is complete)."""
+    import torch
+    n_dst = args.keys or 16000000
+    n_src, shared = n_dst * 3 // 4, n_dst // 2
+    rng = np.random.default_rng(0xA7C4)
+    pool = unique_sorted_keys(rng, n_dst + n_src - shared, KMAX)
+    perm = rng.permutation(pool.size)
+    src_keys = np.sort(pool[perm[:n_src]])
+    dst_keys = np.sort(pool[perm[n_src - shared:]])
+    src_vals = rng.integers(-8, 8, size=n_src).astype(np.float32)
+    dst_vals = rng.integers(-8, 8, size=n_dst).astype(np.float32)
+    d_sk, d_sv, d_dk, d_dv = (to_dev(x, dev) for x in (src_keys, src_vals, dst_keys, dst_vals))
+    torch.cuda.synchronize()
+    ms = np.zeros(2, np.float32)
+    for _ in range(args.warmup):
+        capi.match(d_sk, d_sv, d_dk, d_dv, 1, capi.OP_PLUS)
+    samples = []
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        if sampled(i, args.steps):
+            matched = capi.match(d_sk, d_sv, d_dk, d_dv, 1, capi.OP_PLUS, kernel_ms=ms)
+            samples.append(float(ms[0]))
+        else:
+            matched = capi.match(d_sk, d_sv, d_dk, d_dv, 1, capi.OP_PLUS)
+    dt = time.perf_counter() - t0
+    assert matched == shared, (matched, shared)
+    # closed form: every shared key holds its value plus (warm-up + timed steps) times the source's
+    # (small integers: exact), every other key its own value
+    j = np.searchsorted(src_keys, dst_keys)
+    hit = (j < n_src) & (src_keys[np.minimum(j, n_src - 1)] == dst_keys)
+    want = dst_vals.copy()
+    want[hit] += np.float32(args.warmup + args.steps) * src_vals[j[hit]]
+    assert np.array_equal(d_dv.cpu().numpy().view(np.uint32), want.view(np.uint32)), "merged values differ"
+    # both key sets once, and per matched key the source value in, the destination value in and out
+    alg = 8.0 * (n_src + n_dst) + 12.0 * shared
+    samples = np.array(samples, np.float32)
+    res = {
+        "metric": "source + destination keys/sec of the ordered match and achieved GB/s (% of HBM peak) on 1 MI355X",
+        "value": (n_src + n_dst) * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
+        "dtype": "f32",
+        "config": {"workload": "match: sorted source keys (12M) merged into sorted destination keys (16M, 8M "
+                               "shared), dst[i] += src[j] where the keys are equal, one float per key",
+                   "dst_keys": n_dst, "src_keys": n_src, "shared_keys": shared, "value_len": 1,
+                   "key_dtype": "u64"},
+        "roofline": dict(roofline(alg, len(samples), float(samples.sum()), traffic("match_keys", n_src + n_dst),
+                                  samples),
+                         kernel="k_match_keys<k = 1> (stretch of source keys through LDS, values combined)",
+                         bytes_per_key=round(alg / (n_src + n_dst), 2)),
+    }
+    return res, (src_keys, src_vals, dst_keys, dst_vals)
+
+
+def cpu_match(orc, src_keys, src_vals, dst_keys, dst_vals, budget_s=15.0):
+    done = 0
+    dv = dst_vals
+    t0 = time.perf_counter()
+    while done < 1 or time.perf_counter() - t0 < budget_s:
+        _, dv, _ = orc.ordered_match(src_keys, src_vals, dst_keys, dv, 1, orc.OP_PLUS)
+        done += 1
+    dt = time.perf_counter() - t0
+    return {"value": (src_keys.size + dst_keys.size) * done / dt, "unit": "keys/s", "cores": 1, "kind": "port",
+            "sample": "%d calls of the reference's two-pointer loop on the same key sets, one thread (the "
+                      "binding copies the destination values once per call)" % done}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="sparse_lr", choices=["sparse_lr", "dense", "varlen", "zipf", "sparse_repeat"])
+    ap.add_argument("--workload", default="sparse_lr", choices=["sparse_lr", "dense", "varlen", "zipf", "sparse_repeat", "match"])
     ap.add_argument("--keys", type=int, default=0, help="keys per step (default: the config's)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the dense-chunk side measurement")
@@ -858,6 +929,8 @@ def main():
         res, zipf_batches, zipf_n = run_zipf(args, capi, dev)
     elif args.workload == "sparse_repeat":
         res, repeat_inputs = run_sparse_repeat(args, capi, dev)
+    elif args.workload == "match":
+        res, match_inputs = run_match(args, capi, dev)
     else:
         res, varlen_inputs = run_varlen(args, capi, dev)
 
@@ -888,12 +961,14 @@ def main():
             cpu = cpu_zipf(orc, zipf_batches, zipf_n)
         elif args.workload == "sparse_repeat":
             cpu = cpu_sparse_repeat(orc, *repeat_inputs)
+        elif args.workload == "match":
+            cpu = cpu_match(orc, *match_inputs)
         else:
             cpu = cpu_varlen(orc, *varlen_inputs)
         cpu["host"] = host_info()
 
     line = {
-        "metric": "push+pull keys/sec and achieved GB/s (% of HBM peak) on 1 MI355X",
+        "metric": res.get("metric", "push+pull keys/sec and achieved GB/s (% of HBM peak) on 1 MI355X"),
         "value": res["value"], "unit": res["unit"], "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": res["ms_per_step"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": res["dtype"], "data": "synthetic",

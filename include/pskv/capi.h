@@ -216,6 +216,26 @@ int pskv_assemble_pull(int device, const uint64_t* req_keys, size_t n, size_t R,
                        const int32_t* const* resp_lens, float* out, size_t out_cap,
                        int32_t* out_lens, size_t* out_nvals, int memkind);
 
+/* Ordered match of two sorted key sets, ParallelOrderedMatch
+ * (include/ps/internal/parallel_kv_match.h:29-120; operators: assign_op.h:12-41):
+ *     if (dst_keys[i] == src_keys[j])  dst_vals[i*k .. i*k+k)  op=  src_vals[j*k .. j*k+k)
+ * for sorted unique keys (a key set that repeats a key is a caller error with an unspecified
+ * result, as the reference's "Keys must be unique and sorted", :79). Destination values without
+ * a matching source key are left as they are. *matched (may be NULL) = k times the number of
+ * matched keys: the reference counts values (:52). The bit operators of assign_op.h:20-22 are
+ * for integers only (:38) and give PSKV_EINVAL here. The call returns when dst_vals is complete;
+ * calls on one device take turns. kernel_ms (no counterpart in the reference) is NULL or room for
+ * two floats: the device time of this call's key kernel and of its row kernel (0 for k == 1,
+ * which needs none), read from events that the launches carry. */
+#define PSKV_OP_ASSIGN 0 /* a = b */
+#define PSKV_OP_PLUS 1   /* a += b */
+#define PSKV_OP_MINUS 2  /* a -= b */
+#define PSKV_OP_TIMES 3  /* a *= b */
+#define PSKV_OP_DIVIDE 4 /* a /= b (assign_op.h:17 says "a -= b"; the code divides, :34) */
+int pskv_match(int device, const uint64_t* src_keys, size_t n_src, const float* src_vals,
+               const uint64_t* dst_keys, size_t n_dst, float* dst_vals, size_t k, int op,
+               uint64_t* matched, float* kernel_ms, int memkind);
+
 /* Device-time accounting for roofline figures (no counterpart in the reference).
  * While enabled, every launch of the kernels listed above is bracketed by HIP
  * events on the table's stream. pskv_prof_read waits for the stream and returns

@@ -50,6 +50,8 @@ def load():
         lib.pskv_oracle_find_range.argtypes = [vp, sz, u64, u64, ctypes.POINTER(u64),
                                                ctypes.POINTER(u64)]
         lib.pskv_oracle_find_range.restype = None
+        lib.pskv_oracle_ordered_match.argtypes = [vp, sz, vp, vp, sz, vp, sz, ctypes.c_int,
+                                                  ctypes.POINTER(sz)]
         _lib = lib
     return _lib
 
@@ -246,3 +248,18 @@ def assemble_pull(req_keys, responses, want_lens=False):
                                           None if out_lens is None else _p(out_lens),
                                           ctypes.byref(got))
     return rc, out, out_lens
+
+
+OP_ASSIGN, OP_PLUS, OP_MINUS, OP_TIMES, OP_DIVIDE = range(5)
+
+
+def ordered_match(src_keys, src_vals, dst_keys, dst_vals, k=1, op=OP_ASSIGN):
+    """ParallelOrderedMatch: returns (status, new dst_vals, matched values)."""
+    sk, dk = _u64(src_keys), _u64(dst_keys)
+    sv = np.ascontiguousarray(src_vals, dtype=np.float32)
+    dv = np.array(dst_vals, dtype=np.float32, copy=True)
+    assert sv.size == sk.size * k and dv.size == dk.size * k
+    got = ctypes.c_size_t(0)
+    rc = load().pskv_oracle_ordered_match(_p(sk), sk.size, _p(sv), _p(dk), dk.size, _p(dv), k, op,
+                                          ctypes.byref(got))
+    return rc, dv, got.value

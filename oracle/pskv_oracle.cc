@@ -346,4 +346,47 @@ int pskv_oracle_assemble_pull(const uint64_t* req_keys, size_t n, size_t R,
   return PSKV_ORACLE_OK;
 }
 
+// include/ps/internal/parallel_kv_match.h:29-60 with the operators of assign_op.h:12-41. The
+// reference splits dst in halves over threads (:61-73); every half runs the loop below on its
+// own dst range against the whole of src, so the sequential loop gives the same result.
+int pskv_oracle_ordered_match(const uint64_t* src_keys, size_t n_src, const float* src_vals,
+                              const uint64_t* dst_keys, size_t n_dst, float* dst_vals, size_t k,
+                              int op, size_t* matched) {
+  if (matched) *matched = 0;
+  if (op < 0 || op > 4) return PSKV_ORACLE_EINVAL;  // assign_op.h:38: the bit operators are for integers
+  if (n_dst == 0 || n_src == 0) return PSKV_ORACLE_OK;  // :36
+  const uint64_t* src_end = src_keys + n_src;
+  const uint64_t* dst_end = dst_keys + n_dst;
+  const uint64_t* sk = std::lower_bound(src_keys, src_end, *dst_keys);  // :39
+  const float* sv = src_vals + (sk - src_keys) * k;                     // :40
+  const uint64_t* dk = dst_keys;
+  float* dv = dst_vals;
+  size_t n = 0;
+  while (dk != dst_end && sk != src_end) {  // :43-58
+    if (*sk < *dk) {
+      ++sk;
+      sv += k;
+    } else {
+      if (!(*dk < *sk)) {
+        for (size_t i = 0; i < k; ++i) {
+          switch (op) {  // assign_op.h:26-36: right op= left
+            case 0: dv[i] = sv[i]; break;
+            case 1: dv[i] += sv[i]; break;
+            case 2: dv[i] -= sv[i]; break;
+            case 3: dv[i] *= sv[i]; break;
+            case 4: dv[i] /= sv[i]; break;
+          }
+        }
+        ++sk;
+        sv += k;
+        n += k;  // :52 counts values, not keys
+      }
+      ++dk;
+      dv += k;
+    }
+  }
+  if (matched) *matched = n;
+  return PSKV_ORACLE_OK;
+}
+
 }  // extern "C"

@@ -21,6 +21,9 @@
  *   pskv_oracle_handle fixed-k / var-len (extended)
  *                              k=1 equals scalar, numpy row sums, closed forms
  *   pskv_oracle_assemble_pull  numpy concatenation after argsort, FindRange doc example
+ *   pskv_oracle_ordered_match  (the reference's header does not compile, so there is no build
+ *                              of it to compare with) numpy searchsorted model, closed forms:
+ *                              equal key sets, disjoint key sets, one-sided subsets, k > 1
  */
 #ifndef PSKV_ORACLE_H_
 #define PSKV_ORACLE_H_
@@ -103,6 +106,14 @@ int pskv_oracle_assemble_pull(const uint64_t* req_keys, size_t n, size_t R,
 /* FindRange, include/ps/sarray.h:281-287: index range of keys within [lower, upper). */
 void pskv_oracle_find_range(const uint64_t* arr, size_t n, uint64_t lower, uint64_t upper,
                             uint64_t* begin, uint64_t* end);
+
+/* ParallelOrderedMatch, include/ps/internal/parallel_kv_match.h:29-120: for sorted unique keys,
+ * dst_vals[i*k .. i*k+k) op= src_vals[j*k .. j*k+k) wherever dst_keys[i] == src_keys[j]; other
+ * destination values stay. op: 0 ASSIGN, 1 PLUS, 2 MINUS, 3 TIMES, 4 DIVIDE (assign_op.h:12-21).
+ * *matched = k * matched keys (:52). */
+int pskv_oracle_ordered_match(const uint64_t* src_keys, size_t n_src, const float* src_vals,
+                              const uint64_t* dst_keys, size_t n_dst, float* dst_vals, size_t k,
+                              int op, size_t* matched);
 
 #ifdef __cplusplus
 }

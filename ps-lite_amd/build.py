@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 REPO = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libpskv.so")
-SOURCES = ["table.hip", "slice.hip", "hostmem.hip", "stager.hip", "meta_codec.cc"]
+SOURCES = ["table.hip", "slice.hip", "hostmem.hip", "stager.hip", "match.hip", "meta_codec.cc"]
 HEADERS = ["device_common.h", "host_common.h", "scan.h", "stager.h", "table_kernels.h"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -40,7 +40,7 @@ ERROR_NAMES = {
 SYMBOLS = [
     "pskv_table_create", "pskv_table_destroy", "pskv_push", "pskv_pull", "pskv_pushpull",
     "pskv_sync", "pskv_table_stream", "pskv_push_multi", "pskv_pull_multi", "pskv_sync_multi", "pskv_size", "pskv_dump", "pskv_slice", "pskv_slice_noalloc", "pskv_server_ranges",
-    "pskv_assemble_pull", "pskv_prof_enable", "pskv_prof_reset", "pskv_prof_read", "pskv_prof_samples",
+    "pskv_assemble_pull", "pskv_match", "pskv_prof_enable", "pskv_prof_reset", "pskv_prof_read", "pskv_prof_samples",
     "pskv_copy_probe", "pskv_host_alloc", "pskv_host_free", "pskv_host_trim", "pskv_last_error",
     "pskv_version",
 ]
@@ -97,6 +97,7 @@ def load():
     lib.pskv_server_ranges.argtypes = [u64, vp, vp]
     lib.pskv_assemble_pull.argtypes = [i32, vp, sz, sz, vp, vp, vp, vp, vp, vp, sz, vp,
                                        ctypes.POINTER(sz), i32]
+    lib.pskv_match.argtypes = [i32, vp, sz, vp, vp, sz, vp, sz, i32, ctypes.POINTER(u64), vp, i32]
     lib.pskv_prof_enable.argtypes = [vp, i32]
     lib.pskv_prof_reset.argtypes = [vp]
     lib.pskv_prof_read.argtypes = [vp, i32, ctypes.POINTER(u64), ctypes.POINTER(ctypes.c_double)]
@@ -394,6 +395,28 @@ def assemble_pull(req_keys, responses, out, out_lens=None, device=0):
     _check(load().pskv_assemble_pull(device, kp, n, R, kptr, nk, vptr, nv,
                                      lptr if have_lens else None, op, cap, olp, ctypes.byref(got),
                                      MEM_DEVICE))
+    return got.value
+
+
+OP_ASSIGN, OP_PLUS, OP_MINUS, OP_TIMES, OP_DIVIDE = range(5)
+
+
+def match(src_keys, src_vals, dst_keys, dst_vals, k=1, op=OP_ASSIGN, device=0, kernel_ms=None):
+    """ParallelOrderedMatch (parallel_kv_match.h:29-120) on the GPU: dst_vals[i] op= src_vals[j] wherever
+    dst_keys[i] == src_keys[j], in place. numpy arrays (host memory) or torch tensors on the device.
+    Returns the number of matched VALUES (k per matched key). kernel_ms: None, or a float32 numpy array of
+    two entries that receives the device time of the call's key kernel and row kernel."""
+    skp, ns, m1 = _buf(src_keys, np.uint64, "int64")
+    svp, nsv, m2 = _buf(src_vals, np.float32, "float32")
+    dkp, nd, m3 = _buf(dst_keys, np.uint64, "int64")
+    dvp, ndv, m4 = _buf(dst_vals, np.float32, "float32")
+    assert nsv == ns * k and ndv == nd * k, "k values per key on both sides"
+    if not _is_tensor(dst_vals):
+        assert isinstance(dst_vals, np.ndarray) and dst_vals.dtype == np.float32 and \
+            dst_vals.flags.c_contiguous, "dst_vals is changed in place"
+    got = ctypes.c_uint64(0)
+    _check(load().pskv_match(device, skp, ns, svp, dkp, nd, dvp, k, op, ctypes.byref(got),
+                             None if kernel_ms is None else kernel_ms.ctypes.data, _memkind(m1, m2, m3, m4)))
     return got.value
 
 
