@@ -36,11 +36,11 @@ sys.path.insert(0, REPO)
 import __graft_entry__ as graft  # noqa: E402
 
 KMAX = (1 << 64) - 1
-HBM_PEAK_GBS = 8000.0
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # Launches that carry their own start/stop events cost host time (about 15 us each) and a
 # few microseconds on the GPU, so the timed steps are sampled: every SAMPLE_EVERY-th step
 # times its launches (for the many-table workloads: those of one table, taken in turn).
-SAMPLE_EVERY = 4  # MI355X HBM3E, published
+SAMPLE_EVERY = 4  # (--sample-every)
 
 # HBM bytes per launch (read + written) of the dominant kernels come from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs of this very script (a counter run cannot be nested in a timing
@@ -893,6 +893,7 @@ def cpu_match(orc, src_keys, src_vals, dst_keys, dst_vals, budget_s=15.0):
 
 
 def main():
+    global SAMPLE_EVERY
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
@@ -901,6 +902,8 @@ def main():
     ap.add_argument("--keys", type=int, default=0, help="keys per step (default: the config's)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the dense-chunk side measurement")
+    ap.add_argument("--sample-every", type=int, default=SAMPLE_EVERY,
+                    help="every how many timed steps the launches carry events of their own")
     ap.add_argument("--per-table", action="store_true",
                     help="sparse_lr / varlen: serve the key ranges with one pskv_push / pskv_pull per table "
                          "instead of one pskv_push_multi / pskv_pull_multi over all of them")
@@ -908,6 +911,7 @@ def main():
                     help="sparse_lr / varlen: also time the steps with one stream per table "
                          "(reported under extra.own_streams; kernels of different ranges overlap)")
     args = ap.parse_args()
+    SAMPLE_EVERY = max(1, args.sample_every)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures ONE GPU: a table lives on one device and nothing here uses a "
               "second one; run it with --gpus 1", file=sys.stderr)
