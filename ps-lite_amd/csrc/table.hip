@@ -113,6 +113,7 @@ struct pskv_table {
   float max_load = 0.5f;
 
   Slot* slots = nullptr;
+  bool slots_pooled = false, arena_pooled = false;  // taken from the stream-ordered pool by a growth
   uint64_t cap = 0;        // slots, a power of two
   uint64_t count = 0;      // key count at the last read_state()
 
@@ -310,8 +311,46 @@ int report_device_errors(pskv_table* t) {
   return set_error(PSKV_ELEN_CHANGED, "a pushed row length differs from the stored length");
 }
 
-int alloc_slots(uint64_t cap, Slot** out, hipStream_t stream) {
-  PSKV_HIP(hipMalloc(reinterpret_cast<void**>(out), cap * sizeof(Slot)));
+// Slot arrays and arenas come from, and go back to, the device's stream-ordered pool where the
+// runtime has one: a growth releases the old array behind the kernel that empties it, without a
+// wait on the host (a plain hipFree of a few hundred MB blocks the host for ~350 us, longer than the
+// re-insertion itself). `pooled` says how the array must be released later.
+int alloc_for_growth(void** out, size_t bytes, hipStream_t stream, bool* pooled) {
+  static const bool have_pool = [] {
+    int dev = 0, ok = 0;
+    if (std::getenv("PSKV_NO_ASYNC_ALLOC")) return false;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    if (hipDeviceGetAttribute(&ok, hipDeviceAttributeMemoryPoolsSupported, dev) != hipSuccess) ok = 0;
+    (void)hipGetLastError();
+    return ok != 0;
+  }();
+  if (have_pool) {
+    if (hipMallocAsync(out, bytes, stream) == hipSuccess) {
+      *pooled = true;
+      return PSKV_OK;
+    }
+    (void)hipGetLastError();
+  }
+  *pooled = false;
+  PSKV_HIP(hipMalloc(out, bytes));
+  return PSKV_OK;
+}
+
+// Releases an array that kernels already enqueued on `stream` may still use.
+int release_after(void* ptr, bool pooled, hipStream_t stream) {
+  if (!ptr) return PSKV_OK;
+  if (pooled) {
+    PSKV_HIP(hipFreeAsync(ptr, stream));
+    return PSKV_OK;
+  }
+  PSKV_HIP(hipStreamSynchronize(stream));
+  PSKV_HIP(hipFree(ptr));
+  return PSKV_OK;
+}
+
+int alloc_slots(uint64_t cap, Slot** out, hipStream_t stream, bool* pooled) {
+  int rc = alloc_for_growth(reinterpret_cast<void**>(out), cap * sizeof(Slot), stream, pooled);
+  if (rc) return rc;
   // all-ones bytes: key = empty marker
   PSKV_HIP(hipMemsetAsync(*out, 0xFF, cap * sizeof(Slot), stream));
   return PSKV_OK;
@@ -368,32 +407,35 @@ int grow_slots(pskv_table* t, uint64_t keys_needed) {
     if (rc) return rc;
     t->cache_valid = false;
   }
-  rc = alloc_slots(want, &fresh, t->stream);
+  bool pooled = false;
+  rc = alloc_slots(want, &fresh, t->stream, &pooled);
   if (rc) return rc;
   launch(t, PSKV_KERNEL_REHASH, k_rehash, dim3(grid_for(t->cap, kBlock, kMaxGrid)), dim3(kBlock),
          (const Slot*)t->slots, t->cap, fresh, want - 1, t->st);
   PSKV_HIP(hipGetLastError());
-  PSKV_HIP(hipStreamSynchronize(t->stream));
-  PSKV_HIP(hipFree(t->slots));
+  rc = release_after(t->slots, t->slots_pooled, t->stream);
   t->slots = fresh;
+  t->slots_pooled = pooled;
   t->cap = want;
-  return PSKV_OK;
+  return rc;
 }
 
 int grow_arena(pskv_table* t, uint64_t floats_needed, uint64_t live_floats) {
   uint64_t want = std::max(floats_needed, t->arena_cap + t->arena_cap / 2);
   want = (want + 1023) & ~(uint64_t)1023;
   float* fresh = nullptr;
-  PSKV_HIP(hipMalloc(reinterpret_cast<void**>(&fresh), want * sizeof(float)));
+  bool pooled = false;
+  int rc = alloc_for_growth(reinterpret_cast<void**>(&fresh), want * sizeof(float), t->stream, &pooled);
+  if (rc) return rc;
   if (live_floats && t->arena) {
     PSKV_HIP(hipMemcpyAsync(fresh, t->arena, live_floats * sizeof(float), hipMemcpyDeviceToDevice,
                             t->stream));
   }
-  PSKV_HIP(hipStreamSynchronize(t->stream));
-  if (t->arena) PSKV_HIP(hipFree(t->arena));
+  rc = release_after(t->arena, t->arena_pooled, t->stream);
   t->arena = fresh;
+  t->arena_pooled = pooled;
   t->arena_cap = want;
-  return PSKV_OK;
+  return rc;
 }
 
 // Begins a request that may create up to `n` keys and take up to `units` allocation units
@@ -1492,7 +1534,7 @@ int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
   }
   const uint64_t keys = opts->initial_capacity ? opts->initial_capacity : kDefaultCapacity;
   t->cap = std::max(kMinSlots, next_pow2((uint64_t)((double)keys / t->max_load) + 1));
-  int rc = alloc_slots(t->cap, &t->slots, t->stream);
+  int rc = alloc_slots(t->cap, &t->slots, t->stream, &t->slots_pooled);
   if (rc) return fail(rc);
   if (hipMalloc(reinterpret_cast<void**>(&t->st), sizeof(DevState)) != hipSuccess ||
       hipMemsetAsync(t->st, 0, sizeof(DevState), t->stream) != hipSuccess ||
@@ -1512,7 +1554,8 @@ int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
   *t->outcome = 0ull;
   if (t->mode != PSKV_MODE_SCALAR && opts->arena_floats) {
     t->arena_cap = (opts->arena_floats + 1023) & ~(uint64_t)1023;
-    if (hipMalloc(reinterpret_cast<void**>(&t->arena), t->arena_cap * sizeof(float)) != hipSuccess)
+    if (alloc_for_growth(reinterpret_cast<void**>(&t->arena), t->arena_cap * sizeof(float), t->stream,
+                         &t->arena_pooled) != PSKV_OK)
       return fail(set_error(PSKV_ENOMEM, "cannot allocate %llu floats of row storage",
                             (unsigned long long)t->arena_cap));
   }
@@ -1535,7 +1578,17 @@ int pskv_table_destroy(pskv_table* t) {
     (void)hipEventDestroy(ev.a);
     (void)hipEventDestroy(ev.b);
   }
-  if (t->slots) (void)hipFree(t->slots);
+  // (arrays that a growth took from the stream-ordered pool go back to it)
+  if (t->slots && t->slots_pooled) {
+    (void)hipFreeAsync(t->slots, t->stream);
+  } else if (t->slots) {
+    (void)hipFree(t->slots);
+  }
+  if (t->arena && t->arena_pooled) {
+    (void)hipFreeAsync(t->arena, t->stream);
+    t->arena = nullptr;
+  }
+  if (t->slots_pooled || t->arena_pooled) (void)hipStreamSynchronize(t->stream);
   if (t->st) (void)hipFree(t->st);
   if (t->st_host) (void)hipHostFree(t->st_host);
   if (t->snap) (void)hipHostFree(t->snap);
