@@ -316,14 +316,23 @@ int report_device_errors(pskv_table* t) {
 // wait on the host (a plain hipFree of a few hundred MB blocks the host for ~350 us, longer than the
 // re-insertion itself). `pooled` says how the array must be released later.
 int alloc_for_growth(void** out, size_t bytes, hipStream_t stream, bool* pooled) {
-  static const bool have_pool = [] {
-    int dev = 0, ok = 0;
-    if (std::getenv("PSKV_NO_ASYNC_ALLOC")) return false;
-    if (hipGetDevice(&dev) != hipSuccess) return false;
-    if (hipDeviceGetAttribute(&ok, hipDeviceAttributeMemoryPoolsSupported, dev) != hipSuccess) ok = 0;
-    (void)hipGetLastError();
-    return ok != 0;
-  }();
+  // asked once per device (0 = not asked yet, 1 = no pool, 2 = pool)
+  static std::atomic<int> known[64];
+  int dev = 0;
+  bool have_pool = false;
+  if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
+    int k = known[dev].load(std::memory_order_relaxed);
+    if (k == 0) {
+      int ok = 0;
+      if (std::getenv("PSKV_NO_ASYNC_ALLOC") ||
+          hipDeviceGetAttribute(&ok, hipDeviceAttributeMemoryPoolsSupported, dev) != hipSuccess)
+        ok = 0;
+      (void)hipGetLastError();
+      k = ok ? 2 : 1;
+      known[dev].store(k, std::memory_order_relaxed);
+    }
+    have_pool = k == 2;
+  }
   if (have_pool) {
     if (hipMallocAsync(out, bytes, stream) == hipSuccess) {
       *pooled = true;
