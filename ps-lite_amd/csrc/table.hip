@@ -141,6 +141,10 @@ struct pskv_table {
   GrowBuf tiles_aff;  // VARLEN: one TileNote per tile
   char* small_in = nullptr;   // pinned, kSmallBytes: small host-resident requests, read in place
   char* small_out = nullptr;  // pinned, kSmallBytes: their responses, written in place
+  // A small host-resident SCALAR push returns once its kernel is queued: nothing comes back from
+  // it, and the next request that writes small_in waits for this event first.
+  hipEvent_t small_done = nullptr;
+  bool small_pending = false;
   GrowBuf stage;      // device copies of host-resident request buffers
   GrowBuf stage_out;  // device-side response of a host-resident or undersized pull
   bool no_growth = false;  // set while dumping: every key is known to be present
@@ -1274,7 +1278,11 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
     int32_t* dlens = c.take<int32_t>(want_lens ? n : 0);
     int32_t* dout_lens = nullptr;
     if (small) {
-      // every host-resident request ends with a wait, so the previous one is done with the buffers
+      // the previous request is done with the buffers: it ended with a wait, or left an event
+      if (t->small_pending) {
+        PSKV_HIP(hipEventSynchronize(t->small_done));
+        t->small_pending = false;
+      }
       if (n) std::memcpy(dkeys, keys, n * 8);
       if (r.nvals) std::memcpy(dvals, vals, r.nvals * 4);
       if (want_lens && n) std::memcpy(dlens, lens, n * 4);
@@ -1374,7 +1382,12 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
     }
     if (pull && varlen && out_lens && n && !lens_pinned)
       PSKV_HIP(hipMemcpyAsync(out_lens, r.out_lens, n * 4, hipMemcpyDeviceToHost, t->stream));
-    if (t->mode == PSKV_MODE_SCALAR) {
+    if (t->mode == PSKV_MODE_SCALAR && small && !pull && t->small_done) {
+      // no device-detected errors in this mode and nothing to hand back: the caller's buffers have
+      // been copied, the kernel is queued, later requests follow it on the stream
+      PSKV_HIP(hipEventRecord(t->small_done, t->stream));
+      t->small_pending = true;
+    } else if (t->mode == PSKV_MODE_SCALAR) {
       // no device-detected errors in this mode: waiting for the stream is all that is left
       PSKV_HIP(hipStreamSynchronize(t->stream));
     } else {
@@ -1557,7 +1570,8 @@ int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
       hipHostMalloc(reinterpret_cast<void**>(&t->small_in), kSmallBytes, hipHostMallocCoherent) !=
           hipSuccess ||
       hipHostMalloc(reinterpret_cast<void**>(&t->small_out), kSmallBytes, hipHostMallocCoherent) !=
-          hipSuccess)
+          hipSuccess ||
+      hipEventCreateWithFlags(&t->small_done, hipEventDisableTiming) != hipSuccess)
     return fail(set_error(PSKV_ENOMEM, "cannot allocate table state"));
   std::memset(t->snap, 0xFF, sizeof(Snapshot));  // names no request
   *t->outcome = 0ull;
@@ -1604,6 +1618,7 @@ int pskv_table_destroy(pskv_table* t) {
   if (t->outcome) (void)hipHostFree(t->outcome);
   if (t->sc_vals.ptr) (void)hipFree(t->sc_vals.ptr);
   if (t->sc_slots.ptr) (void)hipFree(t->sc_slots.ptr);
+  if (t->small_done) (void)hipEventDestroy(t->small_done);
   if (t->small_in) (void)hipHostFree(t->small_in);
   if (t->small_out) (void)hipHostFree(t->small_out);
   if (t->arena) (void)hipFree(t->arena);
