@@ -339,7 +339,8 @@ extern "C" int pskv_match(int device, const uint64_t* src_keys, size_t n_src, co
   if (memkind != PSKV_MEM_DEVICE && memkind != PSKV_MEM_HOST) return set_error(PSKV_EINVAL, "bad memkind");
   if (n_src == 0 || n_dst == 0) return PSKV_OK;  // parallel_kv_match.h:36
   if (!src_keys || !src_vals || !dst_keys || !dst_vals) return set_error(PSKV_EINVAL, "null buffer");
-  if (k > (1ull << 31) || n_src > (1ull << 40) || n_dst > (1ull << 40))
+  if (k > (1ull << 31) || n_src > (1ull << 40) || n_dst > (1ull << 40) ||
+      (n_src > n_dst ? n_src : n_dst) > (1ull << 44) / k)  // (2^44 floats: no product below overflows)
     return set_error(PSKV_EINVAL, "sizes beyond what one call handles");
   DeviceGuard guard(device);
   if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", device);
