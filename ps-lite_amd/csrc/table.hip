@@ -621,12 +621,48 @@ int read_state_batch(Batch& bt) {
   return PSKV_OK;
 }
 
-// Numbers a request that takes part in the key cache and says whether the key cache has the right shape for it.
-ReqTag next_tag(pskv_table* t, const Request& r) {
+// What the device has reported about the comparisons of earlier requests with the cached keys
+// (a pinned word, read whenever the host gets here, never waited for): comparisons that keep
+// finding other keys switch the comparison off for 2, 4, ... 64 requests of that kind.
+void note_outcomes(pskv_table* t) {
+  const unsigned long long seen = *static_cast<volatile unsigned long long*>(t->outcome);
+  if (seen == t->sc_seen) return;
+  t->sc_seen = seen;
+  const unsigned long long e = seen >> 1;
+  if (e + pskv_table::kScKinds <= t->epoch) return;  // the note of its kind has been overwritten
+  pskv_table::ScTrack& tr = t->sc_track[t->sc_kind[e % pskv_table::kScKinds] & 1];
+  if (seen & 1ull) {
+    tr.fail = 0;
+    tr.hit = true;
+  } else {
+    tr.fail = std::min(tr.fail + 1u, 6u);
+    tr.skip = 1u << tr.fail;
+    tr.hit = false;
+  }
+}
+
+// Numbers a request that takes part in the key cache and says whether the key cache has the
+// right shape for it. Row modes (`back_off`): a request of the right shape is still not compared
+// while comparisons of its kind (pushes, pulls) are in a spell of finding other keys, as the
+// requests of an embedding table do that names other rows in every batch; the request then goes
+// the general way, which leaves its keys behind as the new cache all the same.
+ReqTag next_tag(pskv_table* t, const Request& r, bool back_off = false) {
   ReqTag tag;
   tag.epoch = ++t->epoch;
   tag.pad = 0;
-  tag.try_cache = (t->cache_valid && t->cache_n == r.n) ? 1u : 0u;
+  bool compare = t->cache_valid && t->cache_n == r.n;
+  if (back_off && compare) {
+    note_outcomes(t);
+    const int kind = r.push ? 0 : 1;
+    pskv_table::ScTrack& tr = t->sc_track[kind];
+    if (tr.skip) {
+      --tr.skip;
+      compare = false;
+    } else {
+      t->sc_kind[tag.epoch % pskv_table::kScKinds] = (unsigned char)kind;
+    }
+  }
+  tag.try_cache = compare ? 1u : 0u;
   return tag;
 }
 
@@ -653,22 +689,7 @@ bool scalar_cache_eligible(const pskv_table* t, const Request& r) {
 }
 
 ScalarCacheUse scalar_cache_use(pskv_table* t, const Request& r) {
-  const unsigned long long seen = *static_cast<volatile unsigned long long*>(t->outcome);
-  if (seen != t->sc_seen) {
-    t->sc_seen = seen;
-    const unsigned long long e = seen >> 1;
-    if (e + pskv_table::kScKinds > t->epoch) {  // (else the note of its kind has been overwritten)
-      pskv_table::ScTrack& tr = t->sc_track[t->sc_kind[e % pskv_table::kScKinds] & 1];
-      if (seen & 1ull) {
-        tr.fail = 0;
-        tr.hit = true;
-      } else {
-        tr.fail = std::min(tr.fail + 1u, 6u);
-        tr.skip = 1u << tr.fail;
-        tr.hit = false;
-      }
-    }
-  }
+  note_outcomes(t);
   const int kind = r.push ? 0 : 1;
   // a worker that pushes gradients and pulls the weights of the same keys right away shows as a
   // pull behind a push of its own size, whatever that size is from one step to the next
@@ -865,8 +886,9 @@ int launch_rows(Batch& bt, int op) {
 int begin_row_request(Batch& bt) {
   for (Item& it : bt) {
     if (!it.r.n) continue;
-    it.tag = next_tag(it.t, it.r);
+    it.tag = next_tag(it.t, it.r, true);
     it.d.tag = it.tag;
+    it.d.outcome = it.t->outcome;
   }
   return launch_batch(bt, PSKV_KERNEL_SAME_KEYS, k_same_keys, [](const Item& it) {
     return (it.r.n && it.tag.try_cache) ? (it.r.n + kBlock * kSameKeysItems - 1) / (kBlock * kSameKeysItems)
@@ -1036,8 +1058,9 @@ int run_varlen(Batch& bt, bool push, bool pull) {
       int rc = reserve(t, r.n, r.nvals / 4 + r.n + kArenaPadUnits * it.nparts, 4, &it.pub);
       if (rc) return rc;
       if (t->cache_nvals != r.nvals) t->cache_valid = false;  // same lens would mean the same total
-      it.tag = next_tag(t, r);
+      it.tag = next_tag(t, r, true);
       TableReq& d = it.d;
+      d.outcome = t->outcome;
       d.slots = t->slots;
       d.mask = t->cap - 1;
       d.arena = t->arena;

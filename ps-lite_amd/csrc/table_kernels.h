@@ -291,8 +291,9 @@ __device__ __forceinline__ void decide_same(DevState* st, const ReqTag& tag, boo
   } else {
     st->cache_epoch = tag.epoch;
   }
-  // the host reads this when it gets to it (never waits for it): epoch << 1 | same
-  if (outcome) *outcome = (tag.epoch << 1) | (same ? 1ull : 0ull);
+  // the host reads this when it gets to it (never waits for it): epoch << 1 | same; only a
+  // request that was in fact compared reports
+  if (outcome && tag.try_cache) *outcome = (tag.epoch << 1) | (same ? 1ull : 0ull);
 }
 
 // Compares the keys of a request with the cached ones and reaches the decision for the whole
@@ -515,7 +516,7 @@ __global__ __launch_bounds__(kBlock) void k_var_push_begin(ReqBatch b) {
   }
   if (!scan_pass1_block(s, flags, part, st, nblk, red, fred, &s_last)) return;
   flags = scan_pass1_last(part, st, nblk, tag.epoch, red, &carry_s);
-  if (threadIdx.x == 0) decide_same(st, tag, (flags & kReqDiffer) != 0u);
+  if (threadIdx.x == 0) decide_same(st, tag, (flags & kReqDiffer) != 0u, d.outcome);
 }
 
 // VARLEN push, second kernel: pass 2 of the lens scan (request-side offsets and the tile
