@@ -822,6 +822,107 @@ def cpu_sparse_repeat(orc, keys, vals, n, budget_s=20.0):
 
 
 # ------------------------------------------------------------------------------------
+# embed: rows of an embedding table, other rows in every batch (fixed-length values, kv_app.h:17-22)
+# ------------------------------------------------------------------------------------
+def run_embed(args, capi, dev):
+    """One FIXED table of 8M rows of 64 floats. A step is what a worker does per batch: pull the rows of
+    1M keys (another random subset every step), then push a gradient for the same keys. The pull has to
+    look its keys up (its comparison with the cached keys would fail, and is soon skipped); the push
+    repeats the pull's keys and reuses their row references."""
+    import torch
+    n, rows, k = args.keys or 1000000, 8000000, 64
+    rng = np.random.default_rng(0xE3BED)
+    all_keys = unique_sorted_keys(rng, rows, KMAX)
+    t = capi.Table(capi.MODE_FIXED, initial_capacity=2 * rows, row_len=k, arena_floats=rows * k + (1 << 20))
+    init = torch.ones(rows // 8 * k, dtype=torch.float32, device=dev)
+    for c in range(8):  # fill the table: row i starts as all ones
+        t.push(to_dev(np.ascontiguousarray(all_keys[c * (rows // 8):(c + 1) * (rows // 8)]), dev), init)
+    t.sync()
+    del init
+    total = args.warmup + args.steps
+    batches = []
+    for s_ in range(total):
+        keys = np.sort(rng.choice(all_keys, size=n, replace=False))
+        batches.append(keys)
+    d_keys = [to_dev(kk, dev) for kk in batches]
+    grad = to_dev(rng.integers(-4, 4, size=n * k).astype(np.float32), dev)  # the same gradient values every step
+    out = torch.empty(n * k, dtype=torch.float32, device=dev)
+    torch.cuda.synchronize()
+
+    def step(i):
+        kp = d_keys[i].data_ptr()
+        t.pull_raw(kp, n, out.data_ptr(), n * k)
+        t.push_raw(kp, n, grad.data_ptr(), n * k)
+
+    for i in range(args.warmup):
+        step(i)
+    t.sync()
+    t.prof_reset()
+    t0 = time.perf_counter()
+    for i in range(args.warmup, total):
+        t.prof_enable(sampled(i - args.warmup, args.steps))
+        step(i)
+    t.sync()
+    dt = time.perf_counter() - t0
+    t.prof_enable(False)
+    acc = kernel_stats([t], capi.KERNEL_ROWS_ACC)
+    gat = kernel_stats([t], capi.KERNEL_ROWS_GATHER)
+    look = kernel_stats([t], capi.KERNEL_LOOKUP)
+    # the last pull answered the rows as they were before the last push: ones plus, for every
+    # earlier step that named the row, the gradient at the row's place in that step's batch
+    # (small integers: exact)
+    sample = rng.choice(n, size=2048, replace=False)
+    g = grad.cpu().numpy().reshape(n, k)
+    keys_s = batches[-1][sample]
+    want = np.ones((sample.size, k), np.float32)
+    for kk in batches[:-1]:
+        at = np.minimum(np.searchsorted(kk, keys_s), n - 1)
+        hit = kk[at] == keys_s
+        want[hit] += g[at[hit]]
+    got = out.cpu().numpy().reshape(n, k)[sample]
+    assert np.array_equal(got, want.astype(np.float32)), "pulled rows differ"
+    assert t.size()[0] == rows
+    res = {
+        "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
+        "dtype": "f32",
+        "config": {"workload": "embed: one table of 8M rows of 64 floats; a step pulls the rows of 1M keys "
+                               "(another random subset every step) and pushes a gradient for the same keys",
+                   "keys_per_step": n, "ranges": 1, "value_len": k, "key_dtype": "u64",
+                   "store_keys_after_timed_steps": rows},
+        "gbps": (12.0 + 8.0) * n * k * args.steps / dt / 1e9,
+        # gradient in, row in, row out: 12 B/float, the rows scattered over the arena
+        "roofline": dict(roofline(12.0 * n * k, acc[0], acc[1], traffic("rows_acc_embed", n * k), acc[2]),
+                         kernel="k_rows<acc,fixed> (row += in, rows scattered)", bytes_per_float=12),
+        "kernels": {"rows_gather": dict(roofline(8.0 * n * k, gat[0], gat[1],
+                                                 traffic("rows_gather_embed", n * k), gat[2]),
+                                        bytes_per_float=8),
+                    "lookup": dict(roofline(24.0 * n, look[0], look[1], traffic("lookup_embed", n), look[2]),
+                                   kernel="k_lookup_fixed (key -> row, the pull's; the push reuses it)",
+                                   bytes_per_key=24)},
+    }
+    return res, (all_keys, batches[args.warmup:], g.reshape(-1), n, rows, k)
+
+
+def cpu_embed(orc, all_keys, batches, grad, n, rows, k, budget_s=20.0):
+    store = orc.Store(orc.MODE_FIXED)
+    ones = np.ones(rows // 8 * k, np.float32)
+    for c in range(8):
+        store.push(all_keys[c * (rows // 8):(c + 1) * (rows // 8)], ones)
+    done = 0
+    t0 = time.perf_counter()
+    for keys in batches:
+        store.handle(False, True, keys, out_cap=n * k)
+        store.push(keys, grad)
+        done += 1
+        if time.perf_counter() - t0 > budget_s:
+            break
+    dt = time.perf_counter() - t0
+    return {"value": 2.0 * n * done / dt, "unit": "keys/s", "cores": 1, "kind": "port",
+            "sample": "first %d of the timed steps (pull + push of %d rows of %d floats) on a "
+                      "std::unordered_map of rows that holds the %d keys already, one thread" % (done, n, k, rows)}
+
+
+# ------------------------------------------------------------------------------------
 # match: the ordered match of two sorted key sets (parallel_kv_match.h:29-120), worker side
 # ------------------------------------------------------------------------------------
 def run_match(args, capi, dev):
@@ -898,7 +999,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="sparse_lr", choices=["sparse_lr", "dense", "varlen", "zipf", "sparse_repeat", "match"])
+    ap.add_argument("--workload", default="sparse_lr", choices=["sparse_lr", "dense", "varlen", "zipf", "sparse_repeat", "embed", "match"])
     ap.add_argument("--keys", type=int, default=0, help="keys per step (default: the config's)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the dense-chunk side measurement")
@@ -935,6 +1036,8 @@ def main():
         res, repeat_inputs = run_sparse_repeat(args, capi, dev)
     elif args.workload == "match":
         res, match_inputs = run_match(args, capi, dev)
+    elif args.workload == "embed":
+        res, embed_inputs = run_embed(args, capi, dev)
     else:
         res, varlen_inputs = run_varlen(args, capi, dev)
 
@@ -967,6 +1070,8 @@ def main():
             cpu = cpu_sparse_repeat(orc, *repeat_inputs)
         elif args.workload == "match":
             cpu = cpu_match(orc, *match_inputs)
+        elif args.workload == "embed":
+            cpu = cpu_embed(orc, *embed_inputs)
         else:
             cpu = cpu_varlen(orc, *varlen_inputs)
         cpu["host"] = host_info()
