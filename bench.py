@@ -836,9 +836,10 @@ def run_embed(args, capi, dev):
     t = capi.Table(capi.MODE_FIXED, initial_capacity=2 * rows, row_len=k, arena_floats=rows * k + (1 << 20))
     init = torch.ones(rows // 8 * k, dtype=torch.float32, device=dev)
     for c in range(8):  # fill the table: row i starts as all ones
-        t.push(to_dev(np.ascontiguousarray(all_keys[c * (rows // 8):(c + 1) * (rows // 8)]), dev), init)
-    t.sync()
-    del init
+        chunk = to_dev(np.ascontiguousarray(all_keys[c * (rows // 8):(c + 1) * (rows // 8)]), dev)
+        t.push(chunk, init)
+        t.sync()  # (the call is asynchronous: its buffers stay untouched until the table has used them)
+    del init, chunk
     total = args.warmup + args.steps
     batches = []
     for s_ in range(total):

@@ -149,7 +149,23 @@ def _memkind(*kinds):
     return kind
 
 
-class Table:
+class _Holder:
+    """Device-resident calls are asynchronous: the table reads and writes the caller's tensors after
+    the call has returned. The methods that take tensors therefore keep them referenced until the
+    next wait, so that a temporary (`t.push(to_dev(keys), ...)`) is not handed to someone else by
+    torch's allocator while a kernel is still to read it. The *_raw methods leave that to the caller."""
+
+    def _hold(self, *tensors):
+        held = self.__dict__.setdefault("_held", [])
+        held.extend(x for x in tensors if x is not None and _is_tensor(x) and x.is_cuda)
+        if len(held) > 4096:
+            self.sync()
+
+    def _release(self):
+        self.__dict__["_held"] = []
+
+
+class Table(_Holder):
     """The store behind a KVServer request handle (kv_app.h:440-463)."""
 
     def __init__(self, mode=MODE_SCALAR, device=0, initial_capacity=0, row_len=0, arena_floats=0,
@@ -165,6 +181,7 @@ class Table:
         if self._h:
             self._lib.pskv_table_destroy(self._h)
             self._h = ctypes.c_void_p()
+        self._release()
 
     def __del__(self):
         # Not while the interpreter shuts down: a stream that the caller lent (torch's, say) may be
@@ -180,6 +197,7 @@ class Table:
         kp, n, k1 = _buf(keys, np.uint64, "int64")
         vp, nv, k2 = _buf(vals, np.float32, "float32")
         lp, nl, k3 = _buf(lens, np.int32, "int32")
+        self._hold(keys, vals, lens)
         _check(self._lib.pskv_push(self._h, kp, n, vp, nv, lp, nl, _memkind(k1, k2, k3)))
 
     def pull(self, keys, out, out_lens=None):
@@ -189,6 +207,7 @@ class Table:
         lp, _, k3 = _buf(out_lens, np.int32, "int32")
         got = ctypes.c_size_t(0)
         self.last_out_nvals = None
+        self._hold(keys, out, out_lens)
         rc = self._lib.pskv_pull(self._h, kp, n, op, cap, lp, ctypes.byref(got), _memkind(k1, k2, k3))
         self.last_out_nvals = got.value
         _check(rc)
@@ -201,6 +220,7 @@ class Table:
         op, cap, k4 = _buf(out, np.float32, "float32")
         olp, _, k5 = _buf(out_lens, np.int32, "int32")
         got = ctypes.c_size_t(0)
+        self._hold(keys, vals, lens, out, out_lens)
         rc = self._lib.pskv_pushpull(self._h, kp, n, vp, nv, lp, nl, op, cap, olp, ctypes.byref(got),
                                      _memkind(k1, k2, k3, k4, k5))
         self.last_out_nvals = got.value
@@ -216,7 +236,9 @@ class Table:
                                    MEM_DEVICE))
 
     def sync(self):
-        _check(self._lib.pskv_sync(self._h))
+        rc = self._lib.pskv_sync(self._h)
+        self._release()
+        _check(rc)
 
     def size(self):
         nk, nv = ctypes.c_uint64(0), ctypes.c_uint64(0)
@@ -260,7 +282,7 @@ class Table:
         _check(self._lib.pskv_copy_probe(self._h, dst.data_ptr(), src.data_ptr(), nbytes))
 
 
-class Group:
+class Group(_Holder):
     """Several tables of one process on one GPU that share a stream, so that one launch per
     pipeline step serves all key ranges of a sliced request (pskv_push_multi / pskv_pull_multi)."""
 
@@ -316,19 +338,23 @@ class Group:
 
     def push(self, keys, pos, vals, val_pos, lens=None):
         _memkind(MEM_DEVICE)
+        self._hold(keys, vals, lens)
         self.push_raw(keys.data_ptr() if keys.numel() else None, pos,
                       vals.data_ptr() if vals.numel() else None, val_pos,
                       None if lens is None else (lens.data_ptr() if lens.numel() else None))
 
     def pull(self, keys, pos, out, out_pos=None, out_lens=None, want_sizes=False):
         _memkind(MEM_DEVICE)
+        self._hold(keys, out, out_lens)
         return self.pull_raw(keys.data_ptr() if keys.numel() else None, pos,
                              out.data_ptr() if out.numel() else None, out_pos,
                              None if out_lens is None else (out_lens.data_ptr() if out_lens.numel() else None),
                              want_sizes)
 
     def sync(self):
-        _check(self._lib.pskv_sync_multi(self._arr, self.S))
+        rc = self._lib.pskv_sync_multi(self._arr, self.S)
+        self._release()
+        _check(rc)
 
     def size(self):
         nk = nv = 0

@@ -315,13 +315,11 @@ int report_device_errors(pskv_table* t) {
   return set_error(PSKV_ELEN_CHANGED, "a pushed row length differs from the stored length");
 }
 
-// With PSKV_ASYNC_ALLOC set in the environment, slot arrays and arenas come from, and go back to,
-// the device's stream-ordered pool: a growth then releases the old array behind the kernel that
-// empties it, without a wait on the host (a plain hipFree of a few hundred MB blocks the host
-// for 150-440 us, longer than the re-insertion itself). Off by default: with the pool in use, a
-// run under `rocprofv3 --pmc` (which serialises the kernels) gave wrong sums in a workload whose
-// arena grows several times, and right ones without the pool; the cause is not known, so the
-// default stays with hipMalloc and hipFree. `pooled` says how the array must be released later.
+// Slot arrays and arenas come from, and go back to, the device's stream-ordered pool where the
+// runtime has one (PSKV_NO_ASYNC_ALLOC in the environment goes back to hipMalloc / hipFree): a
+// growth releases the old array behind the kernel that empties it, without a wait on the host
+// (a plain hipFree of a few hundred MB blocks the host for 150-440 us, longer than the
+// re-insertion itself). `pooled` says how the array must be released later.
 int alloc_for_growth(void** out, size_t bytes, hipStream_t stream, bool* pooled) {
   // asked once per device (0 = not asked yet, 1 = no pool, 2 = pool)
   static std::atomic<int> known[64];
@@ -331,7 +329,7 @@ int alloc_for_growth(void** out, size_t bytes, hipStream_t stream, bool* pooled)
     int k = known[dev].load(std::memory_order_relaxed);
     if (k == 0) {
       int ok = 0;
-      if (!std::getenv("PSKV_ASYNC_ALLOC") ||
+      if (std::getenv("PSKV_NO_ASYNC_ALLOC") ||
           hipDeviceGetAttribute(&ok, hipDeviceAttributeMemoryPoolsSupported, dev) != hipSuccess)
         ok = 0;
       (void)hipGetLastError();
