@@ -1025,7 +1025,9 @@ def test_scalar_key_cache_at_its_real_size(capi, orc, dev, memkind):
             buf = torch.full((k.size + 8,), 7.0, dtype=torch.float32, device=dev)
             out = buf[shift:shift + k.size]
             torch.cuda.synchronize()
-            t.pull_raw(to_dev(k, dev).data_ptr(), k.size, out.data_ptr(), k.size)
+            dk = to_dev(k, dev)  # (kept until the wait: the call only enqueues)
+            torch.cuda.synchronize()
+            t.pull_raw(dk.data_ptr(), k.size, out.data_ptr(), k.size)
             t.sync()
             got = from_dev(out)
         else:
