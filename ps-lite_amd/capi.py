@@ -278,6 +278,8 @@ class Table(_Holder):
 
     def copy_probe(self, dst, src):
         assert dst.is_cuda and src.is_cuda
+        _memkind(MEM_DEVICE)  # (torch may still be filling the tensors on its own stream)
+        self._hold(dst, src)
         nbytes = src.numel() * src.element_size()
         _check(self._lib.pskv_copy_probe(self._h, dst.data_ptr(), src.data_ptr(), nbytes))
 
@@ -396,6 +398,7 @@ def slice_keys_noalloc(keys, range_begin, range_end, pos, val_pos, used, status,
     lp, nl, _ = _buf(lens, np.int32, "int32")
     rb = np.ascontiguousarray(range_begin, dtype=np.uint64)
     re = np.ascontiguousarray(range_end, dtype=np.uint64)
+    _memkind(MEM_DEVICE)  # (torch may still be filling the tensors on its own stream)
     _check(load().pskv_slice_noalloc(device, stream, kp, n, lp, nl, nvals, rb.ctypes.data,
                                      re.ctypes.data, rb.size, pos.data_ptr(), val_pos.data_ptr(),
                                      used.data_ptr(), status.data_ptr()))
@@ -418,6 +421,7 @@ def assemble_pull(req_keys, responses, out, out_lens=None, device=0):
     op, cap, _ = _buf(out, np.float32, "float32")
     olp, _, _ = _buf(out_lens, np.int32, "int32")
     got = ctypes.c_size_t(0)
+    _memkind(MEM_DEVICE)  # (torch may still be filling the tensors on its own stream)
     _check(load().pskv_assemble_pull(device, kp, n, R, kptr, nk, vptr, nv,
                                      lptr if have_lens else None, op, cap, olp, ctypes.byref(got),
                                      MEM_DEVICE))
