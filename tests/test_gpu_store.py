@@ -1171,3 +1171,52 @@ def test_pull_right_behind_a_push_compares_key_by_key(capi, orc, dev, memkind, s
     t.sync()
     _check_dump(t, o, "pull behind push")
     t.close()
+
+
+@pytest.mark.parametrize("mode", ["fixed", "varlen"])
+def test_other_rows_in_every_batch(capi, orc, dev, mode):
+    """An embedding table's requests: batches of one size that name other rows every time, each pulled and
+    then pushed by the worker. The pulls' comparisons with the cached keys keep failing and are skipped
+    for longer and longer spells, the pushes repeat their pull's keys; then the same batch comes several
+    times in a row (comparisons resume and hit), then other batches again. Every pull and the final store
+    against the oracle, requests queued without a wait in between."""
+    import torch
+    announce("other_rows_in_every_batch", mode)
+    rng = np.random.default_rng(31)
+    n, universe, k = 700, 5000, 8
+    all_keys = unique_keys(rng, universe)
+    lens_of = rng.choice([4, 8, 12, 40], size=universe).astype(np.int32)
+    m = capi.MODE_FIXED if mode == "fixed" else capi.MODE_VARLEN
+    t = capi.Table(m, initial_capacity=2 * universe, row_len=k if mode == "fixed" else 0)
+    o = orc.Store(orc.MODE_FIXED if mode == "fixed" else orc.MODE_VARLEN, k if mode == "fixed" else 0)
+    held, checks = [], []
+    for step in range(70):
+        if step in range(40, 46):
+            idx = np.arange(100, 100 + n)  # the same batch six times
+        else:
+            idx = np.sort(rng.choice(universe, size=n, replace=False))
+        keys = all_keys[idx]
+        lens = lens_of[idx] if mode == "varlen" else None
+        nvals = int(lens.sum()) if mode == "varlen" else n * k
+        grad = rng.integers(-8, 8, size=nvals).astype(np.float32)
+        dk, dg = to_dev(keys, dev), to_dev(grad, dev)
+        dl = to_dev(lens, dev) if mode == "varlen" else None
+        want, want_lens = o.pull(keys)
+        out = torch.full((max(nvals, 1),), 7.0, dtype=torch.float32, device=dev)
+        out_lens = torch.full((n,), -1, dtype=torch.int32, device=dev)
+        torch.cuda.synchronize()
+        t.pull_raw(dk.data_ptr(), n, out.data_ptr(), out.numel(), out_lens.data_ptr() if mode == "varlen" else None)
+        t.push_raw(dk.data_ptr(), n, dg.data_ptr(), nvals, dl.data_ptr() if mode == "varlen" else None,
+                   n if mode == "varlen" else 0)
+        o.push(keys, grad, lens)
+        held.append((dk, dg, dl))
+        checks.append((step, out, out_lens, want, want_lens))
+        if step % 9 == 8:  # now and then the worker waits
+            t.sync()
+    t.sync()
+    for step, out, out_lens, want, want_lens in checks:
+        assert_bits_equal(from_dev(out)[:want.size], want, "pull of step %d" % step)
+        if mode == "varlen":
+            assert np.array_equal(from_dev(out_lens), want_lens), "lens of step %d" % step
+    _check_dump(t, o, "other rows in every batch")
+    t.close()
