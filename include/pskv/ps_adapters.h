@@ -180,5 +180,31 @@ class GpuKVHandle {
   size_t last_response_ = 0;
 };
 
+/* ParallelOrderedMatch (include/ps/internal/parallel_kv_match.h:95-120) on the GPU, with the
+ * reference's parameter order: merges src_val into *dst_val where the sorted unique keys are
+ * equal, `dst_val[i] op= src_val[j]`, k values per key. *dst_val is resized to
+ * dst_key.size() * k first (new entries are zero, :109), as the reference does. `op` is one of
+ * PSKV_OP_ASSIGN .. PSKV_OP_DIVIDE, numbered like ps::AssignOp (assign_op.h:12-21); the
+ * reference's thread count has no meaning here. Returns the number of matched values. C is
+ * ps::SArray<Val> or std::vector<Val>. */
+template <typename Val, typename C>
+size_t GpuOrderedMatch(const ps::SArray<ps::Key>& src_key, const ps::SArray<Val>& src_val,
+                       const ps::SArray<ps::Key>& dst_key, C* dst_val, int k = 1, int op = PSKV_OP_ASSIGN,
+                       int device = 0) {
+  static_assert(sizeof(ps::Key) == 8 && sizeof(Val) == 4, "64-bit keys, float values");
+  if (k <= 0 || src_key.size() * static_cast<size_t>(k) != src_val.size())  // CHECK_EQ, :107
+    throw dmlc::Error("GpuOrderedMatch: Check failed: src_key.size() * k == src_val.size()");
+  dst_val->resize(dst_key.size() * static_cast<size_t>(k));  // :109
+  if (dst_key.empty()) return 0;
+  uint64_t matched = 0;
+  const int rc = pskv_match(device, reinterpret_cast<const uint64_t*>(src_key.data()), src_key.size(),
+                            reinterpret_cast<const float*>(src_val.data()),
+                            reinterpret_cast<const uint64_t*>(dst_key.data()), dst_key.size(),
+                            reinterpret_cast<float*>(dst_val->data()), static_cast<size_t>(k), op, &matched,
+                            nullptr, PSKV_MEM_HOST);
+  if (rc != PSKV_OK) ThrowStatus(rc, "GpuOrderedMatch");
+  return static_cast<size_t>(matched);
+}
+
 }  // namespace pskv
 #endif  // PSKV_PS_ADAPTERS_H_

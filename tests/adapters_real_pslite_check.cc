@@ -21,3 +21,10 @@ void install(ps::KVWorker<float>* w, ps::KVServer<float>* s) {
   w->set_slicer(pskv::GpuSlicer<float>(0));
   s->set_request_handle(pskv::GpuKVHandle<float>());
 }
+
+// the ordered match with the reference's containers on both ends (parallel_kv_match.h:95-100)
+size_t merge(const ps::SArray<ps::Key>& src_key, const ps::SArray<float>& src_val,
+             const ps::SArray<ps::Key>& dst_key, ps::SArray<float>* into_sarray, std::vector<float>* into_vector) {
+  return pskv::GpuOrderedMatch(src_key, src_val, dst_key, into_sarray, 2, PSKV_OP_PLUS) +
+         pskv::GpuOrderedMatch(src_key, src_val, dst_key, into_vector);
+}

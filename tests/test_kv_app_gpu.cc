@@ -133,6 +133,45 @@ static void RunOneOfTwoWorkers(int app_id, int customer_id) {
   }
 }
 
+// The merge a worker does with what it pulled (parallel_kv_match.h:76-94): values of the keys
+// that both sides hold are combined, the others stay; a destination that is too short grows
+// with zeros first.
+static void RunOrderedMatch() {
+  const int num = 5000, k = 2;
+  SArray<Key> src_key(num), dst_key(num);
+  SArray<float> src_val(num * k);
+  for (int i = 0; i < num; ++i) {
+    src_key[i] = static_cast<Key>(3 * i);      // multiples of 3
+    dst_key[i] = static_cast<Key>(2 * i + 6);  // even numbers from 6: every third one matches
+    src_val[2 * i] = static_cast<float>(i);
+    src_val[2 * i + 1] = static_cast<float>(-i);
+  }
+  std::vector<float> dst_val(10, 100.0f);  // the first five keys hold 100, the rest come as 0
+  const size_t n = pskv::GpuOrderedMatch(src_key, src_val, dst_key, &dst_val, k, PSKV_OP_PLUS);
+  size_t want_n = 0;
+  bool ok = dst_val.size() == static_cast<size_t>(num) * k;
+  for (int i = 0; i < num && ok; ++i) {
+    const Key key = dst_key[i];
+    float a = i < 5 ? 100.0f : 0.0f, b = a;
+    if (key % 3 == 0 && key / 3 < static_cast<Key>(num)) {
+      a += static_cast<float>(key / 3);
+      b -= static_cast<float>(key / 3);
+      want_n += k;
+    }
+    ok = dst_val[2 * i] == a && dst_val[2 * i + 1] == b;
+  }
+  EXPECT(ok);
+  EXPECT(n == want_n);
+  bool threw = false;
+  try {
+    pskv::GpuOrderedMatch(src_key, src_val, dst_key, &dst_val, 3, PSKV_OP_PLUS);  // 3 values per key: sizes do not fit
+  } catch (const dmlc::Error&) {
+    threw = true;
+  }
+  EXPECT(threw);
+  std::printf("ordered match: %zu of %d values matched\n", n, num * k);
+}
+
 static void RunTwoWorkers(int app_id) {
   std::thread t0(RunOneOfTwoWorkers, app_id, 0);
   std::thread t1(RunOneOfTwoWorkers, app_id, 1);
@@ -318,6 +357,7 @@ int main(int argc, char** argv) {
     RunFixed();
     RunVarLen();
     RunFailures(num_servers);
+    RunOrderedMatch();
     auto s6 = StartServers(6, num_servers, PSKV_MODE_SCALAR);
     RunTwoWorkers(6);
     if (argc > 2) {  // floats per key of the dense run from host memory (4194304 is the configuration's)
