@@ -37,6 +37,10 @@ namespace {
 constexpr uint64_t kDefaultCapacity = 1u << 20;
 constexpr uint64_t kMinSlots = 1024;
 constexpr unsigned kMaxGrid = 1u << 20;
+// The write-back of the SCALAR key cache mostly finds nothing to do (the request in flight repeats
+// the cached keys, or the slots are up to date), and a launch costs by the workgroup even then:
+// 62,500 workgroups that leave at once took 15 us. It strides over the keys with this many.
+constexpr unsigned kFlushGrid = 4096;
 constexpr size_t kMaxProfSamples = 65536;
 constexpr uint64_t kSlackBytes = 256ull << 20;  // tables up to this size trade memory for fewer waits
 // Host-resident requests up to this size (per direction) skip the copy commands: the kernels
@@ -403,7 +407,7 @@ int flush_scalar_cache(pskv_table* t) {
   d.arena = static_cast<float*>(t->sc_vals.ptr);
   d.tile_key = static_cast<uint32_t*>(t->sc_slots.ptr);
   d.cache_mode = kFlushAlways;
-  d.nblk = grid_for(t->cache_n, kBlock, kMaxGrid);
+  d.nblk = grid_for(t->cache_n, kBlock, kFlushGrid);
   hipLaunchKernelGGL(k_scalar_flush, dim3(d.nblk, 1), dim3(kBlock), 0, t->stream, rb);
   PSKV_HIP(hipGetLastError());
   t->sc_dirty = false;
@@ -789,7 +793,7 @@ int run_scalar(Batch& bt, bool push, bool pull) {
     // does NOT repeat the cached keys (cache_mode reads as kFlushUnlessSame in that kernel)
     static_assert(kFlushUnlessSame == kCacheOn, "one descriptor serves both kernels");
     rc = launch_batch(bt, -1, k_scalar_flush, [](const Item& it) {
-      return it.flush_unless_same ? (uint64_t)grid_for(it.r.n, kBlock, kMaxGrid) : 0ull;
+      return it.flush_unless_same ? (uint64_t)grid_for(it.r.n, kBlock, kFlushGrid) : 0ull;
     });
     if (rc) return rc;
   }

@@ -1220,3 +1220,28 @@ def test_other_rows_in_every_batch(capi, orc, dev, mode):
             assert np.array_equal(from_dev(out_lens), want_lens), "lens of step %d" % step
     _check_dump(t, o, "other rows in every batch")
     t.close()
+
+
+def test_scalar_key_cache_written_back_at_scale(capi, orc, dev):
+    """1.5M keys pushed four times (the values then live in the request-ordered array, ahead of the
+    slots), then other keys: the write-back to the slots, whose launch strides over the keys with a
+    bounded number of workgroups, has to bring every slot up to date first. Whole store against the
+    oracle."""
+    announce("scalar_key_cache_write_back")
+    rng = np.random.default_rng(41)
+    n = 1500000
+    keys = unique_keys(rng, n)
+    other = unique_keys(rng, 200000)
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=4 * n)
+    o = orc.Store(orc.MODE_SCALAR)
+    dk = to_dev(keys, dev)
+    for _ in range(4):
+        v = rng.normal(0, 1, size=n).astype(np.float32)
+        t.push(dk, to_dev(v, dev))
+        o.push(keys, v)
+    v = rng.normal(0, 1, size=other.size).astype(np.float32)
+    t.push(to_dev(other, dev), to_dev(v, dev))
+    o.push(other, v)
+    t.sync()
+    _check_dump(t, o, "write-back at scale")
+    t.close()
