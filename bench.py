@@ -14,6 +14,13 @@ Workloads (BASELINE.json `configs`):
       step is one push of all keys followed by a pull with lens. value = keys/s.
   zipf (configs[3]): one table; a step pushes 4,000,000 distinct Zipf(1.1)-popular keys
       of a 100M-key universe and pulls them back; 8 steps. value = keys/s.
+Further workloads (not BASELINE configurations):
+  sparse_repeat: the same 16,000,000 keys pushed and pulled every step (the shape of the
+      reference's own test, tests/test_kv_app.cc:27-41, at the size of a model).
+  embed: one table of 8M rows of 64 floats; a step pulls the rows of 1,000,000 keys, another
+      random subset every step, and pushes a gradient for the same keys.
+  match: the ordered match of two sorted key sets (parallel_kv_match.h:29-120), 12M source
+      keys merged into 16M destination keys. value = keys of both sides / s.
 
 Prints ONE JSON line. Inputs are resident in HBM before the clock starts. `value` comes
 from exactly K timed steps. `roofline` is the dominant kernel of the workload, timed inside
@@ -48,7 +55,8 @@ SAMPLE_EVERY = 4  # (--sample-every)
 # runs under profiles/ carry one line per kernel and launch shape,
 #   traffic_per_launch: kind=<kind> units=<keys or floats per launch> read_bytes=<r> written_bytes=<w>
 # and this script reports a figure only when it finds the line for the launch shape it ran.
-TRAFFIC_FILES = ("sparse_lr.txt", "dense.txt", "varlen.txt", "zipf.txt", "sparse_repeat.txt")
+TRAFFIC_FILES = ("sparse_lr.txt", "dense.txt", "varlen.txt", "zipf.txt", "sparse_repeat.txt", "embed.txt",
+                 "match.txt")
 _traffic_cache = None
 
 
@@ -968,6 +976,16 @@ def run_match(args, capi, dev):
     # both key sets once, and per matched key the source value in, the destination value in and out
     alg = 8.0 * (n_src + n_dst) + 12.0 * shared
     samples = np.array(samples, np.float32)
+    # the same kernel when both sides hold the same keys (a worker that pulled all of its keys):
+    # every value line is used in full
+    own = torch.zeros(n_dst, dtype=torch.float32, device=dev)
+    equal_ms = []
+    for i in range(6):
+        assert capi.match(d_dk, d_dv, d_dk, own, 1, capi.OP_ASSIGN, kernel_ms=ms) == n_dst
+        if i:
+            equal_ms.append(float(ms[0]))
+    assert torch.equal(own, d_dv)
+    equal_ms = np.array(equal_ms, np.float32)
     res = {
         "metric": "source + destination keys/sec of the ordered match and achieved GB/s (% of HBM peak) on 1 MI355X",
         "value": (n_src + n_dst) * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
@@ -980,6 +998,11 @@ def run_match(args, capi, dev):
                                   samples),
                          kernel="k_match_keys<k = 1> (stretch of source keys through LDS, values combined)",
                          bytes_per_key=round(alg / (n_src + n_dst), 2)),
+        # 8 B per key of either side, source value in, destination value out (ASSIGN reads no old value)
+        "kernels": {"match_equal_key_sets": dict(roofline(24.0 * n_dst, len(equal_ms), float(equal_ms.sum()), None,
+                                                          equal_ms),
+                                                 kernel="k_match_keys<k = 1>, both sides the same %d keys, "
+                                                        "dst[i] = src[i]" % n_dst, bytes_per_key=12)},
     }
     return res, (src_keys, src_vals, dst_keys, dst_vals)
 
