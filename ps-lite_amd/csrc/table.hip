@@ -416,7 +416,9 @@ int flush_scalar_cache(pskv_table* t) {
 
 int grow_slots(pskv_table* t, uint64_t keys_needed) {
   uint64_t want = next_pow2((uint64_t)((double)keys_needed / t->max_load) + 1);
-  want = std::max(want, t->cap * 2);
+  // at least twice the slots; four times while that stays a small array (a table that starts at the
+  // default size and keeps growing then re-inserts its keys half as often on the way up)
+  want = std::max(want, t->cap * 4 * sizeof(Slot) <= kSlackBytes ? t->cap * 4 : t->cap * 2);
   Slot* fresh = nullptr;
   int rc = PSKV_OK;
   if (t->mode == PSKV_MODE_SCALAR) {
