@@ -267,6 +267,16 @@ void* pskv_host_alloc(size_t bytes);
 void pskv_host_free(void* ptr);
 int pskv_host_trim(void);
 
+/* Device memory the library keeps for reuse goes back to the system (no counterpart in the
+ * reference): the slot arrays and row storage that growths have replaced (they stay in a
+ * memory pool of the library, one per device, because releasing a few hundred MB costs
+ * hundreds of microseconds that would land in the caller's next wait; the pool reuses them
+ * for later growths of any table, and gives them up when this is called) and the workspaces
+ * and staging buffers of pskv_match, which only grow (a 16M-key host-resident call leaves
+ * several GiB behind). Memory in use by live tables is not touched. Calls of pskv_match on
+ * the device wait for it and it for them. */
+int pskv_device_trim(int device);
+
 /* Text of the last error on the calling thread ("" if none). */
 const char* pskv_last_error(void);
 /* "pskv <major>.<minor> gfx950" */

@@ -41,7 +41,7 @@ SYMBOLS = [
     "pskv_table_create", "pskv_table_destroy", "pskv_push", "pskv_pull", "pskv_pushpull",
     "pskv_sync", "pskv_table_stream", "pskv_push_multi", "pskv_pull_multi", "pskv_sync_multi", "pskv_size", "pskv_dump", "pskv_slice", "pskv_slice_noalloc", "pskv_server_ranges",
     "pskv_assemble_pull", "pskv_match", "pskv_prof_enable", "pskv_prof_reset", "pskv_prof_read", "pskv_prof_samples",
-    "pskv_copy_probe", "pskv_host_alloc", "pskv_host_free", "pskv_host_trim", "pskv_last_error",
+    "pskv_copy_probe", "pskv_host_alloc", "pskv_host_free", "pskv_host_trim", "pskv_device_trim", "pskv_last_error",
     "pskv_version",
 ]
 
@@ -107,6 +107,7 @@ def load():
     lib.pskv_host_alloc.restype = vp
     lib.pskv_host_free.argtypes = [vp]
     lib.pskv_host_free.restype = None
+    lib.pskv_device_trim.argtypes = [i32]
     lib.pskv_last_error.restype = ctypes.c_char_p
     lib.pskv_version.restype = ctypes.c_char_p
     _lib = lib
@@ -468,6 +469,11 @@ def host_free(ptr):
 
 def host_trim():
     _check(load().pskv_host_trim())
+
+
+def device_trim(device=0):
+    """Gives the device memory that the library keeps for reuse back to the system."""
+    _check(load().pskv_device_trim(device))
 
 
 def host_array(ptr, count, dtype):

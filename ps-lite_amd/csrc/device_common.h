@@ -259,6 +259,15 @@ __device__ __forceinline__ uint64_t mix64(uint64_t x) {
   return x;
 }
 
+// Home slot of a key in an array of mask + 1 slots (a power of two, at least 2): the TOP bits of
+// the hash. A key's home in an array of G times the slots is then G * home + (a few more bits),
+// so the keys of one stretch of an array are the keys of the G times longer stretch at the same
+// relative place of the larger array, which lets a growth stream through both arrays instead of
+// scattering every key (k_regrow).
+__device__ __forceinline__ uint64_t home_slot(uint64_t key, uint64_t mask) {
+  return mix64(key) >> __builtin_clzll(mask);
+}
+
 // Inclusive prefix sum over the 64 lanes of a wavefront. Every lane must call it.
 __device__ __forceinline__ unsigned long long wave_incl_scan_u64(unsigned long long x) {
   const unsigned lane = __lane_id();
@@ -301,7 +310,7 @@ __device__ __forceinline__ uint64_t* find_or_insert(Slot* __restrict__ slots, ui
     seen = st->special_payload;
     return reinterpret_cast<uint64_t*>(&st->special_payload);
   }
-  uint64_t h = mix64(key) & mask;
+  uint64_t h = home_slot(key, mask);
   for (uint64_t probes = 0; probes <= mask; ++probes) {
     const u64x2 s = load_slot(&slots[h]);
     if (s.x == key) {
@@ -333,7 +342,7 @@ __device__ __forceinline__ bool find_only(const Slot* __restrict__ slots, uint64
     payload = st->special_payload;
     return st->special_present != 0u;
   }
-  uint64_t h = mix64(key) & mask;
+  uint64_t h = home_slot(key, mask);
   for (uint64_t probes = 0; probes <= mask; ++probes) {
     const u64x2 s = load_slot(&slots[h]);
     if (s.x == key) {

@@ -17,6 +17,9 @@ void clear_error();
 // Whether [ptr, ptr + bytes) lies inside one buffer handed out by pskv_host_alloc (pinned memory).
 bool host_pool_owns(const void* ptr, size_t bytes);
 
+// Frees the workspaces of the device's ordered-match context (match.hip); part of pskv_device_trim.
+int match_trim(int device);
+
 #define PSKV_HIP(call)                                                                     \
   do {                                                                                     \
     hipError_t e_ = (call);                                                                \

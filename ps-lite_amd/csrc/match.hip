@@ -296,13 +296,13 @@ int room(MatchCtx::Buf* b, size_t bytes, hipStream_t stream) {
   return PSKV_OK;
 }
 
-MatchCtx* match_ctx(int device) {
+MatchCtx* match_ctx(int device, bool create = true) {
   constexpr int kMaxDevices = 64;
   static std::mutex* mu = new std::mutex();
   static MatchCtx* table[kMaxDevices] = {nullptr};
   if (device < 0 || device >= kMaxDevices) return nullptr;
   std::lock_guard<std::mutex> lk(*mu);
-  if (table[device]) return table[device];
+  if (table[device] || !create) return table[device];
   MatchCtx* c = new (std::nothrow) MatchCtx();  // kept until the process ends
   if (!c) return nullptr;
   bool ok = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) == hipSuccess;
@@ -323,6 +323,24 @@ MatchCtx* match_ctx(int device) {
 }
 
 }  // namespace
+
+// Gives back the workspaces and staging buffers the device's match context has grown to (they
+// only grow, and a model-size host-resident call leaves several GiB behind).
+int match_trim(int device) {
+  MatchCtx* c = match_ctx(device, false);
+  if (!c) return PSKV_OK;
+  DeviceGuard guard(device);
+  if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", device);
+  std::lock_guard<std::mutex> lk(c->mu);
+  MatchCtx::Buf* bufs[] = {&c->where, &c->spans, &c->tile_count, &c->stage[0], &c->stage[1], &c->stage[2], &c->stage[3]};
+  for (MatchCtx::Buf* b : bufs) {
+    if (b->ptr) PSKV_HIP(hipFree(b->ptr));
+    b->ptr = nullptr;
+    b->cap = 0;
+  }
+  return PSKV_OK;
+}
+
 }  // namespace pskv
 
 using namespace pskv;

@@ -4,10 +4,13 @@
 // calls in place of KVServerDefaultHandle (include/ps/kv_app.h:440-463).
 #include <algorithm>
 #include <atomic>
+#include <chrono>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include <hip/hip_ext.h>
@@ -43,6 +46,10 @@ constexpr unsigned kMaxGrid = 1u << 20;
 constexpr unsigned kFlushGrid = 4096;
 constexpr size_t kMaxProfSamples = 65536;
 constexpr uint64_t kSlackBytes = 256ull << 20;  // tables up to this size trade memory for fewer waits
+// A slot array that could run short is replaced without asking the device first while the larger
+// one stays below this size; beyond it the host waits for exact counters before it spends the memory.
+constexpr uint64_t kGrowUnaskedBytes = 4096ull << 20;
+constexpr uint64_t kSpareMaxBytes = 16384ull << 20;  // no array larger than this is allocated ahead of need
 // Host-resident requests up to this size (per direction) skip the copy commands: the kernels
 // read the request from, and write the response to, pinned host memory mapped into the GPU.
 constexpr size_t kSmallBytes = 1024u << 10;
@@ -119,6 +126,16 @@ struct pskv_table {
   Slot* slots = nullptr;
   bool slots_pooled = false, arena_pooled = false;  // taken from the stream-ordered pool by a growth
   uint64_t cap = 0;        // slots, a power of two
+  // The array the next growth will move into, allocated ahead of need (once the table is 70 % of
+  // the way to that growth) at the end of a request, while the GPU is busy with that request:
+  // allocating costs the host 50-100 us, which would otherwise be spent with the GPU idle.
+  Slot* spare = nullptr;
+  uint64_t spare_cap = 0;
+  bool spare_pooled = false;
+  // what the sizing logic did, printed when the table goes if PSKV_STATS is set in the environment
+  struct Stats {
+    uint64_t requests = 0, waits = 0, growths = 0, growths_unasked = 0, spare_used = 0, records = 0, catch_ups = 0;
+  } stats;
   uint64_t count = 0;      // key count at the last read_state()
 
   // Host-side bounds of what the device counters can have reached. Requests are enqueued
@@ -132,6 +149,7 @@ struct pskv_table {
   static const int kLog = 64;
   uint64_t log_keys[kLog] = {0}, log_units[kLog] = {0};
   Snapshot* snap = nullptr;  // pinned host memory the device publishes into
+  uint64_t record_seq = ~0ull;  // the newest request that was asked to publish its counters (all ones: none yet)
   DevState* st = nullptr;  // device
   StateView* st_host = nullptr;  // pinned: what read_state() last read of the device state
 
@@ -186,6 +204,7 @@ struct pskv_table {
   unsigned long long sc_seen = 0;         // the value of *outcome the host last looked at
   uint64_t sc_min_keys = 0;               // requests below this size leave the cache alone; 0 = no cache
 
+  bool counted = false;  // among the live tables of its device
   bool prof = false;
   std::vector<EventPair> pending[PSKV_KERNEL_COUNT];
   std::vector<EventPair> free_events;
@@ -202,8 +221,8 @@ namespace {
 // begin/end timestamps of that very dispatch: the same clock a profiler reads,
 // without the idle time that events recorded around a launch would add.
 template <typename... KArgs, typename... Args>
-void launch(pskv_table* t, int prof_kernel, void (*kernel)(KArgs...), dim3 grid, dim3 block,
-            Args... args) {
+void launch_lds(pskv_table* t, int prof_kernel, void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds,
+                Args... args) {
   if (t->prof && prof_kernel >= 0) {
     EventPair ev;
     bool have = false;
@@ -219,12 +238,18 @@ void launch(pskv_table* t, int prof_kernel, void (*kernel)(KArgs...), dim3 grid,
       }
     }
     if (have) {
-      hipExtLaunchKernelGGL(kernel, grid, block, 0, t->stream, ev.a, ev.b, 0, static_cast<KArgs>(args)...);
+      hipExtLaunchKernelGGL(kernel, grid, block, lds, t->stream, ev.a, ev.b, 0, static_cast<KArgs>(args)...);
       t->pending[prof_kernel].push_back(ev);
       return;
     }
   }
-  hipLaunchKernelGGL(kernel, grid, block, 0, t->stream, static_cast<KArgs>(args)...);
+  hipLaunchKernelGGL(kernel, grid, block, lds, t->stream, static_cast<KArgs>(args)...);
+}
+
+template <typename... KArgs, typename... Args>
+void launch(pskv_table* t, int prof_kernel, void (*kernel)(KArgs...), dim3 grid, dim3 block,
+            Args... args) {
+  launch_lds(t, prof_kernel, kernel, grid, block, 0, args...);
 }
 
 int prof_collect(pskv_table* t) {
@@ -324,26 +349,57 @@ int report_device_errors(pskv_table* t) {
 // growth releases the old array behind the kernel that empties it, without a wait on the host
 // (a plain hipFree of a few hundred MB blocks the host for 150-440 us, longer than the
 // re-insertion itself). `pooled` says how the array must be released later.
-int alloc_for_growth(void** out, size_t bytes, hipStream_t stream, bool* pooled) {
-  // asked once per device (0 = not asked yet, 1 = no pool, 2 = pool)
-  static std::atomic<int> known[64];
-  int dev = 0;
-  bool have_pool = false;
-  if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
-    int k = known[dev].load(std::memory_order_relaxed);
+// The pool is the library's own, one per device, and keeps what is freed into it: the default
+// pool hands freed memory back to the system at the next wait of any stream, which for the old
+// array of a growth is an unmapping of hundreds of microseconds in the middle of the caller's
+// loop. pskv_device_trim gives the kept memory back; so does the end of the last table.
+struct DevicePool {
+  std::atomic<int> known{0};  // 0 = not asked yet, 1 = no pool, 2 = pool
+  hipMemPool_t pool = nullptr;
+  std::atomic<long> tables{0};  // live tables on the device
+};
+DevicePool g_pools[64];
+
+hipMemPool_t device_pool(int dev) {
+  if (dev < 0 || dev >= 64) return nullptr;
+  DevicePool& dp = g_pools[dev];
+  int k = dp.known.load(std::memory_order_acquire);
+  if (k == 0) {
+    static std::mutex mu;
+    std::lock_guard<std::mutex> lock(mu);
+    k = dp.known.load(std::memory_order_acquire);
     if (k == 0) {
       int ok = 0;
       if (std::getenv("PSKV_NO_ASYNC_ALLOC") ||
           hipDeviceGetAttribute(&ok, hipDeviceAttributeMemoryPoolsSupported, dev) != hipSuccess)
         ok = 0;
+      if (ok) {
+        hipMemPoolProps props;
+        std::memset(&props, 0, sizeof(props));
+        props.allocType = hipMemAllocationTypePinned;
+        props.handleTypes = hipMemHandleTypeNone;
+        props.location.type = hipMemLocationTypeDevice;
+        props.location.id = dev;
+        uint64_t keep = ~0ull;
+        if (hipMemPoolCreate(&dp.pool, &props) != hipSuccess ||
+            hipMemPoolSetAttribute(dp.pool, hipMemPoolAttrReleaseThreshold, &keep) != hipSuccess) {
+          dp.pool = nullptr;
+          ok = 0;
+        }
+      }
       (void)hipGetLastError();
       k = ok ? 2 : 1;
-      known[dev].store(k, std::memory_order_relaxed);
+      dp.known.store(k, std::memory_order_release);
     }
-    have_pool = k == 2;
   }
-  if (have_pool) {
-    if (hipMallocAsync(out, bytes, stream) == hipSuccess) {
+  return k == 2 ? dp.pool : nullptr;
+}
+
+int alloc_for_growth(void** out, size_t bytes, hipStream_t stream, bool* pooled) {
+  int dev = 0;
+  hipMemPool_t pool = hipGetDevice(&dev) == hipSuccess ? device_pool(dev) : nullptr;
+  if (pool) {
+    if (hipMallocFromPoolAsync(out, bytes, pool, stream) == hipSuccess) {
       *pooled = true;
       return PSKV_OK;
     }
@@ -366,11 +422,11 @@ int release_after(void* ptr, bool pooled, hipStream_t stream) {
   return PSKV_OK;
 }
 
-int alloc_slots(uint64_t cap, Slot** out, hipStream_t stream, bool* pooled) {
+int alloc_slots(uint64_t cap, Slot** out, hipStream_t stream, bool* pooled, bool fill = true) {
   int rc = alloc_for_growth(reinterpret_cast<void**>(out), cap * sizeof(Slot), stream, pooled);
   if (rc) return rc;
-  // all-ones bytes: key = empty marker
-  PSKV_HIP(hipMemsetAsync(*out, 0xFF, cap * sizeof(Slot), stream));
+  // all-ones bytes: key = empty marker (k_regrow writes every slot itself and needs no fill)
+  if (fill) PSKV_HIP(hipMemsetAsync(*out, 0xFF, cap * sizeof(Slot), stream));
   return PSKV_OK;
 }
 
@@ -414,11 +470,16 @@ int flush_scalar_cache(pskv_table* t) {
   return PSKV_OK;
 }
 
+// The slots a growth goes to when the table has to hold `keys_needed` keys: at least twice the
+// slots; four times while that stays a small array (a table that starts at the default size and
+// keeps growing then moves its keys half as often on the way up).
+uint64_t grown_cap(const pskv_table* t, uint64_t keys_needed) {
+  const uint64_t want = next_pow2((uint64_t)((double)keys_needed / t->max_load) + 1);
+  return std::max(want, t->cap * 4 * sizeof(Slot) <= kSlackBytes ? t->cap * 4 : t->cap * 2);
+}
+
 int grow_slots(pskv_table* t, uint64_t keys_needed) {
-  uint64_t want = next_pow2((uint64_t)((double)keys_needed / t->max_load) + 1);
-  // at least twice the slots; four times while that stays a small array (a table that starts at the
-  // default size and keeps growing then re-inserts its keys half as often on the way up)
-  want = std::max(want, t->cap * 4 * sizeof(Slot) <= kSlackBytes ? t->cap * 4 : t->cap * 2);
+  uint64_t want = grown_cap(t, keys_needed);
   Slot* fresh = nullptr;
   int rc = PSKV_OK;
   if (t->mode == PSKV_MODE_SCALAR) {
@@ -428,16 +489,63 @@ int grow_slots(pskv_table* t, uint64_t keys_needed) {
     t->cache_valid = false;
   }
   bool pooled = false;
-  rc = alloc_slots(want, &fresh, t->stream, &pooled);
-  if (rc) return rc;
-  launch(t, PSKV_KERNEL_REHASH, k_rehash, dim3(grid_for(t->cap, kBlock, kMaxGrid)), dim3(kBlock),
-         (const Slot*)t->slots, t->cap, fresh, want - 1, t->st);
+  ++t->stats.growths;
+  if (t->spare && t->spare_cap >= want) {
+    ++t->stats.spare_used;
+    fresh = t->spare;
+    want = t->spare_cap;
+    pooled = t->spare_pooled;
+  } else {
+    if (t->spare) {  // too small after all
+      rc = release_after(t->spare, t->spare_pooled, t->stream);
+      if (rc) return rc;
+    }
+    rc = alloc_slots(want, &fresh, t->stream, &pooled, false);
+    if (rc) return rc;
+  }
+  t->spare = nullptr;
+  t->spare_cap = 0;
+  const uint64_t factor = want / t->cap;
+  if (factor <= (uint64_t)kRegrowMaxFactor) {
+    // two streaming passes: the new array is written whole, slot by slot, from LDS
+    const unsigned nblk = (unsigned)(t->cap / kRegrowOld);
+    const size_t lds = (size_t)kRegrowOld * factor * 2 * sizeof(unsigned long long);
+    launch_lds(t, PSKV_KERNEL_REHASH, k_regrow, dim3(nblk), dim3(kBlock), lds, t->slots, fresh, t->cap - 1,
+               want - 1, (unsigned)factor);
+    PSKV_HIP(hipGetLastError());
+    launch(t, PSKV_KERNEL_REHASH, k_regrow_rest, dim3((nblk * kRestLanes + kBlock - 1) / kBlock), dim3(kBlock),
+           (const Slot*)t->slots, t->cap, fresh, want - 1, t->st);
+  } else {
+    // (a small table that a large request makes much larger: fill and scatter)
+    PSKV_HIP(hipMemsetAsync(fresh, 0xFF, want * sizeof(Slot), t->stream));
+    launch(t, PSKV_KERNEL_REHASH, k_rehash, dim3(grid_for(t->cap, kBlock, kMaxGrid)), dim3(kBlock),
+           (const Slot*)t->slots, t->cap, fresh, want - 1, t->st);
+  }
   PSKV_HIP(hipGetLastError());
   rc = release_after(t->slots, t->slots_pooled, t->stream);
   t->slots = fresh;
   t->slots_pooled = pooled;
   t->cap = want;
   return rc;
+}
+
+// Called at the end of a request, with its kernels queued: allocates the array of the next growth
+// once the keys the table is known to hold have come 70 % of the way to that growth.
+void prepare_growth(pskv_table* t) {
+  if (t->spare || t->no_growth) return;
+  const double limit = (double)t->max_load * (double)t->cap;
+  if ((double)t->base_count <= 0.7 * limit) return;
+  const uint64_t want = grown_cap(t, 0);
+  if (want * sizeof(Slot) > kSpareMaxBytes) return;
+  Slot* fresh = nullptr;
+  bool pooled = false;
+  if (alloc_slots(want, &fresh, t->stream, &pooled, false) != PSKV_OK) {
+    clear_error();  // the growth itself will ask again and report
+    return;
+  }
+  t->spare = fresh;
+  t->spare_cap = want;
+  t->spare_pooled = pooled;
 }
 
 int grow_arena(pskv_table* t, uint64_t floats_needed, uint64_t live_floats) {
@@ -484,9 +592,39 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
   if (t->seq - t->base_seq >= (uint64_t)pskv_table::kLog / 4) adopt_snapshot(t);
   if (slots_short() || arena_short() || t->seq - t->base_seq >= (uint64_t)pskv_table::kLog - 1) {
     adopt_snapshot(t);
-    if (slots_short() || arena_short() || t->seq - t->base_seq >= (uint64_t)pskv_table::kLog - 1) {
+    const bool old_log = t->seq - t->base_seq >= (uint64_t)pskv_table::kLog - 1;
+    if (slots_short() && !arena_short() && !old_log && (double)(t->base_count + n) <= limit &&
+        t->record_seq != ~0ull && t->record_seq >= t->base_seq) {
+      // The array is only short if the requests in flight create most of their keys, and some of
+      // them are going to say how many they did create: the host lets the device catch up until the
+      // newest record settles the matter one way or the other. The device still has the requests
+      // behind that record to work on, so it does not run dry as it would in a wait for the stream;
+      // a caller that runs many requests ahead is merely held back to a few.
+      const auto t0 = std::chrono::steady_clock::now();
+      unsigned spins = 0;
+      while (slots_short() && (double)(t->base_count + n) <= limit && t->record_seq >= t->base_seq) {
+        adopt_snapshot(t);
+        if ((++spins & 63u) == 0) {
+          if (std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(20)) break;
+          std::this_thread::yield();
+        }
+      }
+      ++t->stats.catch_ups;
+    }
+    if (slots_short() && !arena_short() && !old_log &&
+        grown_cap(t, t->base_count + t->pend_keys + n) * sizeof(Slot) <= kGrowUnaskedBytes) {
+      // Only the slots could run short, and the larger array is not a large one: it is taken now,
+      // sized for what the requests in flight could create at most, without asking the device how
+      // many keys they did create. The move is queued behind them; nothing waits.
+      const uint64_t most = t->base_count + t->pend_keys + n;
+      const uint64_t slack_n = t->cap * sizeof(Slot) <= kSlackBytes ? 2 * n : 0;
+      int rc = grow_slots(t, most + slack_n);
+      if (rc) return rc;
+      ++t->stats.growths_unasked;
+    } else if (slots_short() || arena_short() || old_log) {
       int rc = read_state(t);  // exact counters, stream idle
       if (rc) return rc;
+      ++t->stats.waits;
       // The wait happened because requests in flight had to be assumed to create all their
       // keys. Small tables get room for two more such requests, so that a caller who keeps
       // requests of this size in flight does not wait again on every one of them; for large
@@ -516,9 +654,12 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
   // (a base that merely grows old asks for a record every eighth request, not every one)
   const uint64_t age = t->seq - t->base_seq;
   const bool old_base = age >= (uint64_t)pskv_table::kLog / 4 && (age % 8 == 0 || age >= (uint64_t)pskv_table::kLog - 8);
+  ++t->stats.requests;
   if (tight_slots || tight_arena || old_base) {
     pub->snap = t->snap;
     pub->seq = q;
+    t->record_seq = q;
+    ++t->stats.records;
   }
   return PSKV_OK;
 }
@@ -1189,11 +1330,16 @@ int run_varlen(Batch& bt, bool push, bool pull) {
 }
 
 int run_batch(Batch& bt, bool push, bool pull) {
+  int rc;
   switch (bt[0].t->mode) {
-    case PSKV_MODE_SCALAR: return run_scalar(bt, push, pull);
-    case PSKV_MODE_FIXED: return run_fixed(bt, push, pull);
-    default: return run_varlen(bt, push, pull);
+    case PSKV_MODE_SCALAR: rc = run_scalar(bt, push, pull); break;
+    case PSKV_MODE_FIXED: rc = run_fixed(bt, push, pull); break;
+    default: rc = run_varlen(bt, push, pull); break;
   }
+  // the GPU is busy with the request now: the moment to allocate ahead of a coming growth
+  if (!rc)
+    for (Item& it : bt) prepare_growth(it.t);
+  return rc;
 }
 
 // Host-side checks that mirror the CHECKs of the reference and the frozen rules of
@@ -1617,6 +1763,8 @@ int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
           hipSuccess ||
       hipStreamSynchronize(t->stream) != hipSuccess)
     return fail(set_error(PSKV_EHIP, "table initialisation failed"));
+  g_pools[t->device < 64 ? t->device : 63].tables.fetch_add(1);
+  t->counted = true;
   *out = t;
   return PSKV_OK;
 }
@@ -1624,6 +1772,13 @@ int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
 int pskv_table_destroy(pskv_table* t) {
   if (!t) return PSKV_OK;
   DeviceGuard guard(t->device);
+  if (std::getenv("PSKV_STATS"))
+    fprintf(stderr, "[pskv] table %p mode %d: %llu requests, %llu slots at the end, %llu growths (%llu without asking "
+            "the device, %llu into an array allocated ahead), %llu waits for exact counters, %llu for the newest record, %llu counter records\n",
+            (void*)t, t->mode, (unsigned long long)t->stats.requests, (unsigned long long)t->cap,
+            (unsigned long long)t->stats.growths, (unsigned long long)t->stats.growths_unasked,
+            (unsigned long long)t->stats.spare_used, (unsigned long long)t->stats.waits,
+            (unsigned long long)t->stats.catch_ups, (unsigned long long)t->stats.records);
   if (t->stream) (void)hipStreamSynchronize(t->stream);
   for (int k = 0; k < PSKV_KERNEL_COUNT; ++k)
     for (const EventPair& ev : t->pending[k]) t->free_events.push_back(ev);
@@ -1641,7 +1796,12 @@ int pskv_table_destroy(pskv_table* t) {
     (void)hipFreeAsync(t->arena, t->stream);
     t->arena = nullptr;
   }
-  if (t->slots_pooled || t->arena_pooled) (void)hipStreamSynchronize(t->stream);
+  if (t->spare && t->spare_pooled) {
+    (void)hipFreeAsync(t->spare, t->stream);
+  } else if (t->spare) {
+    (void)hipFree(t->spare);
+  }
+  if (t->slots_pooled || t->arena_pooled || t->spare_pooled) (void)hipStreamSynchronize(t->stream);
   if (t->st) (void)hipFree(t->st);
   if (t->st_host) (void)hipHostFree(t->st_host);
   if (t->snap) (void)hipHostFree(t->snap);
@@ -1660,6 +1820,10 @@ int pskv_table_destroy(pskv_table* t) {
   if (t->cache_lens.ptr) (void)hipFree(t->cache_lens.ptr);
   if (t->stage_out.ptr) (void)hipFree(t->stage_out.ptr);
   if (t->own_stream && t->stream) (void)hipStreamDestroy(t->stream);
+  // the last table of a device to go takes the memory the pool has kept with it
+  DevicePool& dp = g_pools[t->device < 64 ? t->device : 63];
+  if (t->counted && dp.tables.fetch_sub(1) == 1 && dp.known.load(std::memory_order_acquire) == 2 && dp.pool)
+    (void)hipMemPoolTrimTo(dp.pool, 0);
   delete t;
   return PSKV_OK;
 }
@@ -1867,6 +2031,19 @@ int pskv_copy_probe(pskv_table* t, void* dst, const void* src, size_t bytes) {
          static_cast<f32x4*>(dst), static_cast<const f32x4*>(src), n16);
   PSKV_HIP(hipGetLastError());
   return PSKV_OK;
+}
+
+int pskv_device_trim(int device) {
+  clear_error();
+  if (device < 0 || device >= 64) return set_error(PSKV_EINVAL, "device %d out of range", device);
+  DevicePool& dp = g_pools[device];
+  DeviceGuard guard(device);
+  if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", device);
+  if (dp.known.load(std::memory_order_acquire) == 2 && dp.pool) {
+    PSKV_HIP(hipDeviceSynchronize());  // what streams have freed into the pool is the pool's once they got there
+    PSKV_HIP(hipMemPoolTrimTo(dp.pool, 0));
+  }
+  return match_trim(device);
 }
 
 const char* pskv_last_error(void) { return g_last_error.c_str(); }

@@ -556,9 +556,15 @@ __global__ __launch_bounds__(kBlock) void k_var_push_lookup(ReqBatch b) {
   }
   // the request is refused as a whole when its lens are invalid or do not add up to vals.size(),
   // or when it repeats a key
-  if (st->req_error & (kDevErrBadLen | kDevErrSizeMismatch | kDevErrDuplicate)) return;
+  // (a refused request creates nothing, so the counter record the host may be waiting for holds
+  // the counters as they are)
+  if (st->req_error & (kDevErrBadLen | kDevErrSizeMismatch | kDevErrDuplicate)) {
+    if (snap && blockIdx.x == 0 && threadIdx.x < 64) publish_snapshot(st, snap, snap_seq);
+    return;
+  }
   if (st->scan_total != nvals) {
     if (blockIdx.x == 0 && threadIdx.x == 0) raise_error(st, kDevErrSizeMismatch, tag.epoch);
+    if (snap && blockIdx.x == 0 && threadIdx.x < 64) publish_snapshot(st, snap, snap_seq);
     return;
   }
   __shared__ unsigned long long wsum[kBlock / 64];
@@ -1172,8 +1178,8 @@ __global__ __launch_bounds__(kBlock) void k_rows(ReqBatch b) {
 // Maintenance kernels.
 // ---------------------------------------------------------------------------------
 
-// Growth: every live slot of the old array is re-inserted into the new one; payloads
-// move bit for bit, so stored sums are unchanged.
+// Growth, the general way: every live slot of the old array is re-inserted into the new one
+// (which starts as all ones); payloads move bit for bit, so stored sums are unchanged.
 __global__ __launch_bounds__(kBlock) void k_rehash(const Slot* __restrict__ old_slots,
                                                   uint64_t old_cap, Slot* __restrict__ slots,
                                                   uint64_t mask, DevState* st) {
@@ -1181,7 +1187,7 @@ __global__ __launch_bounds__(kBlock) void k_rehash(const Slot* __restrict__ old_
   for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < old_cap; i += stride) {
     const ulonglong2 s = *reinterpret_cast<const ulonglong2*>(&old_slots[i]);
     if (s.x == kEmptyKey) continue;
-    uint64_t h = mix64(s.x) & mask;
+    uint64_t h = home_slot(s.x, mask);
     bool placed = false;
     for (uint64_t probes = 0; probes <= mask; ++probes) {
       if (slots[h].key == kEmptyKey) {
@@ -1197,6 +1203,107 @@ __global__ __launch_bounds__(kBlock) void k_rehash(const Slot* __restrict__ old_
       h = (h + 1) & mask;
     }
     if (!placed) atomicOr(&st->error, kDevErrFull);
+  }
+}
+
+// Growth by a small power of two G, as two streaming passes instead of a scatter. A key's home
+// slot is the top bits of its hash, so the keys whose homes lie in the old slots [a, a + R) are
+// exactly the keys whose new homes lie in [G * a, G * (a + R)): one workgroup builds that
+// stretch of the new array in LDS from its R old slots and writes it out whole, empty slots
+// included, with coalesced 128-bit stores (the new array needs no fill, and no atomics reach
+// memory). What it cannot place there is left for the second pass: keys that sit in its old
+// slots but have their home in an earlier stretch (a probe chain that crossed the boundary, or
+// wrapped around the end of the array), and keys whose probe chain would leave the LDS stretch.
+// The workgroup writes those, packed, over the front of its own old slots (it is the only one
+// that reads them) with an empty slot behind the last; k_regrow_rest inserts them the general
+// way once every stretch of the new array is in place. At a fill of one half about one key in
+// 250 takes the second pass. Payloads move bit for bit.
+constexpr int kRegrowOld = kBlock;  // old slots per workgroup, one per thread
+constexpr int kRegrowMaxFactor = 8;
+__global__ __launch_bounds__(kBlock) void k_regrow(Slot* __restrict__ old_slots, Slot* __restrict__ slots,
+                                                  uint64_t old_mask, uint64_t mask, unsigned factor) {
+  extern __shared__ unsigned long long regrow_lds[];  // keys of the stretch, then its payloads
+  const unsigned T = kRegrowOld * factor;
+  unsigned long long* tkey = regrow_lds;
+  unsigned long long* tpay = regrow_lds + T;
+  __shared__ unsigned long long red[kBlock / 64 + 1];
+  const uint64_t a = (uint64_t)blockIdx.x * kRegrowOld;
+  const uint64_t A = a * factor;
+  const u64x2 s = __builtin_nontemporal_load(reinterpret_cast<const u64x2*>(&old_slots[a + threadIdx.x]));
+  for (unsigned j = threadIdx.x; j < T; j += kBlock) {
+    tkey[j] = kEmptyKey;
+    tpay[j] = kPayloadUnset;
+  }
+  __syncthreads();
+  const bool live = s.x != kEmptyKey;
+  bool rest = false;
+  if (live) {
+    const uint64_t oh = home_slot(s.x, old_mask);
+    if (oh >= a && oh <= a + threadIdx.x) {
+      unsigned j = (unsigned)(home_slot(s.x, mask) - A);
+      rest = true;
+      for (; j < T; ++j) {
+        if (atomicCAS(&tkey[j], (unsigned long long)kEmptyKey, (unsigned long long)s.x) == kEmptyKey) {
+          tpay[j] = s.y;
+          rest = false;
+          break;
+        }
+      }
+    } else {
+      rest = true;  // its home lies in another workgroup's stretch
+    }
+  }
+  unsigned long long total;
+  const unsigned long long at = block_excl_scan_u64(rest ? 1ull : 0ull, red, total);  // (two barriers)
+  u64x2* out = reinterpret_cast<u64x2*>(slots + A);
+  for (unsigned j = threadIdx.x; j < T; j += kBlock) {
+    u64x2 v;
+    v.x = tkey[j];
+    v.y = tpay[j];
+    __builtin_nontemporal_store(v, &out[j]);
+  }
+  // every thread has read its old slot (the barriers of the scan lie in between)
+  if (rest) *reinterpret_cast<u64x2*>(&old_slots[a + at]) = s;
+  if (threadIdx.x == 0 && total < (unsigned long long)kRegrowOld) old_slots[a + total].key = kEmptyKey;
+}
+
+// Second pass of a growth by k_regrow: sixteen lanes per stretch of kRegrowOld old slots read the
+// keys the first pass left at its front, up to the first empty slot, and insert them the general way.
+constexpr int kRestLanes = 16;
+__global__ __launch_bounds__(kBlock) void k_regrow_rest(const Slot* __restrict__ old_slots, uint64_t old_cap,
+                                                       Slot* __restrict__ slots, uint64_t mask, DevState* st) {
+  const uint64_t stretch = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kRestLanes;
+  const unsigned l = threadIdx.x % kRestLanes;
+  const unsigned group_shift = (threadIdx.x & 63) / kRestLanes * kRestLanes;
+  const uint64_t a = stretch * kRegrowOld;
+  bool more = a < old_cap;
+  for (unsigned c = 0; c < kRegrowOld / kRestLanes; ++c) {
+    u64x2 s;
+    s.x = kEmptyKey, s.y = 0;
+    if (more) s = *reinterpret_cast<const u64x2*>(&old_slots[a + c * kRestLanes + l]);
+    // the lanes of a wavefront stay together for the ballot; a group that is done reads nothing
+    const unsigned long long ends = __ballot(more && s.x == kEmptyKey);
+    const unsigned mine = (unsigned)(ends >> group_shift) & ((1u << kRestLanes) - 1u);
+    const unsigned first_end = mine ? (unsigned)__builtin_ctz(mine) : (unsigned)kRestLanes;
+    if (more && l < first_end) {
+      uint64_t h = home_slot(s.x, mask);
+      bool placed = false;
+      for (uint64_t probes = 0; probes <= mask; ++probes) {
+        if (slots[h].key == kEmptyKey) {
+          unsigned long long old = atomicCAS(reinterpret_cast<unsigned long long*>(&slots[h].key),
+                                             (unsigned long long)kEmptyKey, (unsigned long long)s.x);
+          if (old == kEmptyKey) {
+            slots[h].payload = s.y;
+            placed = true;
+            break;
+          }
+        }
+        h = (h + 1) & mask;
+      }
+      if (!placed) atomicOr(&st->error, kDevErrFull);
+    }
+    if (mine) more = false;
+    if (!__any(more)) break;
   }
 }
 

@@ -109,6 +109,50 @@ def test_scalar_growth(capi, orc, dev):
     _check_dump(t, o, "growth")
 
 
+@pytest.mark.parametrize("max_load", [0.25, 0.5, 0.9])
+@pytest.mark.parametrize("first,step", [(400, 400), (1000, 1000), (300, 5000), (40000, 9000)])
+def test_growth_by_every_factor(capi, orc, dev, max_load, first, step):
+    """A growth by 2, 4 or 8 streams the old array into the new one stretch by stretch and hands
+    the keys of probe chains that cross a stretch (or wrap around the end of the array, frequent
+    at fill 0.9) to a second pass; a growth by more re-inserts every key. Whatever the factor and
+    the fill, every key and every sum arrives: the dump equals the oracle's after every push."""
+    announce("growth_by_every_factor", max_load, first, step)
+    rng = np.random.default_rng(int(max_load * 100) + first)
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=first, max_load=max_load)
+    o = orc.Store(orc.MODE_SCALAR)
+    universe = unique_keys(rng, 16 * step + first)
+    at = 0
+    for rep in range(12):
+        fresh = universe[at:at + step]
+        at += step
+        again = universe[:at][rng.random(at) < 0.1]  # some of the keys held already
+        keys = np.unique(np.concatenate([fresh, again]))
+        vals = rng.integers(-50, 50, size=keys.size).astype(np.float32)
+        t.push(to_dev(keys, dev), to_dev(vals, dev))
+        o.push(keys, vals)
+        if rep % 3 == 2:
+            _check_dump(t, o, "after push %d" % rep)
+    _check_dump(t, o, "growth")
+
+
+def test_growth_of_a_large_array_by_two(capi, orc, dev):
+    """Arrays beyond 64 MB double: 4.6M keys take a table through 4x growths and then a 2x one."""
+    announce("growth_of_a_large_array")
+    rng = np.random.default_rng(77)
+    t = capi.Table(capi.MODE_SCALAR)
+    o = orc.Store(orc.MODE_SCALAR)
+    universe = unique_keys(rng, 4600000)
+    for part in np.array_split(universe, 10):
+        vals = rng.integers(-50, 50, size=part.size).astype(np.float32)
+        t.push(to_dev(part, dev), to_dev(vals, dev))
+        o.push(part, vals)
+    probe = np.sort(rng.choice(universe, size=200000, replace=False))
+    got = np.zeros(probe.size, np.float32)
+    t.pull(probe, got)
+    assert_bits_equal(got, o.pull(probe)[0], "pull after the growths")
+    _check_dump(t, o, "large growth")
+
+
 @pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
 def test_many_requests_in_flight_while_the_table_grows(capi, orc, dev, mode):
     """Device-resident requests are enqueued without waiting, so the host only has bounds on the
