@@ -12,8 +12,9 @@ Workloads (BASELINE.json `configs`):
       1 GiB followed by one full pull. value = algorithmic GB/s.
   varlen (configs[4]): 2,000,000 keys with lens in {8,16,32,64,128} over 16 ranges; a
       step is one push of all keys followed by a pull with lens. value = keys/s.
-  zipf (configs[3]): one table; a step pushes 4,000,000 distinct Zipf(1.1)-popular keys
-      of a 100M-key universe and pulls them back; 8 steps. value = keys/s.
+  zipf (configs[3]): one table; 8 pushes of 4,000,000 distinct Zipf(1.1)-popular keys of a
+      100M-key universe, then one pull of 16,000,000 such keys, most of them absent (the pull
+      inserts them). value = (pushed + pulled keys) / s.
 Further workloads (not BASELINE configurations):
   sparse_repeat: the same 16,000,000 keys pushed and pulled every step (the shape of the
       reference's own test, tests/test_kv_app.cc:27-41, at the size of a model).
@@ -216,161 +217,152 @@ def run_sparse_lr(args, capi, dev):
     rb, re = capi.server_ranges(S)
     d_batches = [(to_dev(k, dev), to_dev(v, dev)) for k, v in batches]
     out = torch.empty(n, dtype=torch.float32, device=dev)
-    # One table per server key range, sized for the keys the run will add. The tables
-    # share one stream: their kernels run back to back, each with the whole GPU, so a
-    # kernel's duration is its own and not that of four overlapping launches.
+    # One table per server key range. The tables share one stream: their kernels run back to
+    # back, each with the whole GPU, so a kernel's duration is its own and not that of four
+    # overlapping launches.
     stream = torch.cuda.Stream()
-    # sized so that the tables end the run about one third of the way to their first growth
-    cap = int(n * (args.warmup + 2 * args.steps) / S * 1.1)
-    group = capi.Group(S, capi.MODE_SCALAR, initial_capacity=cap, stream=stream.cuda_stream)
-    tables = group.tables
-    per_table = args.per_table
+    last = total_steps - 1
+    want = batches[last][1] + np.float32(0.0)  # each key was pushed once: 0.0f + v
 
-    prof_on = [-1]  # the table whose launches carry events at the moment (-1: none)
-
-    def slice_step(i):
-        return capi.slice_keys(d_batches[i][0], rb, re, nvals=n)
-
-    def step(i, sliced, sample=True):
-        # Kernel durations are sampled INSIDE the timed steps: in every SAMPLE_EVERY-th step the
-        # launches carry their own start/stop events (booked to the first table of the group; with
-        # --per-table those of one of the S tables, taken in turn). Events on every launch would
-        # cost more host time per step than the GPU needs for it.
-        if sample:
-            j = i - args.warmup
-            on = sampled(j, args.steps)
-            which = ((j // SAMPLE_EVERY) % S if per_table else 0) if on else -1
-            if which != prof_on[0]:
-                for s in range(S):
-                    tables[s].prof_enable(s == which)
-                prof_on[0] = which
-        dk, dv = d_batches[i]
-        kp, vp, op = dk.data_ptr(), dv.data_ptr(), out.data_ptr()
-        pos, _, used = sliced
-        if not per_table:
-            # one launch per step of the pipeline over all S key ranges
-            group.push_raw(kp, pos, vp, pos)
-            group.pull_raw(kp, pos, op)
-            return
-        pos = [int(x) for x in pos]
-        for s in range(S):
-            if used[s]:
-                c = pos[s + 1] - pos[s]
-                tables[s].push_raw(kp + 8 * pos[s], c, vp + 4 * pos[s], c)
-        for s in range(S):
-            if used[s]:
-                c = pos[s + 1] - pos[s]
-                tables[s].pull_raw(kp + 8 * pos[s], c, op + 4 * pos[s], c)
-
-    def steps(first, last, sample=True):
-        # Every step slices its keys, pushes and pulls, in line. (Slicing the keys of coming steps
-        # ahead of time, on this thread or on a second one, was measured and gains nothing: the
-        # slicer's short kernel shares the GPU with the store's long ones either way.)
-        for i in range(first, last):
-            step(i, slice_step(i), sample)
-
-    def drain():
-        if per_table:
-            for t in tables:
-                t.sync()
+    def measure(cap, per_table, sample, own_streams=False):
+        """The warm-up and the timed steps on fresh tables of `cap` keys each (0: the library's
+        default, tables that grow while the clock runs). Returns seconds and kernel statistics."""
+        if own_streams:
+            tables = [capi.Table(capi.MODE_SCALAR, initial_capacity=cap) for _ in range(S)]
+            group = None
         else:
-            group.sync()
-        torch.cuda.synchronize()
+            group = capi.Group(S, capi.MODE_SCALAR, initial_capacity=cap, stream=stream.cuda_stream)
+            tables = group.tables
+        prof_on = [-1]  # the table whose launches carry events at the moment (-1: none)
 
-    steps(0, args.warmup)
-    drain()
-    for t in tables:
-        t.prof_reset()
-    t0 = time.perf_counter()
-    steps(args.warmup, args.warmup + args.steps)
-    drain()
-    dt = time.perf_counter() - t0
-    push_n, push_ms, push_s = kernel_stats(tables, capi.KERNEL_PUSH_SCALAR)
-    pull_st = kernel_stats(tables, capi.KERNEL_PULL_SCALAR)
-    same_st = kernel_stats(tables, capi.KERNEL_SAME_KEYS)
-    per_key_st = kernel_stats(tables, capi.KERNEL_PULL_PER_KEY)
-    for t in tables:
-        t.prof_enable(False)
+        def step(i):
+            # Kernel durations are sampled INSIDE the timed steps: in every SAMPLE_EVERY-th step the
+            # launches carry their own start/stop events (booked to the first table of the group; with
+            # one call per table those of one of the S tables, taken in turn). Events on every launch
+            # would cost more host time per step than the GPU needs for it.
+            if sample:
+                j = i - args.warmup
+                on = sampled(j, args.steps)
+                which = ((j // SAMPLE_EVERY) % S if per_table else 0) if on else -1
+                if which != prof_on[0]:
+                    for s_ in range(S):
+                        tables[s_].prof_enable(s_ == which)
+                    prof_on[0] = which
+            dk, dv = d_batches[i]
+            # Every step slices its keys, pushes and pulls, in line. (Slicing the keys of coming steps
+            # ahead of time, on this thread or on a second one, was measured and gains nothing: the
+            # slicer's short kernel shares the GPU with the store's long ones either way.)
+            pos, _, used = capi.slice_keys(dk, rb, re, nvals=n)
+            kp, vp, op = dk.data_ptr(), dv.data_ptr(), out.data_ptr()
+            if not per_table:
+                # one launch per step of the pipeline over all S key ranges
+                group.push_raw(kp, pos, vp, pos)
+                group.pull_raw(kp, pos, op)
+                return
+            pos = [int(x) for x in pos]
+            for s_ in range(S):
+                if used[s_]:
+                    c = pos[s_ + 1] - pos[s_]
+                    tables[s_].push_raw(kp + 8 * pos[s_], c, vp + 4 * pos[s_], c)
+            for s_ in range(S):
+                if used[s_]:
+                    c = pos[s_ + 1] - pos[s_]
+                    tables[s_].pull_raw(kp + 8 * pos[s_], c, op + 4 * pos[s_], c)
 
-    # last pull must hold exactly the pushed values: each key was pushed once (0.0f + v)
-    last = args.warmup + args.steps - 1
-    want = batches[last][1] + np.float32(0.0)
-    got = out.cpu().numpy()
-    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "pulled values differ"
-    held = sum(t.size()[0] for t in tables)
-    assert held == n * (args.warmup + args.steps), (held, n * (args.warmup + args.steps))
+        def drain():
+            if per_table:
+                for t in tables:
+                    t.sync()
+            else:
+                group.sync()
+            torch.cuda.synchronize()
 
-    # On request, the same timed steps once more on fresh tables that keep the library's default
-    # of one stream per table: kernels of different key ranges then overlap, so whole-job
-    # throughput is higher, but a kernel's duration is no longer its own, which is why the
-    # headline figures come from the shared-stream run (and why this pass is not part of the
-    # default command, whose kernel statistics a profiler run is compared with).
-    dt_own = None
-    if args.own_streams:
-        own = [capi.Table(capi.MODE_SCALAR, initial_capacity=cap) for _ in range(S)]
-        shared, tables = tables, own
-        was_per_table, per_table = per_table, True  # tables with streams of their own go one by one
-        steps(0, args.warmup, sample=False)
+        for i in range(args.warmup):
+            step(i)
         drain()
-        t1 = time.perf_counter()
-        steps(args.warmup, args.warmup + args.steps, sample=False)
+        for t in tables:
+            t.prof_reset()
+        t0 = time.perf_counter()
+        for i in range(args.warmup, total_steps):
+            step(i)
         drain()
-        dt_own = time.perf_counter() - t1
-        assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32)), "pulled values differ"
-        for t in own:
-            t.close()
-        tables, per_table = shared, was_per_table
-    # The same steps once more on tables that start at the library's default size and grow
-    # (allocate twice the slots, re-insert everything) while the clock runs, as the CPU's
-    # std::unordered_map does inside its own timing.
-    growing = None
-    if not args.no_extra and not per_table:
-        main_group, main_tables = group, tables
-        group = capi.Group(S, capi.MODE_SCALAR, stream=stream.cuda_stream)
-        tables = group.tables
-        steps(0, args.warmup, sample=False)
-        drain()
-        t2 = time.perf_counter()
-        steps(args.warmup, args.warmup + args.steps, sample=False)
-        drain()
-        dt_grow = time.perf_counter() - t2
-        assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32)), "pulled values differ"
-        growing = {"value": 2.0 * n * args.steps / dt_grow, "unit": "keys/s",
-                   "ms_per_step": dt_grow / args.steps * 1e3,
-                   "note": "same steps on tables created with the default capacity (1M keys each, %d keys "
-                           "held at the end): they grow inside the timed steps" % sum(t.size()[0] for t in tables)}
-        group.close()
-        group, tables = main_group, main_tables
-    # the slicer alone on an idle GPU: two small launches and one read-back of S+1 positions
-    t_s = time.perf_counter()
-    for _ in range(50):
-        capi.slice_keys(d_batches[0][0], rb, re, nvals=n)
-    slice_us = (time.perf_counter() - t_s) / 50 * 1e6
+        dt = time.perf_counter() - t0
+        st = {"push": kernel_stats(tables, capi.KERNEL_PUSH_SCALAR),
+              "pull": kernel_stats(tables, capi.KERNEL_PULL_SCALAR),
+              "same": kernel_stats(tables, capi.KERNEL_SAME_KEYS),
+              "per_key": kernel_stats(tables, capi.KERNEL_PULL_PER_KEY),
+              "growth": kernel_stats(tables, capi.KERNEL_REHASH)}
+        for t in tables:
+            t.prof_enable(False)
+        # the last pull must hold exactly the pushed values, the tables every key of the run
+        got = out.cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "pulled values differ"
+        held = sum(t.size()[0] for t in tables)
+        assert held == n * total_steps, (held, n * total_steps)
+        if group is not None:
+            group.close()
+        else:
+            for t in tables:
+                t.close()
+        return dt, st, held
+
+    per_table = args.per_table
+    cap_presized = int(n * (args.warmup + 2 * args.steps) / S * 1.1)
+    # THE measured run: tables created with the library's defaults (room for 1M keys each), which
+    # grow while the clock runs, as the std::unordered_map of the reference's handle does (kv_app.h:462)
+    dt, st, held = measure(0, per_table, True)
     keys_per_launch = n / S if per_table else n
     res = {
         "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
         "dtype": "f32",
         "config": {"workload": "sparse_lr: 1M sorted unique uint64 keys/step over 4 key ranges, "
-                               "push then pull, store grows by 1M keys/step", "keys_per_step": n,
+                               "push then pull, store grows by 1M keys/step; tables created with the "
+                               "default capacity, their growths inside the timed steps", "keys_per_step": n,
                    "ranges": S, "value_len": 1, "key_dtype": "u64",
                    "store_keys_after_timed_steps": held,
                    "launches": "one launch per table" if per_table else
                                "one launch over all %d key ranges (pskv_push_multi / pskv_pull_multi)" % S},
         # every pushed key is new: 8 key + 4 val in, 8 slot read, 8 key + 4 val written
-        "roofline": dict(roofline(32.0 * keys_per_launch, push_n, push_ms,
-                                  traffic("push_scalar", keys_per_launch), push_s),
+        "roofline": dict(roofline(32.0 * keys_per_launch, st["push"][0], st["push"][1],
+                                  traffic("push_scalar", keys_per_launch), st["push"][2]),
                          kernel="k_scalar<push> (find-or-insert + add)", bytes_per_key=32),
-        "kernels": dict(pull_entries(keys_per_launch, pull_st, same_st, per_key_st,
+        "kernels": dict(pull_entries(keys_per_launch, st["pull"], st["same"], st["per_key"],
                                      traffic("pull_scalar", keys_per_launch),
                                      traffic("pull_per_key", keys_per_launch)),
-                        slicer={"wall_us_per_call": round(slice_us, 1), "keys": n, "ranges": S}),
+                        growth={"launches": st["growth"][0], "total_us": round(st["growth"][1] * 1e3, 1),
+                                "note": "k_regrow + k_regrow_rest of the sampled steps only"}),
     }
-    if dt_own is not None:
+    if not args.no_extra:
+        # the same steps on tables sized up front for every key of the run (no growth, lower fill)
+        dt_p, st_p, _ = measure(cap_presized, per_table, True)
+        res["presized"] = {"value": 2.0 * n * args.steps / dt_p, "unit": "keys/s",
+                           "ms_per_step": dt_p / args.steps * 1e3,
+                           "push_kernel": roofline(32.0 * keys_per_launch, st_p["push"][0], st_p["push"][1],
+                                                   traffic("push_scalar", keys_per_launch), st_p["push"][2]),
+                           "note": "same steps on tables created with room for %d keys each: no growth "
+                                   "inside the timed steps, fill below 0.2" % cap_presized}
+        # ... and with one call per table, which is what S separate KVServers on one GPU would issue
+        dt_t, _, _ = measure(0, not per_table, False)
+        res["per_table" if not per_table else "multi"] = {
+            "value": 2.0 * n * args.steps / dt_t, "unit": "keys/s", "ms_per_step": dt_t / args.steps * 1e3,
+            "note": "same steps, default-capacity tables, " +
+                    ("one pskv_push / pskv_pull per table" if not per_table else
+                     "one pskv_push_multi / pskv_pull_multi over all ranges")}
+    # On request, the same timed steps once more on fresh tables that keep the library's default
+    # of one stream per table: kernels of different key ranges then overlap, so whole-job
+    # throughput is higher, but a kernel's duration is no longer its own, which is why the
+    # headline figures come from the shared-stream run.
+    if args.own_streams:
+        dt_own, _, _ = measure(0, True, False, own_streams=True)
         res["own_streams"] = {"value": 2.0 * n * args.steps / dt_own, "unit": "keys/s",
                               "ms_per_step": dt_own / args.steps * 1e3,
                               "note": "same steps, one stream per table (kernels of different ranges overlap)"}
-    if growing is not None:
-        res["growing_tables"] = growing
+    # the slicer alone on an idle GPU: one launch and one read-back of S+1 positions
+    t_s = time.perf_counter()
+    for _ in range(50):
+        capi.slice_keys(d_batches[0][0], rb, re, nvals=n)
+    slice_us = (time.perf_counter() - t_s) / 50 * 1e6
+    res["kernels"]["slicer"] = {"wall_us_per_call": round(slice_us, 1), "keys": n, "ranges": S}
     return res, batches[args.warmup:args.warmup + args.steps], (n, S)
 
 
@@ -395,14 +387,13 @@ def cpu_sparse_lr(orc, batches, n, S, budget_s=25.0):
     return {"value": 2.0 * n * done / dt, "unit": "keys/s", "cores": 1, "kind": "port",
             "sample": "first %d of the timed steps (slice + push + pull of %d keys each), "
                       "std::unordered_map store per range, one thread; the maps start empty and rehash as "
-                      "they grow inside this timing, whereas the GPU tables of `value` are sized up front "
-                      "(extra.growing_tables is the GPU run whose tables grow inside the timing too)" % (done, n)}
+                      "they grow inside this timing, as the GPU tables of `value` do" % (done, n)}
 
 
 # ------------------------------------------------------------------------------------
 # dense: configs[2]
 # ------------------------------------------------------------------------------------
-def measure_dense(capi, dev, steps, warmup, nk=64, k=4194304):
+def measure_dense(capi, dev, steps, warmup, nk=64, k=4194304, every_step=False):
     """Returns (seconds for `steps` push+pull steps, accumulate stats, gather stats)."""
     import torch
     keys = to_dev(np.uint64(KMAX // nk) * np.arange(nk, dtype=np.uint64), dev)
@@ -422,7 +413,7 @@ def measure_dense(capi, dev, steps, warmup, nk=64, k=4194304):
     t.prof_reset()
     t0 = time.perf_counter()
     for i in range(steps):
-        t.prof_enable(sampled(i, steps))
+        t.prof_enable(every_step or sampled(i, steps))  # (15 us of events next to 500 us kernels)
         t.push(keys, vals)
         t.pull(keys, out)
     t.sync()
@@ -468,7 +459,7 @@ def run_dense(args, capi, dev):
     return res
 
 
-def cpu_dense(orc, nk=64, k=4194304, sample_keys=16):
+def cpu_dense(orc, nk=64, k=4194304, sample_keys=16, budget_s=10.0):
     rng = np.random.default_rng(0xD15E)
     keys = (np.uint64(KMAX // nk) * np.arange(sample_keys, dtype=np.uint64))
     vals = rng.uniform(-1, 1, size=sample_keys * k).astype(np.float32)
@@ -476,7 +467,7 @@ def cpu_dense(orc, nk=64, k=4194304, sample_keys=16):
     st.push(keys, vals)
     t0 = time.perf_counter()
     reps = 0
-    while reps < 3 or time.perf_counter() - t0 < 10.0:
+    while reps < 3 or time.perf_counter() - t0 < budget_s:
         st.push(keys, vals)
         st.handle(False, True, keys, out_cap=vals.size)
         reps += 1
@@ -667,88 +658,159 @@ def cpu_varlen(orc, keys, lens, nvals, n, S, budget_s=15.0):
 # ------------------------------------------------------------------------------------
 # zipf: configs[3]
 # ------------------------------------------------------------------------------------
-def zipf_unique_keys(rng, n, universe, s=1.1):
-    """n distinct keys whose ranks in [0, universe) have Zipf(s) popularity, sorted. A rank
-    becomes a key through an injective scatter over the covered key space."""
-    got = np.zeros(0, np.int64)
-    while got.size < n:
-        r = rng.zipf(s, size=2 * n).astype(np.int64) - 1
-        got = np.unique(np.concatenate([got, r[(r >= 0) & (r < universe)]]))
-    if got.size > n:
-        got = np.sort(rng.choice(got, size=n, replace=False))
-    keys = (got.astype(np.uint64) * np.uint64(0x9E3779B97F4A7C15)) >> np.uint64(1)
-    return np.sort(keys)
+_zipf_weights = {}
 
 
-def run_zipf(args, capi, dev):
-    """A step is one worker's push of 4M Zipf-popular keys (a growing share of them already
-    stored) followed by a pull of the same keys; one table, which grows (and rehashes) inside
-    the timed region as it would in service."""
+def zipf_distinct_ranks(rng, n, universe, s=1.1):
+    """The n distinct ranks of [0, universe) that a long run of Zipf(s) draws over the universe
+    names, sorted. Drawing rank after rank until n distinct ones have come up takes about 45
+    draws per key at these sizes (minutes of host time for the 16M-key pull); the shortcut: D
+    draws name rank k at least once with probability 1 - exp(-D p_k), independently for every k
+    when the number of draws is Poisson, so one exponential variate per rank, compared with
+    D p_k, gives the set of named ranks directly. D is aimed so that about n ranks come up; the
+    set is then thinned at random, or topped up with further draws by popularity, to exactly n."""
+    key = (universe, s)
+    if key not in _zipf_weights:
+        w = np.power(np.arange(1, universe + 1, dtype=np.float32), np.float32(-s))
+        _zipf_weights.clear()
+        _zipf_weights[key] = (w / np.float32(w.sum(dtype=np.float64)), np.cumsum(w[::1024], dtype=np.float64))
+    p, _ = _zipf_weights[key]
+    sub = p[::97].astype(np.float64)  # the expected count on a thinned copy is close enough to aim with
+    lo, hi = 1.0, 1e13
+    for _ in range(60):
+        d = (lo * hi) ** 0.5
+        if (1.0 - np.exp(-d * sub)).sum() * 97 < n * 1.002:
+            lo = d
+        else:
+            hi = d
+    e = rng.standard_exponential(universe, dtype=np.float32)
+    ranks = np.flatnonzero(e < np.float32(hi) * p)
+    del e
+    while ranks.size < n:
+        more = (rng.zipf(s, size=4 * (n - ranks.size) + 1024) - 1)
+        ranks = np.unique(np.concatenate([ranks, more[(more >= 0) & (more < universe)]]))
+    if ranks.size > n:
+        ranks = np.sort(rng.choice(ranks, size=n, replace=False))
+    return ranks
+
+
+def rank_to_key(ranks):
+    """An injective scatter of ranks over the covered key space (odd multiplier mod 2^64, then >> 1)."""
+    return (ranks.astype(np.uint64) * np.uint64(0x9E3779B97F4A7C15)) >> np.uint64(1)
+
+
+def gen_zipf(pushes, n_push, n_pull, universe):
+    """The inputs of configs[3]: `pushes` worker requests of n_push distinct Zipf(1.1)-popular keys
+    with N(0,1) values, and the n_pull distinct Zipf-popular keys of the pull."""
+    batches = []
+    for w in range(pushes):
+        rng = np.random.default_rng(0x21F + w)
+        keys = np.sort(rank_to_key(zipf_distinct_ranks(rng, n_push, universe)))
+        batches.append((keys, rng.standard_normal(n_push).astype(np.float32)))
+    rng = np.random.default_rng(0x9011)
+    probe = np.sort(rank_to_key(zipf_distinct_ranks(rng, n_pull, universe)))
+    _zipf_weights.clear()  # (400 MB)
+    return batches, probe
+
+
+def run_zipf(args, capi, dev, pushes=8):
+    """configs[3] as it stands: 8 worker pushes of 4M distinct Zipf-popular keys each into one table
+    (a growing share of every push is already stored), applied in order, then ONE pull of 16M
+    distinct Zipf-popular keys, most of which the store has never seen and which the pull inserts
+    with value 0 (kv_app.h:456-458). The table starts at the default capacity and grows inside the
+    timed region as it would in service. The clock covers the 8 pushes and the pull."""
     import torch
     n, universe = args.keys or 4000000, 100000000
-    total = args.warmup + args.steps
-    log("generating %d Zipf batches of %d keys" % (total, n))
-    batches = []
-    for w in range(total):
-        rng = np.random.default_rng(0x21F + w)
-        batches.append((zipf_unique_keys(rng, n, universe), rng.standard_normal(n).astype(np.float32)))
+    n_pull = 4 * n
+    log("generating %d Zipf batches of %d keys and a pull of %d" % (pushes, n, n_pull))
+    batches, probe = gen_zipf(pushes, n, n_pull, universe)
     d_batches = [(to_dev(k, dev), to_dev(v, dev)) for k, v in batches]
-    out = torch.empty(n, dtype=torch.float32, device=dev)
-    t = capi.Table(capi.MODE_SCALAR, initial_capacity=1 << 20)
-    t.prof_enable(True)  # one launch per request: per-launch events cost nothing that matters here
-
-    def step(i):
-        dk, dv = d_batches[i]
-        t.push(dk, dv)
-        t.pull(dk, out)
-
-    for i in range(args.warmup):
-        step(i)
-    t.sync()
-    t.prof_reset()
+    d_probe = to_dev(probe, dev)
+    out = torch.empty(n_pull, dtype=torch.float32, device=dev)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.warmup, total):
-        step(i)
-    t.sync()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+
+    def once(prof):
+        t = capi.Table(capi.MODE_SCALAR)
+        t.prof_enable(prof)  # one launch per request: per-launch events cost nothing that matters here
+        t.sync()
+        t0 = time.perf_counter()
+        for dk, dv in d_batches:
+            t.push(dk, dv)
+        t.sync()
+        t1 = time.perf_counter()
+        t.pull(d_probe, out)
+        t.sync()
+        t2 = time.perf_counter()
+        return t, t1 - t0, t2 - t1
+
+    for _ in range(max(1, min(args.warmup, 2))):  # whole runs on tables of their own: the first one loads the code
+        t, _, _ = once(False)
+        t.close()
+    t, dt_push, dt_pull = once(True)
     push = kernel_stats([t], capi.KERNEL_PUSH_SCALAR)
     pull = kernel_stats([t], capi.KERNEL_PULL_SCALAR)
-    same = kernel_stats([t], capi.KERNEL_SAME_KEYS)
-    per_key = kernel_stats([t], capi.KERNEL_PULL_PER_KEY)
     rehash = kernel_stats([t], capi.KERNEL_REHASH)
     held = t.size()[0]
+    everything = np.unique(np.concatenate([k for k, _ in batches] + [probe]))
+    assert held == everything.size, (held, everything.size)
+    # spot check against sequential float adds in push order: 4096 pulled keys
+    pick = np.random.default_rng(5).choice(n_pull, size=4096, replace=False)
+    want = np.zeros(4096, np.float32)
+    for keys, vals in batches:
+        at = np.minimum(np.searchsorted(keys, probe[pick]), keys.size - 1)
+        hit = keys[at] == probe[pick]
+        want[hit] = want[hit] + vals[at[hit]]
+    got = out.cpu().numpy()[pick]
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "pulled values differ"
+    stored_before = np.unique(np.concatenate([k for k, _ in batches]))
+    missing = n_pull - int(np.isin(probe, stored_before, assume_unique=True).sum())
+    t.close()
+    dt = dt_push + dt_pull
+    total_keys = pushes * n + n_pull
     res = {
-        "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
+        "value": total_keys / dt, "unit": "keys/s", "ms_per_step": dt / pushes * 1e3,
         "dtype": "f32",
-        "config": {"workload": "zipf: pushes of 4M distinct Zipf(1.1)-popular keys from a 100M-key "
-                               "universe into one table, each followed by a pull of the same keys",
-                   "keys_per_step": n, "ranges": 1, "value_len": 1, "key_dtype": "u64",
-                   "store_keys_after_timed_steps": held},
+        "config": {"workload": "zipf: %d pushes of 4M distinct Zipf(1.1)-popular keys from a 100M-key universe "
+                               "into one table that starts at the default capacity, then one pull of 16M "
+                               "distinct Zipf-popular keys (%d of them absent: inserted with value 0); a step "
+                               "is one push, the pull's time is spread over the steps" % (pushes, missing),
+                   "keys_per_step": n, "pull_keys": n_pull, "pull_keys_absent": missing, "ranges": 1,
+                   "value_len": 1, "key_dtype": "u64", "store_keys_at_the_end": held},
+        "phases": {"pushes_ms": dt_push * 1e3, "pull_ms": dt_pull * 1e3,
+                   "push_keys_per_s": pushes * n / dt_push, "pull_keys_per_s": n_pull / dt_pull},
+        # a pulled key that is absent: 8 key in, 8 slot read, 8 key written, 4 out = 28 B/key; the present
+        # ones read the value instead of writing the key: 24 B/key; priced as misses
+        "roofline": dict(roofline(28.0 * n_pull, pull[0], pull[1], traffic("pull_miss_insert", n_pull), pull[2]),
+                         kernel="k_scalar<pull> (find, or insert 0, then answer), %d of %d keys absent" % (missing, n_pull),
+                         bytes_per_key=28),
         # between a hit (28 B/key) and an insert (32 B/key); priced as inserts
-        "roofline": dict(roofline(32.0 * n, push[0], push[1], None, push[2]),
-                         kernel="k_scalar<push> (find-or-insert + add)", bytes_per_key=32),
-        "kernels": dict(pull_entries(n, pull, same, per_key, None),
-                        rehash={"launches": rehash[0], "total_us": round(rehash[1] * 1e3, 1)}),
+        "kernels": {"push_scalar": dict(roofline(32.0 * n, push[0], push[1], traffic("push_scalar_zipf", n), push[2]),
+                                        kernel="k_scalar<push> (find-or-insert + add), 4M keys", bytes_per_key=32),
+                    "growth": {"launches": rehash[0], "total_us": round(rehash[1] * 1e3, 1),
+                               "kernels": "k_regrow + k_regrow_rest per growth"}},
     }
-    return res, batches[args.warmup:], n
+    return res, (batches, probe)
 
 
-def cpu_zipf(orc, batches, n, budget_s=25.0):
+def cpu_zipf(orc, batches, probe, budget_s=25.0):
     store = orc.Store(orc.MODE_SCALAR)
     done = 0
     t0 = time.perf_counter()
     for keys, vals in batches:
         store.push(keys, vals)
-        store.handle(False, True, keys, out_cap=n)
-        done += 1
+        done += keys.size
         if time.perf_counter() - t0 > budget_s:
             break
+    pulled = False
+    if done == sum(k.size for k, _ in batches):
+        store.handle(False, True, probe, out_cap=probe.size)
+        done += probe.size
+        pulled = True
     dt = time.perf_counter() - t0
-    return {"value": 2.0 * n * done / dt, "unit": "keys/s", "cores": 1, "kind": "port",
-            "sample": "first %d of the timed steps (push + pull of %d keys each), one "
-                      "std::unordered_map store, one thread" % (done, n)}
+    return {"value": done / dt, "unit": "keys/s", "cores": 1, "kind": "port",
+            "sample": "%s on one std::unordered_map store, one thread" % (
+                "the same %d pushes and the pull of %d keys" % (len(batches), probe.size) if pulled else
+                "the pushes that fit %d s (%d keys), without the pull" % (budget_s, done))}
 
 
 # ------------------------------------------------------------------------------------
@@ -1020,6 +1082,100 @@ def cpu_match(orc, src_keys, src_vals, dst_keys, dst_vals, budget_s=15.0):
                       "binding copies the destination values once per call)" % done}
 
 
+# ------------------------------------------------------------------------------------
+# Side measurements of the default run: the other BASELINE configurations, each with the CPU
+# oracle on the same inputs beside it
+# ------------------------------------------------------------------------------------
+def extra_plumbing(capi, orc, reps=5):
+    """configs[0], the shape of the reference's own test (tests/test_kv_app.cc:27-60) through the
+    calls a ps-lite worker and server make: 1,000 keys kMaxKey/1000*i with values 1.0, one server
+    range; 50 times slice + push, then slice + pull, everything from and to ordinary host memory
+    (PSKV_MEM_HOST). Wall time per request (a request = its slice and its handle call), the
+    oracle's slicer and handle on the same arrays beside it."""
+    num, S, pushes = 1000, 1, 50
+    keys = np.uint64(KMAX // num) * np.arange(num, dtype=np.uint64)
+    vals = np.ones(num, np.float32)
+    out = np.zeros(num, np.float32)
+    rb, re = capi.server_ranges(S)
+    walls = []
+    for rep in range(reps + 1):  # the first run loads the GPU code and is not counted
+        t = capi.Table(capi.MODE_SCALAR)
+        t0 = time.perf_counter()
+        for _ in range(pushes):
+            capi.slice_keys(keys, rb, re, nvals=num)
+            t.push(keys, vals)
+        capi.slice_keys(keys, rb, re, nvals=0)
+        t.pull(keys, out)
+        walls.append(time.perf_counter() - t0)
+        assert np.all(out == np.float32(pushes)), "pull differs from 50 * v"
+        t.close()
+    walls = np.array(walls[1:])
+    orb, ore = orc.server_ranges(S)
+    cpu_walls = []
+    for rep in range(reps):
+        st = orc.Store(orc.MODE_SCALAR)
+        t0 = time.perf_counter()
+        for _ in range(pushes):
+            orc.slice_keys(keys, orb, ore, nvals=num)
+            st.push(keys, vals)
+        orc.slice_keys(keys, orb, ore, nvals=0)
+        got = st.handle(False, True, keys, out_cap=num)
+        cpu_walls.append(time.perf_counter() - t0)
+    cpu_walls = np.array(cpu_walls)
+    return {"workload": "plumbing: 1,000 keys, 50 x (slice + push) then slice + pull, one key range, host "
+                        "buffers through pskv_slice / pskv_push / pskv_pull (PSKV_MEM_HOST)",
+            "requests": pushes + 1, "wall_ms": round(float(np.median(walls)) * 1e3, 3),
+            "us_per_request": round(float(np.median(walls)) / (pushes + 1) * 1e6, 2),
+            "min_us_per_request": round(float(walls.min()) / (pushes + 1) * 1e6, 2),
+            "keys_per_s": num * (pushes + 1) / float(np.median(walls)),
+            "cpu_baseline": {"us_per_request": round(float(np.median(cpu_walls)) / (pushes + 1) * 1e6, 2),
+                             "keys_per_s": num * (pushes + 1) / float(np.median(cpu_walls)), "cores": 1,
+                             "kind": "port", "sample": "the same 51 requests through the oracle's slicer and "
+                                                       "std::unordered_map handle (ctypes calls included on "
+                                                       "both sides), median of %d runs" % reps}}
+
+
+def extra_host_staged(capi, reps=2, nk=64, k=4194304):
+    """configs[2] from and to ordinary (pageable) host memory, as a server gets it from the
+    transport: 1 GiB per push and per pull through PSKV_MEM_HOST. PCIe-inclusive, never `value`."""
+    keys = np.uint64(KMAX // nk) * np.arange(nk, dtype=np.uint64)
+    vals = np.full(nk * k, 0.5, np.float32)
+    out = np.empty(nk * k, np.float32)
+    out[::1024] = 0  # (touch the pages)
+    t = capi.Table(capi.MODE_FIXED, initial_capacity=1024, row_len=k, arena_floats=nk * k)
+    t.push(keys, vals)  # creates the rows; also warms the staging ring
+    push_s, pull_s = [], []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        t.push(keys, vals)
+        t1 = time.perf_counter()
+        t.pull(keys, out)
+        t2 = time.perf_counter()
+        push_s.append(t1 - t0)
+        pull_s.append(t2 - t1)
+    assert out[12345] == np.float32(0.5 * (reps + 1)) and out[-1] == np.float32(0.5 * (reps + 1))
+    t.close()
+    gib = nk * k * 4 / 1e9
+    return {"workload": "dense from host memory: 64 keys x 4,194,304 f32 (1 GiB) pushed from and pulled "
+                        "into ordinary host memory, PCIe-inclusive",
+            "push_gb_per_s": round(gib / min(push_s), 2), "pull_gb_per_s": round(gib / min(pull_s), 2),
+            "push_ms": round(min(push_s) * 1e3, 2), "pull_ms": round(min(pull_s) * 1e3, 2),
+            "note": "best of %d; inside this Python process the HIP runtime that torch brings serves the "
+                    "library, whose device-to-pinned copies block the calling thread: a C++ server gets "
+                    "about twice this pull rate" % reps}
+
+
+def brief(res, cpu=None):
+    """What an `extra` entry keeps of a workload's result."""
+    out = {k: res[k] for k in ("value", "unit", "ms_per_step", "gbps", "phases") if k in res}
+    out["workload"] = res["config"]["workload"]
+    out["roofline"] = res["roofline"]
+    out["kernels"] = res.get("kernels")
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
+    return out
+
+
 def main():
     global SAMPLE_EVERY
     ap = argparse.ArgumentParser()
@@ -1056,9 +1212,8 @@ def main():
     elif args.workload == "dense":
         res = run_dense(args, capi, dev)
     elif args.workload == "zipf":
-        if args.steps == 20:
-            args.steps = 8  # the configuration has 8 worker pushes
-        res, zipf_batches, zipf_n = run_zipf(args, capi, dev)
+        args.steps = 8  # the configuration is 8 worker pushes and a pull
+        res, zipf_inputs = run_zipf(args, capi, dev)
     elif args.workload == "sparse_repeat":
         res, repeat_inputs = run_sparse_repeat(args, capi, dev)
     elif args.workload == "match":
@@ -1069,11 +1224,14 @@ def main():
         res, varlen_inputs = run_varlen(args, capi, dev)
 
     extra = {}
+    orc = None if args.no_cpu else graft.load_oracle()
     if args.workload == "sparse_lr" and not args.no_extra:
         # the dense-chunk kernels carry the bandwidth target of this path; measure them
-        # beside the default workload (10 push+pull steps of 1 GiB, well under a second)
-        dt, acc, gat, cp, nk, k = measure_dense(capi, dev, 10, 2)
+        # beside the default workload (12 push+pull steps of 1 GiB, every launch timed)
+        dt, acc, gat, cp, nk, k = measure_dense(capi, dev, 12, 2, every_step=True)
         extra["dense_chunk"] = {
+            "workload": "dense: 64 keys x 4,194,304 f32 (1 GiB), push-accumulate then full pull, 12 steps",
+            "value": 20.0 * nk * k * 12 / dt / 1e9, "unit": "GB/s", "ms_per_step": dt / 12 * 1e3,
             "rows_acc": dict(roofline(12.0 * nk * k, acc[0], acc[1], traffic("rows_acc_fixed", nk * k), acc[2]),
                              bytes_per_float=12),
             "rows_gather": dict(roofline(8.0 * nk * k, gat[0], gat[1],
@@ -1081,10 +1239,25 @@ def main():
             "copy_ceiling": dict(roofline(8.0 * nk * k, cp[0], cp[1], 8.0 * nk * k, cp[2]),
                                  kernel="k_copy (plain copy of 1 GiB)"),
         }
+        if orc is not None:
+            extra["dense_chunk"]["cpu_baseline"] = cpu_dense(orc, budget_s=3.0)
+        extra["host_staged"] = extra_host_staged(capi)
+        sub = argparse.Namespace(**vars(args))
+        sub.steps, sub.warmup, sub.keys, sub.per_table, sub.own_streams = 10, 2, 0, False, False
+        log("extra: varlen")
+        vres, vin = run_varlen(sub, capi, dev)
+        extra["varlen"] = brief(vres, cpu_varlen(orc, *vin, budget_s=4.0) if orc is not None else None)
+        del vin
+        log("extra: zipf")
+        zres, zin = run_zipf(sub, capi, dev)
+        extra["zipf"] = brief(zres, cpu_zipf(orc, *zin, budget_s=12.0) if orc is not None else None)
+        del zin
+        if orc is not None:
+            log("extra: plumbing")
+            extra["plumbing"] = extra_plumbing(capi, orc)
 
     cpu = None
     if not args.no_cpu:
-        orc = graft.load_oracle()
         log("timing the CPU oracle (bounded sample)")
         if args.workload == "sparse_lr":
             cpu = cpu_sparse_lr(orc, timed_batches, n, S)
@@ -1092,7 +1265,7 @@ def main():
             cpu = cpu_dense(orc)
             extra["cpu_baseline_all_cores"] = cpu_dense_all_cores(orc)
         elif args.workload == "zipf":
-            cpu = cpu_zipf(orc, zipf_batches, zipf_n)
+            cpu = cpu_zipf(orc, *zipf_inputs)
         elif args.workload == "sparse_repeat":
             cpu = cpu_sparse_repeat(orc, *repeat_inputs)
         elif args.workload == "match":
@@ -1116,10 +1289,11 @@ def main():
         "kernel; read at run time from " + ", ".join(sorted(TRAFFIC_SOURCES))) if TRAFFIC_SOURCES else None
     if "gbps" in res:
         line["gbps"] = res["gbps"]
-    if "own_streams" in res:
-        extra["own_streams"] = res["own_streams"]
-    if "growing_tables" in res:
-        extra["growing_tables"] = res["growing_tables"]
+    for k in ("own_streams", "presized", "per_table", "multi"):
+        if k in res:
+            extra[k] = res[k]
+    if "phases" in res:
+        line["phases"] = res["phases"]
     if extra:
         line["extra"] = extra
     print(json.dumps(line, allow_nan=False), flush=True)  # strict JSON: a NaN would be a bug

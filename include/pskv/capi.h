@@ -20,9 +20,10 @@
  *    until pskv_sync(). Input buffers written by other streams must be complete
  *    before the call. Calls with PSKV_MEM_HOST buffers return when the caller's
  *    buffers are the caller's again: inputs have been read, responses are in place.
- *    (A pure push of a PSKV_MODE_SCALAR table that fits the pinned request buffer,
- *    1 MiB, has nothing to hand back and returns once its kernel is queued; later
- *    requests follow it in call order, pskv_sync() waits for it.)
+ *    (A pure push of a PSKV_MODE_SCALAR table of up to 128 KiB of keys and values, about
+ *    10,000 keys, has nothing to hand back and returns once its input has been copied to
+ *    pinned memory and its kernel is queued; up to eight such pushes are in flight at a
+ *    time, later requests follow them in call order, pskv_sync() waits for them.)
  *  - Keys within one request must be unique (ps-lite requires sorted unique
  *    keys, include/ps/kv_app.h:17); requests on one table are applied in call
  *    order. A SORTED request that repeats a key: the row modes refuse it as a whole with

@@ -311,25 +311,44 @@ __device__ __forceinline__ uint64_t* find_or_insert(Slot* __restrict__ slots, ui
     return reinterpret_cast<uint64_t*>(&st->special_payload);
   }
   uint64_t h = home_slot(key, mask);
-  for (uint64_t probes = 0; probes <= mask; ++probes) {
-    const u64x2 s = load_slot(&slots[h]);
+  // Tries to settle the key at slot `at`, whose contents `s` were read a moment ago: 1 = found,
+  // 2 = claimed, 0 = the slot belongs to another key.
+  auto settle = [&](uint64_t at, const u64x2& s) -> int {
     if (s.x == key) {
       seen = s.y;
-      return &slots[h].payload;
+      return 1;
     }
     if (s.x == kEmptyKey) {
-      unsigned long long old = atomicCAS(reinterpret_cast<unsigned long long*>(&slots[h].key),
+      unsigned long long old = atomicCAS(reinterpret_cast<unsigned long long*>(&slots[at].key),
                                          (unsigned long long)kEmptyKey, (unsigned long long)key);
       if (old == kEmptyKey) {
         is_new = true;
-        return &slots[h].payload;
+        return 2;
       }
       if (old == key) {  // same key twice in one request: undefined for callers, but stay sane
-        seen = slots[h].payload;
-        return &slots[h].payload;
+        seen = slots[at].payload;
+        return 1;
       }
     }
-    h = (h + 1) & mask;
+    return 0;
+  };
+  // The home slot alone first: at the fills this table runs at, most keys are settled there, and
+  // one load per lane keeps the most wavefronts in flight. A key that has to walk on asks for the
+  // next three slots at once (a walk of one slot per round trip made a push a tenth slower at a
+  // fill of 0.4 than at 0.1).
+  {
+    const u64x2 s = load_slot(&slots[h]);
+    if (settle(h, s)) return &slots[h].payload;
+  }
+  for (uint64_t probes = 0; probes <= mask; probes += 3) {
+    const uint64_t h1 = (h + 1) & mask, h2 = (h + 2) & mask, h3 = (h + 3) & mask;
+    const u64x2 s1 = load_slot(&slots[h1]);
+    const u64x2 s2 = load_slot(&slots[h2]);
+    const u64x2 s3 = load_slot(&slots[h3]);
+    if (settle(h1, s1)) return &slots[h1].payload;
+    if (settle(h2, s2)) return &slots[h2].payload;
+    if (settle(h3, s3)) return &slots[h3].payload;
+    h = h3;
   }
   atomicOr(&st->error, kDevErrFull);
   return nullptr;

@@ -299,6 +299,7 @@ struct SliceCtx {
 // a few hundred of them, and the sums one pass, straight from pinned host memory.
 constexpr size_t kSmallStage = 1024u << 10;
 
+
 std::mutex g_pool_mu;
 std::vector<SliceCtx*> g_pool;
 
@@ -419,23 +420,47 @@ int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, 
   }
   const bool has_lens = lens != nullptr && nlens != 0;
 
-  if (n) {
+  const bool do_sums = has_lens && nlens == n;
+  if (n && do_sums && S > 65535) return set_error(PSKV_EINVAL, "more than 65535 ranges with lens");
+  bool sums_on_device = n != 0;  // (device-resident requests: searches and sums on the GPU)
+  if (n && memkind == PSKV_MEM_HOST) {
+    // Keys in host memory are searched where they lie: S+1 lower bounds touch (S+1) log2 n keys,
+    // and shipping all n keys over the host link for that would cost milliseconds at model size
+    // (and a launch and a wait at any size). This is the reference's own loop (kv_app.h:524-541).
+    const uint64_t* begin = keys;
+    const uint64_t* end = keys + n;
+    for (size_t i = 0; i < S; ++i) {
+      if (i == 0) {
+        pos[0] = (uint64_t)(std::lower_bound(begin, end, range_begin[0]) - begin);
+        begin += pos[0];
+      }
+      const size_t len = (size_t)(std::lower_bound(begin, end, range_end[i]) - begin);
+      begin += len;
+      pos[i + 1] = pos[i] + len;
+    }
+    // The lens too: one core adds them up faster (8 MB in 0.2 ms) than pageable memory crosses the
+    // host link (0.28 ms for the same 8 MB, before any kernel runs): the walk of kv_app.h:563-565.
+    sums_on_device = false;
+    if (do_sums) {
+      for (size_t i = 0; i < S; ++i) {
+        uint64_t sum = 0;
+        for (uint64_t j = pos[i]; j < pos[i + 1]; ++j) sum += (uint64_t)(int64_t)lens[j];
+        val_pos[i + 1] = sum;  // per-slice sums for now
+      }
+    }
+  }
+
+  if (sums_on_device) {
     DeviceGuard guard(device);
     if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", device);
     CtxLease lease(device);
     SliceCtx* c = lease.c;
     if (!c) return set_error(PSKV_EHIP, "cannot create a slicer context on device %d", device);
     lease.idle = false;
-    const bool do_sums = has_lens && nlens == n;
-    if (do_sums && S > 65535) return set_error(PSKV_EINVAL, "more than 65535 ranges with lens");
     // device: lb[S+1] | pos[S+1] | sums[S]      pinned: targets[S+1] | pos[S+1] | sums[S]
     const size_t arr = pad256((S + 2) * 8);  // S+1 positions and the word that says they are there
-    const bool host = memkind == PSKV_MEM_HOST;
-    const size_t in_bytes = pad256(n * 8) + (do_sums ? pad256(n * 4) : 0);
-    const bool in_place = host && in_bytes <= kSmallStage;
-    int rc = ctx_reserve(c, 3 * arr, 3 * arr, host && !in_place ? in_bytes : 0);
+    int rc = ctx_reserve(c, 3 * arr, 3 * arr, 0);
     if (rc) return rc;
-    if (in_place && !c->small) PSKV_HIP(hipHostMalloc(&c->small, kSmallStage, hipHostMallocCoherent));
     char* d = static_cast<char*>(c->dev);
     uint64_t* d_lb = reinterpret_cast<uint64_t*>(d);
     uint64_t* d_pos = reinterpret_cast<uint64_t*>(d + arr);
@@ -444,23 +469,7 @@ int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, 
     uint64_t* h_targets = reinterpret_cast<uint64_t*>(h);
     uint64_t* h_pos = reinterpret_cast<uint64_t*>(h + arr);
     unsigned long long* h_sums = reinterpret_cast<unsigned long long*>(h + 2 * arr);
-
-    const uint64_t* d_keys = keys;
     const int32_t* d_lens = lens;
-    if (host) {
-      char* base = static_cast<char*>(in_place ? c->small : c->stage);
-      uint64_t* sk = reinterpret_cast<uint64_t*>(base);
-      int32_t* sl = reinterpret_cast<int32_t*>(base + pad256(n * 8));
-      if (in_place) {
-        std::memcpy(sk, keys, n * 8);
-        if (do_sums) std::memcpy(sl, lens, n * 4);
-      } else {
-        PSKV_HIP(hipMemcpyAsync(sk, keys, n * 8, hipMemcpyHostToDevice, c->stream));
-        if (do_sums) PSKV_HIP(hipMemcpyAsync(sl, lens, n * 4, hipMemcpyHostToDevice, c->stream));
-      }
-      d_keys = sk;
-      if (do_sums) d_lens = sl;
-    }
     h_targets[0] = range_begin[0];
     for (size_t i = 0; i < S; ++i) h_targets[i + 1] = range_end[i];
     // Without lens the positions are all this call waits for, and the kernel that writes them
@@ -471,11 +480,11 @@ int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, 
       FusedTargets ft = {};
       for (size_t i = 0; i <= S; ++i) ft.v[i] = h_targets[i];
       const unsigned waves = (unsigned)std::min<size_t>(S + 1, kFusedWaves);
-      k_bounds_fused<<<dim3(1), dim3(waves * 64), 0, c->stream>>>(d_keys, n, ft, S, d_pos, h_pos,
+      k_bounds_fused<<<dim3(1), dim3(waves * 64), 0, c->stream>>>(keys, n, ft, S, d_pos, h_pos,
                                                                  do_sums ? d_sums : nullptr, watch);
       PSKV_HIP(hipGetLastError());
     } else {
-      rc = launch_bounds_search(d_keys, n, h_targets, S + 1, d_lb, c->stream);
+      rc = launch_bounds_search(keys, n, h_targets, S + 1, d_lb, c->stream);
       if (rc) return rc;
       k_bounds_chain<<<dim3(1), dim3(64), 0, c->stream>>>(d_lb, S, d_pos, h_pos, do_sums ? d_sums : nullptr,
                                                           watch);

@@ -5,8 +5,11 @@
 #include <algorithm>
 #include <atomic>
 #include <chrono>
+#include <condition_variable>
 #include <cstdlib>
 #include <cstring>
+#include <deque>
+#include <memory>
 #include <mutex>
 #include <new>
 #include <string>
@@ -53,6 +56,7 @@ constexpr uint64_t kSpareMaxBytes = 16384ull << 20;  // no array larger than thi
 // Host-resident requests up to this size (per direction) skip the copy commands: the kernels
 // read the request from, and write the response to, pinned host memory mapped into the GPU.
 constexpr size_t kSmallBytes = 1024u << 10;
+constexpr int kSmallParts = 8;  // (128 KiB each: a SCALAR push of up to 10,000 keys)
 // Host-resident buffers from this size on travel piece by piece through the ring of pinned memory
 // (stager.h), copying, transfer and kernels overlapping; smaller ones take one copy command.
 constexpr size_t kPipeBytes = 4u << 20;
@@ -66,6 +70,18 @@ struct GrowBuf {
 struct EventPair {
   hipEvent_t a, b;
 };
+
+// An allocation handed to the library's allocating thread (AllocWorker below).
+struct AllocJob {
+  int device = 0;
+  size_t bytes = 0;
+  hipStream_t stream = nullptr;
+  void* ptr = nullptr;
+  bool pooled = false;
+  int rc = PSKV_OK;
+  bool done = false;  // guarded by AllocWorker::mu
+};
+
 
 // What the host reads back of the device state, written by the device into pinned host memory
 // (a one-wavefront kernel is quicker than a copy command for these few words).
@@ -126,15 +142,17 @@ struct pskv_table {
   Slot* slots = nullptr;
   bool slots_pooled = false, arena_pooled = false;  // taken from the stream-ordered pool by a growth
   uint64_t cap = 0;        // slots, a power of two
-  // The array the next growth will move into, allocated ahead of need (once the table is 70 % of
+  // The array the next growth will move into, allocated ahead of need (once the table is half
   // the way to that growth) at the end of a request, while the GPU is busy with that request:
   // allocating costs the host 50-100 us, which would otherwise be spent with the GPU idle.
   Slot* spare = nullptr;
   uint64_t spare_cap = 0;
   bool spare_pooled = false;
+  std::shared_ptr<AllocJob> spare_job;  // the allocation of `spare` while it is under way
   // what the sizing logic did, printed when the table goes if PSKV_STATS is set in the environment
   struct Stats {
     uint64_t requests = 0, waits = 0, growths = 0, growths_unasked = 0, spare_used = 0, records = 0, catch_ups = 0;
+    double alloc_us = 0, release_us = 0, catch_up_us = 0;  // host time spent allocating, releasing, catching up
   } stats;
   uint64_t count = 0;      // key count at the last read_state()
 
@@ -164,9 +182,12 @@ struct pskv_table {
   char* small_in = nullptr;   // pinned, kSmallBytes: small host-resident requests, read in place
   char* small_out = nullptr;  // pinned, kSmallBytes: their responses, written in place
   // A small host-resident SCALAR push returns once its kernel is queued: nothing comes back from
-  // it, and the next request that writes small_in waits for this event first.
-  hipEvent_t small_done = nullptr;
-  bool small_pending = false;
+  // it. Such pushes take the kSmallParts parts of small_in in turn (when they fit one), so that
+  // several can be in flight; a request that writes a part waits for the event its last user left.
+  hipEvent_t small_done[kSmallParts] = {nullptr};
+  bool small_pending[kSmallParts] = {false};
+  int small_next = 0;      // the part the next such push takes
+  int small_newest = -1;   // the part whose event was recorded last (everything before it is done when it is)
   GrowBuf stage;      // device copies of host-resident request buffers
   GrowBuf stage_out;  // device-side response of a host-resident or undersized pull
   bool no_growth = false;  // set while dumping: every key is known to be present
@@ -410,6 +431,66 @@ int alloc_for_growth(void** out, size_t bytes, hipStream_t stream, bool* pooled)
   return PSKV_OK;
 }
 
+// Allocating a few hundred MB costs the calling thread 50 us on a good day and 800 on a bad one,
+// so the array of a coming growth is allocated by a thread of the library's own while the
+// caller goes on enqueuing requests; the growth picks the result up (and waits for it in the
+// unlikely case that it is not there yet). One thread per process, started with the first job,
+// kept until the process ends.
+class AllocWorker {
+ public:
+  static AllocWorker& get() {
+    static AllocWorker* w = new AllocWorker();  // never destroyed: its thread may outlive static destructors
+    return *w;
+  }
+  void submit(const std::shared_ptr<AllocJob>& job) {
+    {
+      std::lock_guard<std::mutex> lk(mu_);
+      if (!started_) {
+        std::thread(&AllocWorker::run, this).detach();
+        started_ = true;
+      }
+      jobs_.push_back(job);
+    }
+    cv_job_.notify_one();
+  }
+  void wait(const std::shared_ptr<AllocJob>& job) {
+    std::unique_lock<std::mutex> lk(mu_);
+    cv_done_.wait(lk, [&] { return job->done; });
+  }
+  bool finished(const std::shared_ptr<AllocJob>& job) {
+    std::lock_guard<std::mutex> lk(mu_);
+    return job->done;
+  }
+
+ private:
+  void run() {
+    for (;;) {
+      std::shared_ptr<AllocJob> job;
+      {
+        std::unique_lock<std::mutex> lk(mu_);
+        cv_job_.wait(lk, [&] { return !jobs_.empty(); });
+        job = jobs_.front();
+        jobs_.pop_front();
+      }
+      if (hipSetDevice(job->device) != hipSuccess) {
+        (void)hipGetLastError();
+        job->rc = PSKV_EHIP;
+      } else {
+        job->rc = alloc_for_growth(&job->ptr, job->bytes, job->stream, &job->pooled);
+      }
+      {
+        std::lock_guard<std::mutex> lk(mu_);
+        job->done = true;
+      }
+      cv_done_.notify_all();
+    }
+  }
+  std::mutex mu_;
+  std::condition_variable cv_job_, cv_done_;
+  std::deque<std::shared_ptr<AllocJob>> jobs_;
+  bool started_ = false;
+};
+
 // Releases an array that kernels already enqueued on `stream` may still use.
 int release_after(void* ptr, bool pooled, hipStream_t stream) {
   if (!ptr) return PSKV_OK;
@@ -470,6 +551,26 @@ int flush_scalar_cache(pskv_table* t) {
   return PSKV_OK;
 }
 
+// Takes over the array that the allocating thread was asked for, if it is there (`wait`: or
+// once it is there).
+void collect_spare(pskv_table* t, bool wait) {
+  if (!t->spare_job) return;
+  if (wait) {
+    const auto w0 = std::chrono::steady_clock::now();
+    AllocWorker::get().wait(t->spare_job);
+    t->stats.alloc_us += std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - w0).count();
+  } else if (!AllocWorker::get().finished(t->spare_job)) {
+    return;
+  }
+  if (t->spare_job->rc == PSKV_OK && t->spare_job->ptr) {
+    t->spare = static_cast<Slot*>(t->spare_job->ptr);
+    t->spare_pooled = t->spare_job->pooled;
+  } else {
+    t->spare_cap = 0;  // (the growth will ask again itself and report)
+  }
+  t->spare_job.reset();
+}
+
 // The slots a growth goes to when the table has to hold `keys_needed` keys: at least twice the
 // slots; four times while that stays a small array (a table that starts at the default size and
 // keeps growing then moves its keys half as often on the way up).
@@ -490,6 +591,7 @@ int grow_slots(pskv_table* t, uint64_t keys_needed) {
   }
   bool pooled = false;
   ++t->stats.growths;
+  collect_spare(t, true);
   if (t->spare && t->spare_cap >= want) {
     ++t->stats.spare_used;
     fresh = t->spare;
@@ -500,7 +602,9 @@ int grow_slots(pskv_table* t, uint64_t keys_needed) {
       rc = release_after(t->spare, t->spare_pooled, t->stream);
       if (rc) return rc;
     }
+    const auto a0 = std::chrono::steady_clock::now();
     rc = alloc_slots(want, &fresh, t->stream, &pooled, false);
+    t->stats.alloc_us += std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - a0).count();
     if (rc) return rc;
   }
   t->spare = nullptr;
@@ -522,7 +626,9 @@ int grow_slots(pskv_table* t, uint64_t keys_needed) {
            (const Slot*)t->slots, t->cap, fresh, want - 1, t->st);
   }
   PSKV_HIP(hipGetLastError());
+  const auto r0 = std::chrono::steady_clock::now();
   rc = release_after(t->slots, t->slots_pooled, t->stream);
+  t->stats.release_us += std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - r0).count();
   t->slots = fresh;
   t->slots_pooled = pooled;
   t->cap = want;
@@ -530,22 +636,20 @@ int grow_slots(pskv_table* t, uint64_t keys_needed) {
 }
 
 // Called at the end of a request, with its kernels queued: allocates the array of the next growth
-// once the keys the table is known to hold have come 70 % of the way to that growth.
+// once the keys the table is known to hold have come half of the way to that growth.
 void prepare_growth(pskv_table* t) {
-  if (t->spare || t->no_growth) return;
+  if (t->spare || t->spare_job || t->no_growth) return;
   const double limit = (double)t->max_load * (double)t->cap;
-  if ((double)t->base_count <= 0.7 * limit) return;
+  if ((double)t->base_count <= 0.5 * limit) return;
   const uint64_t want = grown_cap(t, 0);
   if (want * sizeof(Slot) > kSpareMaxBytes) return;
-  Slot* fresh = nullptr;
-  bool pooled = false;
-  if (alloc_slots(want, &fresh, t->stream, &pooled, false) != PSKV_OK) {
-    clear_error();  // the growth itself will ask again and report
-    return;
-  }
-  t->spare = fresh;
+  std::shared_ptr<AllocJob> job = std::make_shared<AllocJob>();
+  job->device = t->device;
+  job->bytes = want * sizeof(Slot);
+  job->stream = t->stream;
   t->spare_cap = want;
-  t->spare_pooled = pooled;
+  t->spare_job = job;
+  AllocWorker::get().submit(job);
 }
 
 int grow_arena(pskv_table* t, uint64_t floats_needed, uint64_t live_floats) {
@@ -597,9 +701,9 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
         t->record_seq != ~0ull && t->record_seq >= t->base_seq) {
       // The array is only short if the requests in flight create most of their keys, and some of
       // them are going to say how many they did create: the host lets the device catch up until the
-      // newest record settles the matter one way or the other. The device still has the requests
-      // behind that record to work on, so it does not run dry as it would in a wait for the stream;
-      // a caller that runs many requests ahead is merely held back to a few.
+      // newest record settles the matter one way or the other. A caller that runs many requests
+      // ahead is held back to a few, and the array is not replaced by a larger one before it has to
+      // be (small arrays are the quick ones: four tables of 64 MB sit in the memory-side cache).
       const auto t0 = std::chrono::steady_clock::now();
       unsigned spins = 0;
       while (slots_short() && (double)(t->base_count + n) <= limit && t->record_seq >= t->base_seq) {
@@ -610,6 +714,7 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
         }
       }
       ++t->stats.catch_ups;
+      t->stats.catch_up_us += std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
     }
     if (slots_short() && !arena_short() && !old_log &&
         grown_cap(t, t->base_count + t->pend_keys + n) * sizeof(Slot) <= kGrowUnaskedBytes) {
@@ -1412,6 +1517,7 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
   const bool host = memkind == PSKV_MEM_HOST;
   const bool varlen = t->mode == PSKV_MODE_VARLEN;
   bool small = false;        // host-resident request served from the pinned buffers
+  int small_part = -1;       // the part of small_in it lies in when it does not take all of it
   size_t small_out_at = 0;   // bytes of small_out already given away
 
   // SCALAR and FIXED know the response size up front. A response that does not fit is
@@ -1443,6 +1549,10 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
     const size_t out_lens_need = Carver::need(want_out_lens ? n : 0, 4);
     small = in_need <= kSmallBytes && out_lens_need <= kSmallBytes;
     char* base = t->small_in;
+    // a push that returns at once takes one part of the pinned buffer, the others all of it
+    const bool early = small && t->mode == PSKV_MODE_SCALAR && !pull && t->small_done[0] != nullptr;
+    small_part = (early && in_need <= kSmallBytes / kSmallParts) ? t->small_next : -1;
+    if (small_part >= 0) base += (size_t)small_part * (kSmallBytes / kSmallParts);
     if (!small) {
       rc = grow(t, &t->stage, in_need + out_lens_need);
       if (rc) return rc;
@@ -1454,10 +1564,16 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
     int32_t* dlens = c.take<int32_t>(want_lens ? n : 0);
     int32_t* dout_lens = nullptr;
     if (small) {
-      // the previous request is done with the buffers: it ended with a wait, or left an event
-      if (t->small_pending) {
-        PSKV_HIP(hipEventSynchronize(t->small_done));
-        t->small_pending = false;
+      // earlier requests are done with what this one overwrites: they ended with a wait, or left an event
+      if (small_part >= 0) {
+        if (t->small_pending[small_part]) {
+          PSKV_HIP(hipEventSynchronize(t->small_done[small_part]));
+          t->small_pending[small_part] = false;
+        }
+      } else if (t->small_newest >= 0) {
+        PSKV_HIP(hipEventSynchronize(t->small_done[t->small_newest]));  // (one stream: the others came before)
+        for (int q = 0; q < kSmallParts; ++q) t->small_pending[q] = false;
+        t->small_newest = -1;
       }
       if (n) std::memcpy(dkeys, keys, n * 8);
       if (r.nvals) std::memcpy(dvals, vals, r.nvals * 4);
@@ -1558,11 +1674,13 @@ int request(pskv_table* t, bool push, bool pull, const uint64_t* keys, size_t n,
     }
     if (pull && varlen && out_lens && n && !lens_pinned)
       PSKV_HIP(hipMemcpyAsync(out_lens, r.out_lens, n * 4, hipMemcpyDeviceToHost, t->stream));
-    if (t->mode == PSKV_MODE_SCALAR && small && !pull && t->small_done) {
+    if (small_part >= 0) {
       // no device-detected errors in this mode and nothing to hand back: the caller's buffers have
       // been copied, the kernel is queued, later requests follow it on the stream
-      PSKV_HIP(hipEventRecord(t->small_done, t->stream));
-      t->small_pending = true;
+      PSKV_HIP(hipEventRecord(t->small_done[small_part], t->stream));
+      t->small_pending[small_part] = true;
+      t->small_newest = small_part;
+      t->small_next = (small_part + 1) % kSmallParts;
     } else if (t->mode == PSKV_MODE_SCALAR) {
       // no device-detected errors in this mode: waiting for the stream is all that is left
       PSKV_HIP(hipStreamSynchronize(t->stream));
@@ -1746,9 +1864,11 @@ int pskv_table_create(pskv_table** out, const pskv_opts* opts) {
       hipHostMalloc(reinterpret_cast<void**>(&t->small_in), kSmallBytes, hipHostMallocCoherent) !=
           hipSuccess ||
       hipHostMalloc(reinterpret_cast<void**>(&t->small_out), kSmallBytes, hipHostMallocCoherent) !=
-          hipSuccess ||
-      hipEventCreateWithFlags(&t->small_done, hipEventDisableTiming) != hipSuccess)
+          hipSuccess)
     return fail(set_error(PSKV_ENOMEM, "cannot allocate table state"));
+  for (int q = 0; q < kSmallParts; ++q)
+    if (hipEventCreateWithFlags(&t->small_done[q], hipEventDisableTiming) != hipSuccess)
+      return fail(set_error(PSKV_ENOMEM, "cannot allocate table state"));
   std::memset(t->snap, 0xFF, sizeof(Snapshot));  // names no request
   *t->outcome = 0ull;
   if (t->mode != PSKV_MODE_SCALAR && opts->arena_floats) {
@@ -1774,11 +1894,13 @@ int pskv_table_destroy(pskv_table* t) {
   DeviceGuard guard(t->device);
   if (std::getenv("PSKV_STATS"))
     fprintf(stderr, "[pskv] table %p mode %d: %llu requests, %llu slots at the end, %llu growths (%llu without asking "
-            "the device, %llu into an array allocated ahead), %llu waits for exact counters, %llu for the newest record, %llu counter records\n",
+            "the device, %llu into an array allocated ahead), %llu waits for exact counters, %llu for the newest record (%.0f us), %llu counter records; host time "
+            "allocating %.0f us, releasing %.0f us\n",
             (void*)t, t->mode, (unsigned long long)t->stats.requests, (unsigned long long)t->cap,
             (unsigned long long)t->stats.growths, (unsigned long long)t->stats.growths_unasked,
             (unsigned long long)t->stats.spare_used, (unsigned long long)t->stats.waits,
-            (unsigned long long)t->stats.catch_ups, (unsigned long long)t->stats.records);
+            (unsigned long long)t->stats.catch_ups, t->stats.catch_up_us, (unsigned long long)t->stats.records,
+            t->stats.alloc_us, t->stats.release_us);
   if (t->stream) (void)hipStreamSynchronize(t->stream);
   for (int k = 0; k < PSKV_KERNEL_COUNT; ++k)
     for (const EventPair& ev : t->pending[k]) t->free_events.push_back(ev);
@@ -1796,6 +1918,7 @@ int pskv_table_destroy(pskv_table* t) {
     (void)hipFreeAsync(t->arena, t->stream);
     t->arena = nullptr;
   }
+  collect_spare(t, true);
   if (t->spare && t->spare_pooled) {
     (void)hipFreeAsync(t->spare, t->stream);
   } else if (t->spare) {
@@ -1808,7 +1931,8 @@ int pskv_table_destroy(pskv_table* t) {
   if (t->outcome) (void)hipHostFree(t->outcome);
   if (t->sc_vals.ptr) (void)hipFree(t->sc_vals.ptr);
   if (t->sc_slots.ptr) (void)hipFree(t->sc_slots.ptr);
-  if (t->small_done) (void)hipEventDestroy(t->small_done);
+  for (int q = 0; q < kSmallParts; ++q)
+    if (t->small_done[q]) (void)hipEventDestroy(t->small_done[q]);
   if (t->small_in) (void)hipHostFree(t->small_in);
   if (t->small_out) (void)hipHostFree(t->small_out);
   if (t->arena) (void)hipFree(t->arena);

@@ -66,6 +66,25 @@ def test_slice_sixteen_million_keys(capi, dev, S):
     assert np.array_equal(pos2, pos) and np.array_equal(vpos2.astype(np.int64), 2 * pos.astype(np.int64))
 
 
+@pytest.mark.parametrize("S", [1, 4, 1024])
+def test_slice_sixteen_million_keys_in_host_memory(capi, orc, dev, S):
+    """The same request with its keys (and lens) in ordinary host memory, as the worker's slicer
+    gets them (kv_app.h:517-572): host-resident keys are searched where they lie, the lens of a
+    request this large are added up on the GPU. Positions, value offsets and flags against the oracle."""
+    announce("slice_16M_host", S)
+    n = 16000000
+    rng = np.random.default_rng(61 + S)
+    rb, re = capi.server_ranges(S)
+    keys = unique_keys(rng, n, S)
+    lens = rng.integers(0, 5, size=n).astype(np.int32)
+    assert _compare(capi, orc, keys, rb, re, None, 2 * n, dev, "host") == 0
+    assert _compare(capi, orc, keys, rb, re, lens, int(lens.sum()), dev, "host") == 0
+    # a key past the last range: the reference's CHECK at kv_app.h:542
+    bad = keys.copy()
+    bad[-1] = np.uint64(KMAX)
+    assert _compare(capi, orc, bad, rb, re, None, 2 * n, dev, "host") == capi.EUNCOVERED_KEY
+
+
 @pytest.mark.parametrize("memkind", ["device", "host"])
 def test_slice_skewed_and_edges(capi, orc, dev, memkind):
     """All keys in one range, keys sitting exactly on range boundaries, empty middle slices."""
