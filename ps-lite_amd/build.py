@@ -64,8 +64,8 @@ def build_host_test():
     """Compiles the test program tests/test_kv_app_gpu.cc, which drives the adapters of
     include/pskv/ps_adapters.h the way tests/test_kv_app.cc of the reference drives ps-lite
     (test infrastructure: it uses the in-process ps:: surface of tests/include/pskv/ps_min.h)."""
-    cmd = ["g++", "-std=c++11", "-O2", "-Wall", "-I" + os.path.join(REPO, "include"),
-           "-I" + os.path.join(REPO, "tests", "include"),
+    cmd = ["g++", "-std=c++11", "-O2", "-Wall", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include",
+           "-I" + os.path.join(REPO, "include"), "-I" + os.path.join(REPO, "tests", "include"),
            os.path.join(REPO, "tests", "test_kv_app_gpu.cc"), "-L" + HERE, "-lpskv",
            "-Wl,-rpath,$ORIGIN/../ps-lite_amd", "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib", "-lamdhip64",
            "-o", HOST_TEST]

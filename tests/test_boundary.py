@@ -53,8 +53,8 @@ def test_errors_without_a_device(capi):
 
 
 def test_adapters_compile_with_in_process_surface(tmp_path):
-    subprocess.run(["g++", "-std=c++11", "-Wall", "-Werror", "-I" + os.path.join(REPO, "include"),
-                    "-I" + os.path.join(REPO, "tests", "include"), "-c",
+    subprocess.run(["g++", "-std=c++11", "-Wall", "-Werror", "-D__HIP_PLATFORM_AMD__", "-isystem", "/opt/rocm/include",
+                    "-I" + os.path.join(REPO, "include"), "-I" + os.path.join(REPO, "tests", "include"), "-c",
                     os.path.join(REPO, "tests", "test_kv_app_gpu.cc"), "-o",
                     str(tmp_path / "t.o")], check=True)
 

@@ -138,15 +138,63 @@ def test_config3_dense_chunks_from_host_memory(capi, orc, dev):
         ", ".join("%.1f" % (nk * k * 4 / s / 1e9) for s in secs), nk * k * 4 / pull_s / 1e9))
 
 
+def test_config2_as_the_benchmark_runs_it(capi, orc, dev):
+    """The measured path itself at full size: four tables of the default capacity that share one
+    stream, every step one pskv_slice, ONE pskv_push_multi over the four key ranges and ONE
+    pskv_pull_multi of the same keys (served from what the push left behind once the tables have
+    seen a pull follow a push), no wait inside the run, the tables growing as they go. EVERY
+    step's pull is compared with the oracle's, then the four sizes and the dump of one table."""
+    import torch
+    announce("config2 as benched")
+    n, S, steps = 1000000, 4, 20
+    rb, re = capi.server_ranges(S)
+    group = capi.Group(S, capi.MODE_SCALAR)
+    stores = [orc.Store(orc.MODE_SCALAR) for _ in range(S)]
+    batches = []
+    for p in range(steps):
+        rng = np.random.default_rng(0xC0FFEE + p)
+        keys = unique_keys(rng, n, S)
+        batches.append((keys, rng.normal(0, 0.01, size=n).astype(np.float32)))
+    # three steps repeat earlier key sets, so that pushes also meet keys that are stored already
+    batches[7] = (batches[2][0], batches[7][1])
+    batches[13] = (batches[12][0], batches[13][1])
+    batches[19] = (batches[12][0], batches[19][1])
+    d_batches = [(to_dev(k, dev), to_dev(v, dev)) for k, v in batches]
+    outs = [torch.full((n,), 7.0, dtype=torch.float32, device=dev) for _ in range(steps)]
+    torch.cuda.synchronize()
+    for p in range(steps):
+        dk, dv = d_batches[p]
+        pos, vpos, used = capi.slice_keys(dk, rb, re, nvals=n)
+        group.push_raw(dk.data_ptr(), pos, dv.data_ptr(), vpos)
+        group.pull_raw(dk.data_ptr(), pos, outs[p].data_ptr())
+    group.sync()
+    held = 0
+    for p in range(steps):
+        keys, vals = batches[p]
+        o_pos, _, _ = orc.slice_keys(keys, rb, re, nvals=n)
+        o_pos = [int(x) for x in o_pos]
+        want = np.empty(n, np.float32)
+        for s in range(S):
+            a, b = o_pos[s], o_pos[s + 1]
+            stores[s].push(keys[a:b], vals[a:b])
+            want[a:b] = stores[s].pull(keys[a:b])[0]
+        assert_bits_equal(from_dev(outs[p]), want, "pull of step %d" % p)
+    for s in range(S):
+        assert group.tables[s].size() == stores[s].size(), s
+        held += group.tables[s].size()[0]
+    assert held == np.unique(np.concatenate([k for k, _ in batches])).size
+    gk, _, gv = group.tables[2].dump()
+    ok, _, ov = stores[2].dump()
+    assert np.array_equal(gk, ok)
+    assert_bits_equal(gv, ov, "dump of table 2")
+    group.close()
+
+
 def _zipf_unique(rng, n, universe, s=1.1):
-    """n distinct ranks in [0, universe) with Zipf(s) popularity, sorted."""
-    got = np.zeros(0, np.int64)
-    while got.size < n:
-        r = rng.zipf(s, size=2 * n).astype(np.int64) - 1
-        got = np.unique(np.concatenate([got, r[(r >= 0) & (r < universe)]]))
-    if got.size > n:
-        got = np.sort(rng.choice(got, size=n, replace=False))
-    return got
+    """n distinct ranks with Zipf(s) popularity (the benchmark's generator: the set of ranks that
+    a long run of draws names, without drawing them one by one)."""
+    import bench
+    return bench.zipf_distinct_ranks(rng, n, universe, s)
 
 
 def _rank_to_key(r):

@@ -776,19 +776,16 @@ def small_scalar_cache(monkeypatch):
     monkeypatch.setenv("PSKV_SCALAR_CACHE_MIN_KEYS", "64")
 
 
-@pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
-@pytest.mark.parametrize("seed", [0, 1, 2, 3])
-def test_repeated_and_alternating_key_sets(capi, orc, dev, mode, seed, small_scalar_cache):
-    """Requests that repeat the previous request's keys take a path that skips the hash probes; requests
-    that do not must never see what that path left behind. Random sequences over a few key sets that
-    are equal, differ in one key, differ in one length or differ in size, through every entry point
-    and both memory kinds, checked against the oracle after every pull. (SCALAR: the values of a
-    repeated key set live in a request-ordered array that is ahead of the slots until something else
-    needs them; a larger key set makes the table grow in the middle of that.)"""
+def _drive_key_sets(capi, orc, dev, mode, seed, steps, script="random"):
+    """One random sequence of requests over a few related key sets, through every entry point and
+    both memory kinds, every pull compared with the oracle, the dump at the end. `script` shapes
+    the sequence: "random" draws the key set of every step from all of them; "two_sizes" alternates
+    between two sets of different sizes (each recorded in turn); "threshold" mixes sets below and
+    above the size from which SCALAR requests use the key cache; "growth" keeps bringing sets of
+    new keys between repeats of one set, so that the table grows while that set is cached."""
     import torch
-    announce("repeated_key_sets", mode, seed)
     rng = np.random.default_rng(1000 + seed)
-    n = int(rng.integers(300, 3000))
+    n = int(rng.integers(300, 3000)) if script != "threshold" else int(rng.integers(80, 200))
     k = 1 if mode == "scalar" else 8
     base = unique_keys(rng, n + 50)
     sets = {}
@@ -798,7 +795,23 @@ def test_repeated_and_alternating_key_sets(capi, orc, dev, mode, seed, small_sca
     sets["B"] = np.sort(b)
     sets["C"] = base[10:n + 10].copy()        # same size, shifted
     sets["D"] = base[: n // 2].copy()         # a different size
-    lens_of = {int(key): int(l) for key, l in zip(base.tolist(), rng.choice([0, 4, 8, 12, 40], size=base.size))}
+    names = ["A", "A", "A", "B", "C", "D", "A"]
+    extra_keys = np.zeros(0, np.uint64)
+    if mode == "scalar" and script == "random":
+        sets["E"] = np.union1d(base, unique_keys(rng, 6 * n))  # makes the table grow when it first comes
+        names += ["E"]
+    if script == "two_sizes":
+        names = ["A", "D"]
+    if script == "threshold":  # (the fixture sets the threshold to 64 keys)
+        sets["F"] = base[:40].copy()
+        sets["G"] = base[5:68].copy()   # one key below the threshold
+        sets["H"] = base[5:69].copy()   # exactly at it
+        names = ["A", "F", "G", "H", "A", "H", "F"]
+    if script == "growth":
+        extra_keys = unique_keys(rng, 40 * n)
+        names = ["A", "A", "new", "A", "new", "B"]
+    pool = np.union1d(base, extra_keys)
+    lens_of = {int(key): int(l) for key, l in zip(pool.tolist(), rng.choice([0, 4, 8, 12, 40], size=pool.size))}
     m = {"scalar": capi.MODE_SCALAR, "fixed": capi.MODE_FIXED, "varlen": capi.MODE_VARLEN}[mode]
     om = {"scalar": orc.MODE_SCALAR, "fixed": orc.MODE_FIXED, "varlen": orc.MODE_VARLEN}[mode]
     t = capi.Table(m, initial_capacity=64, row_len=k if mode == "fixed" else 0)  # small: the slot array grows during the sequence
@@ -807,13 +820,14 @@ def test_repeated_and_alternating_key_sets(capi, orc, dev, mode, seed, small_sca
     def lens_for(keys):
         return np.array([lens_of[int(x)] for x in keys.tolist()], np.int32) if mode == "varlen" else None
 
-    names = ["A", "A", "A", "B", "C", "D", "A"]
-    if mode == "scalar":
-        sets["E"] = np.union1d(base, unique_keys(rng, 6 * n))  # makes the table grow when it first comes
-        names += ["E"]
-    for step in range(60 if mode == "scalar" else 40):
-        name = names[int(rng.integers(0, len(names)))]
-        keys = sets[name]
+    fresh_at = 0
+    for step in range(steps):
+        name = names[step % 2] if script == "two_sizes" and step < steps // 2 else names[int(rng.integers(0, len(names)))]
+        if name == "new":
+            keys = extra_keys[fresh_at:fresh_at + n]
+            fresh_at = (fresh_at + n) % (extra_keys.size - n)
+        else:
+            keys = sets[name]
         lens = lens_for(keys)
         nvals = int(lens.sum()) if mode == "varlen" else keys.size * k
         op = ["push", "push", "pull", "pull_async", "pushpull"][int(rng.integers(0, 5))]
@@ -824,7 +838,7 @@ def test_repeated_and_alternating_key_sets(capi, orc, dev, mode, seed, small_sca
         kk = to_dev(keys, dev) if on_dev else keys
         vv = to_dev(vals, dev) if on_dev else vals
         ll = None if lens is None else (to_dev(lens, dev) if on_dev else lens)
-        what = "step %d %s %s %s" % (step, op, name, "dev" if on_dev else "host")
+        what = "seed %d %s step %d %s %s %s" % (seed, script, step, op, name, "dev" if on_dev else "host")
         if op == "push":
             t.push(kk, vv, ll)
             o.push(keys, vals, lens)
@@ -868,7 +882,38 @@ def test_repeated_and_alternating_key_sets(capi, orc, dev, mode, seed, small_sca
             if mode == "varlen":
                 assert np.array_equal(got_lens, want_lens), what
     t.sync()
-    _check_dump(t, o, "after the sequence")
+    _check_dump(t, o, "seed %d %s after the sequence" % (seed, script))
+    t.close()
+
+
+@pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_repeated_and_alternating_key_sets(capi, orc, dev, mode, seed, small_scalar_cache):
+    """Requests that repeat the previous request's keys take a path that skips the hash probes; requests
+    that do not must never see what that path left behind. Random sequences over a few key sets that
+    are equal, differ in one key, differ in one length or differ in size, through every entry point
+    and both memory kinds, checked against the oracle after every pull. (SCALAR: the values of a
+    repeated key set live in a request-ordered array that is ahead of the slots until something else
+    needs them; a larger key set makes the table grow in the middle of that.)"""
+    announce("repeated_key_sets", mode, seed)
+    _drive_key_sets(capi, orc, dev, mode, seed, 60 if mode == "scalar" else 40)
+
+
+@pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
+def test_key_cache_policy_over_many_sequences(capi, orc, dev, mode, small_scalar_cache):
+    """What decides whether a request is compared with, served from or recorded into the key cache
+    is host-side bookkeeping (sizes that repeat, pulls that follow pushes, comparisons that keep
+    failing, the size threshold). 256 further sequences per mode, a quarter each of four shapes: any
+    key set at any step; two sets of different sizes in strict alternation, then at random; sets
+    just below, at and above the threshold; new keys that make the table grow between repeats of
+    a cached set. Stops at the first sequence that differs from the oracle."""
+    import time
+    announce("key_cache_policy", mode)
+    scripts = ["random", "two_sizes", "threshold", "growth"]
+    t0 = time.time()
+    for seed in range(100, 356):
+        _drive_key_sets(capi, orc, dev, mode, seed, 40, scripts[seed % 4])
+    print("256 sequences in %.1f s" % (time.time() - t0), flush=True)
 
 
 def test_refused_push_does_not_poison_repeats(capi, orc, dev):
@@ -1102,6 +1147,40 @@ def test_scalar_key_cache_at_its_real_size(capi, orc, dev, memkind):
         assert_bits_equal(out, out_np, "pushpull")
     t.sync()
     _check_dump(t, o, "scalar key cache")
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_scalar_key_cache_across_its_default_threshold(capi, orc, dev, seed):
+    """Requests of 131,072 keys and more may use the SCALAR key cache, smaller ones never do. Random
+    sequences over key sets of 131,071, 131,072 and 140,000 keys (nested, so that a request below
+    the threshold changes values that the cache holds for a set above it) and a set of other keys,
+    pushes and pulls, device-resident and without a wait between requests: every pull against the
+    oracle, the dump at the end."""
+    import torch
+    announce("scalar_cache_threshold", seed)
+    rng = np.random.default_rng(400 + seed)
+    big = unique_keys(rng, 140000)
+    sets = {"below": big[:131071].copy(), "at": big[:131072].copy(), "above": big,
+            "other": unique_keys(rng, 135000)}
+    names = ["above", "above", "at", "below", "above", "other", "at"]
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=1 << 18)
+    o = orc.Store(orc.MODE_SCALAR)
+    checks = []
+    for step in range(36):
+        name = names[int(rng.integers(0, len(names)))]
+        keys = sets[name]
+        if rng.random() < 0.6:
+            vals = rng.normal(0, 1, size=keys.size).astype(np.float32)
+            t.push(to_dev(keys, dev), to_dev(vals, dev))
+            o.push(keys, vals)
+        else:
+            out = torch.full((keys.size,), 7.0, dtype=torch.float32, device=dev)
+            t.pull(to_dev(keys, dev), out)
+            checks.append((step, name, out, o.pull(keys)[0]))
+    t.sync()
+    for step, name, out, want in checks:
+        assert_bits_equal(from_dev(out), want, "pull of %s at step %d" % (name, step))
+    _check_dump(t, o, "across the threshold")
 
 
 @pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])

@@ -15,6 +15,8 @@
 #include <thread>
 #include <vector>
 
+#include <hip/hip_runtime_api.h>
+
 #include "pskv/ps_min.h"
 #include "pskv/ps_adapters.h"
 
@@ -170,6 +172,55 @@ static void RunOrderedMatch() {
   }
   EXPECT(threw);
   std::printf("ordered match: %zu of %d values matched\n", n, num * k);
+}
+
+// The contract of device-resident calls, through the C ABI alone (nothing keeps the buffers alive
+// for the caller here): a PSKV_MEM_DEVICE call only enqueues work; the table reads the request's
+// buffers, and writes the response, some time before the next pskv_sync returns; after that wait
+// the buffers are the caller's again and may be overwritten or freed. 150,000 keys, above the size
+// from which SCALAR tables keep a request-ordered copy of the last key set, so the pushes also go
+// through that copy; every push brings other values in the SAME device buffer.
+static void RunDeviceBufferContract() {
+  const size_t n = 150000;
+  const int pushes = 12;
+  pskv_opts o = {};
+  o.mode = PSKV_MODE_SCALAR;
+  pskv_table* t = nullptr;
+  EXPECT(pskv_table_create(&t, &o) == PSKV_OK);
+  std::vector<uint64_t> keys(n);
+  std::vector<float> vals(n), want(n, 0.0f), got(n, -1.0f);
+  for (size_t i = 0; i < n; ++i) keys[i] = (~0ull / n) * i + 17;
+  uint64_t* d_keys = nullptr;
+  float *d_vals = nullptr, *d_out = nullptr;
+  EXPECT(hipMalloc(reinterpret_cast<void**>(&d_keys), n * 8) == hipSuccess);
+  EXPECT(hipMalloc(reinterpret_cast<void**>(&d_vals), n * 4) == hipSuccess);
+  EXPECT(hipMalloc(reinterpret_cast<void**>(&d_out), n * 4) == hipSuccess);
+  EXPECT(hipMemcpy(d_keys, keys.data(), n * 8, hipMemcpyHostToDevice) == hipSuccess);
+  for (int p = 0; p < pushes; ++p) {
+    for (size_t i = 0; i < n; ++i) {
+      vals[i] = static_cast<float>((i * 7 + p * 13) % 101) * 0.25f - 3.0f;
+      want[i] = want[i] + vals[i];
+    }
+    // the buffer is the caller's here: the previous push has been waited for
+    EXPECT(hipMemcpy(d_vals, vals.data(), n * 4, hipMemcpyHostToDevice) == hipSuccess);
+    EXPECT(pskv_push(t, d_keys, n, d_vals, n, nullptr, 0, PSKV_MEM_DEVICE) == PSKV_OK);
+    if (p % 3 == 1) EXPECT(pskv_pull(t, d_keys, n, d_out, n, nullptr, nullptr, PSKV_MEM_DEVICE) == PSKV_OK);
+    EXPECT(pskv_sync(t) == PSKV_OK);  // from here on d_vals may change again
+  }
+  EXPECT(pskv_pull(t, d_keys, n, d_out, n, nullptr, nullptr, PSKV_MEM_DEVICE) == PSKV_OK);
+  EXPECT(pskv_sync(t) == PSKV_OK);  // from here on d_out holds the response
+  EXPECT(hipMemcpy(got.data(), d_out, n * 4, hipMemcpyDeviceToHost) == hipSuccess);
+  size_t bad = 0;
+  for (size_t i = 0; i < n; ++i) bad += got[i] != want[i];
+  EXPECT(bad == 0);
+  // buffers may be freed once the wait has returned, with the table still alive
+  EXPECT(hipFree(d_vals) == hipSuccess);
+  EXPECT(hipFree(d_out) == hipSuccess);
+  EXPECT(hipFree(d_keys) == hipSuccess);
+  uint64_t held = 0;
+  EXPECT(pskv_size(t, &held, nullptr) == PSKV_OK && held == n);
+  EXPECT(pskv_table_destroy(t) == PSKV_OK);
+  std::printf("device buffers: %d pushes of %zu keys from one buffer, %zu floats differ\n", pushes, n, bad);
 }
 
 static void RunTwoWorkers(int app_id) {
@@ -358,6 +409,7 @@ int main(int argc, char** argv) {
     RunVarLen();
     RunFailures(num_servers);
     RunOrderedMatch();
+    RunDeviceBufferContract();
     auto s6 = StartServers(6, num_servers, PSKV_MODE_SCALAR);
     RunTwoWorkers(6);
     if (argc > 2) {  // floats per key of the dense run from host memory (4194304 is the configuration's)
