@@ -52,6 +52,7 @@ constexpr uint64_t kSlackBytes = 256ull << 20;  // tables up to this size trade 
 // A slot array that could run short is replaced without asking the device first while the larger
 // one stays below this size; beyond it the host waits for exact counters before it spends the memory.
 constexpr uint64_t kGrowUnaskedBytes = 4096ull << 20;
+constexpr uint64_t kKeepInFlight = 2;  // requests the host leaves unaccounted for when it lets the device catch up
 constexpr uint64_t kSpareMaxBytes = 16384ull << 20;  // no array larger than this is allocated ahead of need
 // Host-resident requests up to this size (per direction) skip the copy commands: the kernels
 // read the request from, and write the response to, pinned host memory mapped into the GPU.
@@ -112,19 +113,6 @@ __global__ void k_read_state(StateBatch sb) {
   out->error = st->error;
   out->req_error = st->req_error;
   out->special_present = st->special_present;
-}
-
-// One wavefront per table that asked for a record (blockIdx.x), launched behind the kernel of
-// a SCALAR request when a table is close to a limit (the row modes let their lookup kernels
-// write the record).
-struct PubBatch {
-  const DevState* st[kMaxBatch];
-  Snapshot* out[kMaxBatch];
-  uint64_t seq[kMaxBatch];
-};
-__global__ void k_publish(PubBatch pb) {
-  if (!pb.out[blockIdx.x]) return;
-  publish_snapshot(pb.st[blockIdx.x], pb.out[blockIdx.x], pb.seq[blockIdx.x]);
 }
 
 }  // namespace
@@ -679,7 +667,7 @@ int grow_arena(pskv_table* t, uint64_t floats_needed, uint64_t live_floats) {
 // Close to a limit the device publishes its counters as they are after the request, so that a
 // later request can move the base forward without waiting for the stream: `pub->snap` is
 // set when a record is wanted, and the caller hands it to the kernel of the request that
-// changes the counters (or launches k_publish behind it).
+// changes the counters.
 struct PublishReq {
   Snapshot* snap = nullptr;
   uint64_t seq = 0;
@@ -698,15 +686,18 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
     adopt_snapshot(t);
     const bool old_log = t->seq - t->base_seq >= (uint64_t)pskv_table::kLog - 1;
     if (slots_short() && !arena_short() && !old_log && (double)(t->base_count + n) <= limit &&
-        t->record_seq != ~0ull && t->record_seq >= t->base_seq) {
+        t->record_seq != ~0ull && t->record_seq >= t->base_seq && t->seq - t->base_seq > kKeepInFlight) {
       // The array is only short if the requests in flight create most of their keys, and some of
-      // them are going to say how many they did create: the host lets the device catch up until the
-      // newest record settles the matter one way or the other. A caller that runs many requests
-      // ahead is held back to a few, and the array is not replaced by a larger one before it has to
-      // be (small arrays are the quick ones: four tables of 64 MB sit in the memory-side cache).
+      // them are going to say how many they did create: the host lets the device catch up, but not
+      // all the way. A caller that runs many requests ahead is held back until only kKeepInFlight
+      // requests are unaccounted for (so the device never runs dry, as it would in a wait for the
+      // stream, and the steps that follow do not run in lock-step with the host); if the array
+      // still looks short then, it is replaced, at most that many requests early and sized for
+      // at most that many requests of uncertainty.
       const auto t0 = std::chrono::steady_clock::now();
       unsigned spins = 0;
-      while (slots_short() && (double)(t->base_count + n) <= limit && t->record_seq >= t->base_seq) {
+      while (slots_short() && (double)(t->base_count + n) <= limit && t->record_seq >= t->base_seq &&
+             t->seq - t->base_seq > kKeepInFlight) {
         adopt_snapshot(t);
         if ((++spins & 63u) == 0) {
           if (std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(20)) break;
@@ -837,24 +828,6 @@ int launch_batch(Batch& bt, int prof_kernel, void (*kernel)(ReqBatch), F nblk_of
   }
   if (!gx) return PSKV_OK;
   launch(lead_of(bt), prof_kernel, kernel, dim3((unsigned)gx, (unsigned)bt.size()), dim3(kBlock), rb);
-  PSKV_HIP(hipGetLastError());
-  return PSKV_OK;
-}
-
-// The counter records the tables of a batch asked for (reserve), one wavefront each.
-int publish_batch(Batch& bt) {
-  PubBatch pb;
-  std::memset(&pb, 0, sizeof(pb));
-  bool any = false;
-  for (size_t i = 0; i < bt.size(); ++i) {
-    if (!bt[i].pub.snap) continue;
-    pb.st[i] = bt[i].t->st;
-    pb.out[i] = bt[i].pub.snap;
-    pb.seq[i] = bt[i].pub.seq;
-    any = true;
-  }
-  if (!any) return PSKV_OK;
-  k_publish<<<dim3((unsigned)bt.size()), dim3(64), 0, bt[0].t->stream>>>(pb);
   PSKV_HIP(hipGetLastError());
   return PSKV_OK;
 }
@@ -1027,6 +1000,8 @@ int run_scalar(Batch& bt, bool push, bool pull) {
     d.vals = r.vals;
     d.out = r.out;
     d.n = r.n;
+    d.snap = it.pub.snap;  // the request's kernel leaves the counter record itself
+    d.snap_seq = it.pub.seq;
     n_largest = std::max(n_largest, r.n);
   }
   if (!n_largest) return PSKV_OK;
@@ -1073,7 +1048,7 @@ int run_scalar(Batch& bt, bool push, bool pull) {
     t->cache_n = bt[i].r.n;
     if (push && use[i] == kScTry) t->sc_dirty = true;  // served from the cache: the slots lag behind
   }
-  return publish_batch(bt);
+  return PSKV_OK;
 }
 
 // Requests at least this large (4 MiB) are streamed with non-temporal accesses: between two

@@ -127,6 +127,8 @@ __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
         }
       }
     }
+    // (no key is created on this path: the counters are what they were)
+    if (d.snap && blockIdx.x == 0 && threadIdx.x < 64) publish_snapshot(st, d.snap, d.snap_seq);
     return;
   }
   if (record && blockIdx.x == 0 && threadIdx.x == 0) st->cache_epoch = d.tag.epoch;
@@ -234,16 +236,24 @@ __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
     }
   }
   block_count_add(st, created, red);
-  if (kPerKey && d.cache_mode == kCachePerKey) {
-    // tell the host, which never waits for it, whether every key sat at its cached position
-    const int any = __syncthreads_or(differs ? 1 : 0);
+  // The workgroup that finishes last tells the host, which never waits for either, whether every
+  // key of a key-by-key pull sat at its cached position and, when the host asked for it (the
+  // table is close to a limit), what the counters are after this request.
+  const bool want_outcome = kPerKey && d.cache_mode == kCachePerKey;
+  if (want_outcome || d.snap) {
+    __shared__ unsigned s_last;
+    const int any = want_outcome ? __syncthreads_or(differs ? 1 : 0) : 0;
     if (threadIdx.x == 0) {
       if (any) atomicOr(&st->req_flags, kReqDiffer);
-      if (ticket_last(st, nblk)) {
-        const bool all = (atomicExch(&st->req_flags, 0u) & kReqDiffer) == 0u && per_key;
-        if (d.outcome) *d.outcome = (d.tag.epoch << 1) | (all ? 1ull : 0ull);
-      }
+      s_last = ticket_last(st, nblk) ? 1u : 0u;
     }
+    __syncthreads();
+    if (!s_last) return;
+    if (want_outcome && threadIdx.x == 0) {
+      const bool all = (atomicExch(&st->req_flags, 0u) & kReqDiffer) == 0u && per_key;
+      if (d.outcome) *d.outcome = (d.tag.epoch << 1) | (all ? 1ull : 0ull);
+    }
+    if (d.snap && threadIdx.x < 64) publish_snapshot(st, d.snap, d.snap_seq);
   }
 }
 
