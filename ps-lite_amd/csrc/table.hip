@@ -130,7 +130,7 @@ struct pskv_table {
   Slot* slots = nullptr;
   bool slots_pooled = false, arena_pooled = false;  // taken from the stream-ordered pool by a growth
   uint64_t cap = 0;        // slots, a power of two
-  // The array the next growth will move into, allocated ahead of need (once the table is half
+  // The array the next growth will move into, allocated ahead of need (once the table is 40 % of
   // the way to that growth) at the end of a request, while the GPU is busy with that request:
   // allocating costs the host 50-100 us, which would otherwise be spent with the GPU idle.
   Slot* spare = nullptr;
@@ -624,11 +624,12 @@ int grow_slots(pskv_table* t, uint64_t keys_needed) {
 }
 
 // Called at the end of a request, with its kernels queued: allocates the array of the next growth
-// once the keys the table is known to hold have come half of the way to that growth.
+// once the keys the table is known to hold have come 40 % of the way to that growth.
 void prepare_growth(pskv_table* t) {
   if (t->spare || t->spare_job || t->no_growth) return;
+  adopt_snapshot(t);  // (a read of pinned memory)
   const double limit = (double)t->max_load * (double)t->cap;
-  if ((double)t->base_count <= 0.5 * limit) return;
+  if ((double)t->base_count <= 0.4 * limit) return;
   const uint64_t want = grown_cap(t, 0);
   if (want * sizeof(Slot) > kSpareMaxBytes) return;
   std::shared_ptr<AllocJob> job = std::make_shared<AllocJob>();
@@ -743,8 +744,11 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
   t->log_units[q % pskv_table::kLog] = units;
   t->pend_keys += n;
   t->pend_units += units;
+  // From a third of the way to the next growth on, every request leaves a record (its kernel's
+  // last workgroup writes four words): the host then knows how full the table is, give or take
+  // the requests in flight, early enough to have the next array allocated by the time it is needed.
   const double limit_now = (double)t->max_load * (double)t->cap;
-  const bool tight_slots = (double)(t->base_count + t->pend_keys + 2 * n) > limit_now;
+  const bool tight_slots = (double)(t->base_count + t->pend_keys + 2 * n) > 0.35 * limit_now;
   const bool tight_arena =
       units && (t->base_top + t->pend_units + 2 * units) * floats_per_unit > t->arena_cap;
   // (a base that merely grows old asks for a record every eighth request, not every one)
@@ -1992,6 +1996,7 @@ int pskv_sync(pskv_table* t) {
   DeviceGuard guard(t->device);
   int rc = read_state(t);
   if (rc) return rc;
+  prepare_growth(t);  // (the counters are exact now)
   return report_device_errors(t);
 }
 
