@@ -153,6 +153,35 @@ def test_growth_of_a_large_array_by_two(capi, orc, dev):
     _check_dump(t, o, "large growth")
 
 
+def test_device_trim_between_growths(capi, orc, dev):
+    """pskv_device_trim gives back what the pool keeps (the arrays that growths have replaced) and the
+    workspaces of pskv_match; tables that are alive keep working, grow again and stay exact."""
+    import torch
+    announce("device_trim")
+    rng = np.random.default_rng(808)
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=1000)
+    o = orc.Store(orc.MODE_SCALAR)
+    universe = unique_keys(rng, 400000)
+    for part in np.array_split(universe, 8)[:4]:
+        vals = rng.integers(-9, 9, size=part.size).astype(np.float32)
+        t.push(to_dev(part, dev), to_dev(vals, dev))
+        o.push(part, vals)
+    sk = unique_keys(rng, 5000)
+    dst = torch.zeros(sk.size, dtype=torch.float32, device=dev)
+    assert capi.match(to_dev(sk, dev), to_dev(np.ones(sk.size, np.float32), dev), to_dev(sk, dev), dst, 1, capi.OP_PLUS) == sk.size
+    capi.device_trim()   # requests may be in flight: the call waits for the device first
+    capi.device_trim()   # nothing left to give back: still fine
+    for part in np.array_split(universe, 8)[4:]:
+        vals = rng.integers(-9, 9, size=part.size).astype(np.float32)
+        t.push(to_dev(part, dev), to_dev(vals, dev))
+        o.push(part, vals)
+    assert capi.match(to_dev(sk, dev), to_dev(np.ones(sk.size, np.float32), dev), to_dev(sk, dev), dst, 1, capi.OP_PLUS) == sk.size
+    assert torch.all(dst == 2.0)
+    _check_dump(t, o, "after the trim")
+    t.close()
+    capi.device_trim()
+
+
 @pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
 def test_many_requests_in_flight_while_the_table_grows(capi, orc, dev, mode):
     """Device-resident requests are enqueued without waiting, so the host only has bounds on the
