@@ -128,6 +128,21 @@ def to_dev(a, dev):
     return torch.from_numpy(a).to(dev)
 
 
+def wake_gpu(dev, seconds=2.0):
+    """A fresh box hands over a GPU that has been idle: its first second of work runs slower than
+    every later one (the first of several identical runs on a box read 10-25 % low, later ones
+    agreed to 2 %). Untimed streaming work of a couple of seconds comes before anything is measured."""
+    import torch
+    x = torch.zeros(1 << 28, device=dev)
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            x.add_(1.0)
+        torch.cuda.synchronize()
+    del x
+    torch.cuda.empty_cache()
+
+
 def sampled(j, steps):
     """Whether timed step j (0-based) is one whose launches carry events: every SAMPLE_EVERY-th,
     and no more than a quarter of a short run (but the first step always)."""
@@ -1206,6 +1221,7 @@ def main():
     dev = torch.device("cuda:0")
     capi = graft.load_package().capi
     capi.load()  # raises if libpskv.so is missing: there is no other path
+    wake_gpu(dev)
 
     if args.workload == "sparse_lr":
         res, timed_batches, (n, S) = run_sparse_lr(args, capi, dev)

@@ -744,11 +744,13 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
   t->log_units[q % pskv_table::kLog] = units;
   t->pend_keys += n;
   t->pend_units += units;
-  // From a third of the way to the next growth on, every request leaves a record (its kernel's
-  // last workgroup writes four words): the host then knows how full the table is, give or take
-  // the requests in flight, early enough to have the next array allocated by the time it is needed.
+  // Close to a limit every request leaves a record; from a third of the way to the next growth on,
+  // every fourth one does (the election of a kernel's last workgroup costs a 1M-key launch about
+  // 6 us): the host then knows how full the table is early enough to have the next array allocated
+  // by the time it is needed.
   const double limit_now = (double)t->max_load * (double)t->cap;
-  const bool tight_slots = (double)(t->base_count + t->pend_keys + 2 * n) > 0.35 * limit_now;
+  const double reach = (double)(t->base_count + t->pend_keys + 2 * n);
+  const bool tight_slots = reach > limit_now || (reach > 0.35 * limit_now && q % 4 == 0);
   const bool tight_arena =
       units && (t->base_top + t->pend_units + 2 * units) * floats_per_unit > t->arena_cap;
   // (a base that merely grows old asks for a record every eighth request, not every one)
