@@ -36,14 +36,36 @@ inline void ThrowStatus(int rc, const char* where) {
   throw dmlc::Error(std::string(where) + ": " + pskv_last_error() + " (status " + std::to_string(rc) + ")");
 }
 
+namespace detail {
+/* The C ABI takes 64-bit keys. A ps-lite built with USE_KEY32 (include/ps/base.h:10-16) has 32-bit
+ * keys: the adapters widen them into a buffer of their own for the duration of the call (order,
+ * uniqueness and the key ranges of Postoffice::GetServerKeyRanges, which are uint64_t either way,
+ * are kept; responses share the request's own key buffer, kv_app.h:449, so nothing is narrowed). */
+template <typename K, bool kNative = sizeof(K) == 8>
+struct Keys64;
+template <typename K>
+struct Keys64<K, true> {
+  Keys64(const K* p, size_t) : ptr(reinterpret_cast<const uint64_t*>(p)) {}
+  const uint64_t* ptr;
+};
+template <typename K>
+struct Keys64<K, false> {
+  static_assert(sizeof(K) == 4, "ps::Key is 32 or 64 bits wide");
+  Keys64(const K* p, size_t n) : buf(n) {
+    for (size_t i = 0; i < n; ++i) buf[i] = static_cast<uint64_t>(p[i]);
+    ptr = buf.data();
+  }
+  std::vector<uint64_t> buf;
+  const uint64_t* ptr;
+};
+}  // namespace detail
+
 /* The KVWorker::Slicer that runs the boundary search and the lens sums on the GPU.
  * Copyable and re-entrant (KVWorker::Push may be called from several threads,
  * kv_app.h:101-104). The slices are zero-copy segments of the request, exactly like
  * the reference's (SArray::segment, sarray.h:248-255). */
 template <typename Val>
 class GpuSlicer {
-  static_assert(sizeof(ps::Key) == 8, "the GPU slicer handles 64-bit keys (USE_KEY32 is not supported)");
-
  public:
   using SlicedKVs = typename ps::KVWorker<Val>::SlicedKVs;
   explicit GpuSlicer(int device = 0) : device_(device) {}
@@ -58,7 +80,8 @@ class GpuSlicer {
       rb[i] = ranges[i].begin();
       re[i] = ranges[i].end();
     }
-    const int rc = pskv_slice(device_, reinterpret_cast<const uint64_t*>(send.keys.data()), send.keys.size(),
+    const detail::Keys64<ps::Key> keys(send.keys.data(), send.keys.size());
+    const int rc = pskv_slice(device_, keys.ptr, send.keys.size(),
                               reinterpret_cast<const int32_t*>(send.lens.data()), send.lens.size(),
                               send.vals.size(), rb.data(), re.data(), S, pos.data(), val_pos.data(),
                               used.data(), PSKV_MEM_HOST);
@@ -94,7 +117,6 @@ class GpuSlicer {
 template <typename Val>
 class GpuKVHandle {
   static_assert(std::is_same<Val, float>::value, "the GPU store holds float32 values");
-  static_assert(sizeof(ps::Key) == 8, "the GPU store handles 64-bit keys (USE_KEY32 is not supported)");
 
  public:
   explicit GpuKVHandle(const pskv_opts& opts) : table_(Create(opts)), mode_(opts.mode) {}
@@ -102,7 +124,8 @@ class GpuKVHandle {
 
   void operator()(const ps::KVMeta& req_meta, const ps::KVPairs<Val>& req_data, ps::KVServer<Val>* server) {
     const size_t n = req_data.keys.size();
-    const uint64_t* keys = reinterpret_cast<const uint64_t*>(req_data.keys.data());
+    const detail::Keys64<ps::Key> wide(req_data.keys.data(), n);
+    const uint64_t* keys = wide.ptr;
     const float* vals = req_data.vals.data();
     const int32_t* lens = reinterpret_cast<const int32_t*>(req_data.lens.data());
     const size_t nlens = mode_ == PSKV_MODE_VARLEN ? req_data.lens.size() : 0;
@@ -191,15 +214,15 @@ template <typename Val, typename C>
 size_t GpuOrderedMatch(const ps::SArray<ps::Key>& src_key, const ps::SArray<Val>& src_val,
                        const ps::SArray<ps::Key>& dst_key, C* dst_val, int k = 1, int op = PSKV_OP_ASSIGN,
                        int device = 0) {
-  static_assert(sizeof(ps::Key) == 8 && sizeof(Val) == 4, "64-bit keys, float values");
+  static_assert(sizeof(Val) == 4, "float values");
   if (k <= 0 || src_key.size() * static_cast<size_t>(k) != src_val.size())  // CHECK_EQ, :107
     throw dmlc::Error("GpuOrderedMatch: Check failed: src_key.size() * k == src_val.size()");
   dst_val->resize(dst_key.size() * static_cast<size_t>(k));  // :109
   if (dst_key.empty()) return 0;
   uint64_t matched = 0;
-  const int rc = pskv_match(device, reinterpret_cast<const uint64_t*>(src_key.data()), src_key.size(),
-                            reinterpret_cast<const float*>(src_val.data()),
-                            reinterpret_cast<const uint64_t*>(dst_key.data()), dst_key.size(),
+  const detail::Keys64<ps::Key> src(src_key.data(), src_key.size()), dst(dst_key.data(), dst_key.size());
+  const int rc = pskv_match(device, src.ptr, src_key.size(), reinterpret_cast<const float*>(src_val.data()),
+                            dst.ptr, dst_key.size(),
                             reinterpret_cast<float*>(dst_val->data()), static_cast<size_t>(k), op, &matched,
                             nullptr, PSKV_MEM_HOST);
   if (rc != PSKV_OK) ThrowStatus(rc, "GpuOrderedMatch");

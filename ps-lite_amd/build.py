@@ -70,6 +70,8 @@ def build_host_test():
            "-Wl,-rpath,$ORIGIN/../ps-lite_amd", "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib", "-lamdhip64",
            "-o", HOST_TEST]
     subprocess.run(cmd, check=True)
+    # the same program for a ps-lite built with 32-bit keys (USE_KEY32, include/ps/base.h:10-16)
+    subprocess.run(cmd[:-1] + [HOST_TEST + "32", "-DUSE_KEY32=1"], check=True)
     return HOST_TEST
 
 

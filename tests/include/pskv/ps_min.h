@@ -48,7 +48,11 @@ struct Error : public std::runtime_error {
 namespace ps {
 
 /* include/ps/base.h:15-18 */
+#if USE_KEY32  // (include/ps/base.h:10-16)
+using Key = uint32_t;
+#else
 using Key = uint64_t;
+#endif
 static const Key kMaxKey = std::numeric_limits<Key>::max();
 
 namespace detail {

@@ -59,11 +59,13 @@ def test_adapters_compile_with_in_process_surface(tmp_path):
                     str(tmp_path / "t.o")], check=True)
 
 
-def test_adapters_fit_real_pslite_headers(tmp_path):
-    """KVWorker::set_slicer / KVServer::set_request_handle of the real library accept the adapters."""
+@pytest.mark.parametrize("key32", [0, 1])
+def test_adapters_fit_real_pslite_headers(tmp_path, key32):
+    """KVWorker::set_slicer / KVServer::set_request_handle of the real library accept the adapters,
+    with its 64-bit keys and in a USE_KEY32 build (include/ps/base.h:10-16)."""
     if not os.path.exists(os.path.join(REFERENCE, "include", "ps", "ps.h")):
         pytest.skip("the reference tree is not present on this machine")
-    subprocess.run(["g++", "-std=c++11", "-I" + os.path.join(REFERENCE, "include"),
+    subprocess.run(["g++", "-std=c++11", "-DUSE_KEY32=%d" % key32, "-I" + os.path.join(REFERENCE, "include"),
                     "-I" + os.path.join(REPO, "include"), "-c",
                     os.path.join(REPO, "tests", "adapters_real_pslite_check.cc"), "-o", str(tmp_path / "c.o")],
                    check=True)
