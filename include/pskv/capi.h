@@ -268,6 +268,19 @@ void* pskv_host_alloc(size_t bytes);
 void pskv_host_free(void* ptr);
 int pskv_host_trim(void);
 
+/* What the sizing logic of a table has done so far (no counterpart in the reference; host-side
+ * bookkeeping, no device work): writes min(cap, PSKV_COUNTER_COUNT) values to out, in this order. */
+#define PSKV_COUNTER_REQUESTS 0        /* requests that could create keys */
+#define PSKV_COUNTER_GROWTHS 1         /* times the slot array was replaced by a larger one */
+#define PSKV_COUNTER_GROWTHS_UNASKED 2 /* ... decided from the host's bounds, without a wait */
+#define PSKV_COUNTER_GROWTHS_AHEAD 3   /* ... into an array that had been allocated ahead of need */
+#define PSKV_COUNTER_WAITS 4           /* waits for the stream to read exact counters */
+#define PSKV_COUNTER_CATCH_UPS 5       /* times the host let the device catch up on published counters */
+#define PSKV_COUNTER_RECORDS 6         /* requests that were asked to publish the counters */
+#define PSKV_COUNTER_SLOTS 7           /* slots of the array now */
+#define PSKV_COUNTER_COUNT 8
+int pskv_table_counters(pskv_table* t, uint64_t* out, size_t cap);
+
 /* Device memory the library keeps for reuse goes back to the system (no counterpart in the
  * reference): the slot arrays and row storage that growths have replaced (they stay in a
  * memory pool of the library, one per device, because releasing a few hundred MB costs

@@ -41,7 +41,7 @@ SYMBOLS = [
     "pskv_table_create", "pskv_table_destroy", "pskv_push", "pskv_pull", "pskv_pushpull",
     "pskv_sync", "pskv_table_stream", "pskv_push_multi", "pskv_pull_multi", "pskv_sync_multi", "pskv_size", "pskv_dump", "pskv_slice", "pskv_slice_noalloc", "pskv_server_ranges",
     "pskv_assemble_pull", "pskv_match", "pskv_prof_enable", "pskv_prof_reset", "pskv_prof_read", "pskv_prof_samples",
-    "pskv_copy_probe", "pskv_host_alloc", "pskv_host_free", "pskv_host_trim", "pskv_device_trim", "pskv_last_error",
+    "pskv_copy_probe", "pskv_host_alloc", "pskv_host_free", "pskv_host_trim", "pskv_device_trim", "pskv_table_counters", "pskv_last_error",
     "pskv_version",
 ]
 
@@ -108,6 +108,7 @@ def load():
     lib.pskv_host_free.argtypes = [vp]
     lib.pskv_host_free.restype = None
     lib.pskv_device_trim.argtypes = [i32]
+    lib.pskv_table_counters.argtypes = [vp, vp, sz]
     lib.pskv_last_error.restype = ctypes.c_char_p
     lib.pskv_version.restype = ctypes.c_char_p
     _lib = lib
@@ -245,6 +246,13 @@ class Table(_Holder):
         nk, nv = ctypes.c_uint64(0), ctypes.c_uint64(0)
         _check(self._lib.pskv_size(self._h, ctypes.byref(nk), ctypes.byref(nv)))
         return nk.value, nv.value
+
+    def counters(self):
+        """What the table's sizing logic has done so far, by name (pskv_table_counters)."""
+        out = np.zeros(8, np.uint64)
+        _check(self._lib.pskv_table_counters(self._h, out.ctypes.data, out.size))
+        names = ("requests", "growths", "growths_unasked", "growths_ahead", "waits", "catch_ups", "records", "slots")
+        return {k: int(v) for k, v in zip(names, out)}
 
     def dump(self):
         """(keys sorted, lens, vals) as numpy arrays."""

@@ -2139,6 +2139,16 @@ int pskv_copy_probe(pskv_table* t, void* dst, const void* src, size_t bytes) {
   return PSKV_OK;
 }
 
+int pskv_table_counters(pskv_table* t, uint64_t* out, size_t cap) {
+  clear_error();
+  if (!t || (!out && cap)) return set_error(PSKV_EINVAL, "null argument");
+  const uint64_t v[PSKV_COUNTER_COUNT] = {t->stats.requests, t->stats.growths, t->stats.growths_unasked,
+                                          t->stats.spare_used, t->stats.waits, t->stats.catch_ups,
+                                          t->stats.records, t->cap};
+  for (size_t i = 0; i < cap && i < (size_t)PSKV_COUNTER_COUNT; ++i) out[i] = v[i];
+  return PSKV_OK;
+}
+
 int pskv_device_trim(int device) {
   clear_error();
   if (device < 0 || device >= 64) return set_error(PSKV_EINVAL, "device %d out of range", device);

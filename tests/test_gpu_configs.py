@@ -180,6 +180,9 @@ def test_config2_as_the_benchmark_runs_it(capi, orc, dev):
             want[a:b] = stores[s].pull(keys[a:b])[0]
         assert_bits_equal(from_dev(outs[p]), want, "pull of step %d" % p)
     for s in range(S):
+        c = group.tables[s].counters()
+        # every table grew (from 4M slots) without ever waiting for the stream to size itself
+        assert c["growths"] >= 1 and c["growths_unasked"] == c["growths"] and c["waits"] == 0, c
         assert group.tables[s].size() == stores[s].size(), s
         held += group.tables[s].size()[0]
     assert held == np.unique(np.concatenate([k for k, _ in batches])).size

@@ -625,6 +625,40 @@ def test_varlen_errors(capi, orc, dev):
     assert e.value.code == capi.ESIZE_MISMATCH and t.last_out_nvals == 5
 
 
+def test_refused_push_still_publishes_its_counters(capi, orc, dev):
+    """Close to a limit the host asks the request's own kernel for the counters as they are after
+    it, and sizes the next request from that record instead of waiting for the stream. A var-len
+    push that the device refuses (its lens do not add up to the values it brought) changes no
+    counter but must leave its record all the same, or the host would count its keys as pending
+    for good and wait for exact counters before every later request."""
+    import time
+    announce("refused_push_publishes")
+    rng = np.random.default_rng(321)
+    n, row = 1000, 16
+    keys = [unique_keys(rng, n) for _ in range(3)]
+    lens = np.full(n, row, np.int32)
+    vals = rng.integers(-5, 5, size=n * row).astype(np.float32)
+    # room for two requests and a half by the host's upper bound (rows + one unit per key + padding)
+    t = capi.Table(capi.MODE_VARLEN, initial_capacity=8 * n, arena_floats=52000)
+    o = orc.Store(orc.MODE_VARLEN)
+    t.push(to_dev(keys[0], dev), to_dev(vals, dev), to_dev(lens, dev))
+    o.push(keys[0], vals, lens)
+    t.sync()
+    before = t.counters()
+    t.push(to_dev(keys[1], dev), to_dev(vals[:-4], dev), to_dev(lens, dev))  # four floats short: refused on the device
+    time.sleep(0.05)  # (the device gets there; nothing here waits for it)
+    t.push(to_dev(keys[2], dev), to_dev(vals, dev), to_dev(lens, dev))
+    o.push(keys[2], vals, lens)
+    after = t.counters()
+    assert after["waits"] == before["waits"], (before, after)
+    assert after["growths"] == before["growths"], (before, after)
+    with pytest.raises(capi.PskvError) as e:
+        t.sync()
+    assert e.value.code == capi.ESIZE_MISMATCH
+    t.sync()
+    _check_dump(t, o, "after the refused push")
+
+
 def test_varlen_pull_without_host_round_trip(capi, orc, dev):
     """out_nvals == NULL keeps a var-len pull asynchronous: the kernels take the response size from
     the device-side scan. Too small a buffer writes nothing and is reported by the next sync."""
