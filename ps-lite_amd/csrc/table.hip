@@ -156,6 +156,7 @@ struct pskv_table {
   uint64_t log_keys[kLog] = {0}, log_units[kLog] = {0};
   Snapshot* snap = nullptr;  // pinned host memory the device publishes into
   uint64_t record_seq = ~0ull;  // the newest request that was asked to publish its counters (all ones: none yet)
+  double new_share = 0.0;  // share of the keys named by requests that were new, over the latest records
   DevState* st = nullptr;  // device
   StateView* st_host = nullptr;  // pinned: what read_state() last read of the device state
 
@@ -509,9 +510,16 @@ void adopt_snapshot(pskv_table* t) {
   std::atomic_thread_fence(std::memory_order_acquire);
   const uint64_t s0 = sn->seq_begin;
   if (s0 != s1 || s1 < t->base_seq || s1 >= t->seq) return;  // (the initial record is all ones)
+  uint64_t named = 0;
   for (uint64_t r = t->base_seq; r <= s1; ++r) {
+    named += t->log_keys[r % pskv_table::kLog];
     t->pend_keys -= t->log_keys[r % pskv_table::kLog];
     t->pend_units -= t->log_units[r % pskv_table::kLog];
+  }
+  // which share of the keys that requests named turned out to be new, lately (a moving average)
+  if (named) {
+    const double share = c > t->base_count ? std::min(1.0, (double)(c - t->base_count) / (double)named) : 0.0;
+    t->new_share = 0.5 * t->new_share + 0.5 * share;
   }
   t->base_seq = s1 + 1;
   t->base_count = c;
@@ -629,7 +637,11 @@ void prepare_growth(pskv_table* t) {
   if (t->spare || t->spare_job || t->no_growth) return;
   adopt_snapshot(t);  // (a read of pinned memory)
   const double limit = (double)t->max_load * (double)t->cap;
-  if ((double)t->base_count <= 0.4 * limit) return;
+  // the keys known to be held, plus, while requests have mostly been bringing new keys, the share of
+  // the keys in flight that will be new if that goes on (a caller that runs far ahead of the device
+  // would otherwise learn too late how full the table is)
+  const double expected = (double)t->base_count + (t->new_share >= 0.5 ? t->new_share * (double)t->pend_keys : 0.0);
+  if (expected <= 0.4 * limit) return;
   const uint64_t want = grown_cap(t, 0);
   if (want * sizeof(Slot) > kSpareMaxBytes) return;
   std::shared_ptr<AllocJob> job = std::make_shared<AllocJob>();
@@ -972,11 +984,11 @@ int run_scalar(Batch& bt, bool push, bool pull) {
       if (push || use[i] == kScRecord) t->cache_valid = false;
     }
     TableReq& d = it.d;
-    if (use[i] != kScTry && scalar_cache_eligible(t, r)) {
-      // Room for this request in the cache, whether or not it is recorded: a table that sees
-      // requests of this size allocates once, on the first of them, and not in the middle of a
-      // run when the cache comes into use. (The cache has been written back above; kScTry needs
-      // nothing: the buffers have the cached request's size.)
+    if (use[i] == kScRecord) {
+      // Room for this request in the cache (it has been written back above; kScTry needs nothing:
+      // the buffers have the cached request's size). Only a request that is going to be recorded
+      // pays for it: a one-off pull of 16M keys would otherwise allocate 256 MB it never uses, and
+      // wait for the stream to do so.
       rc = grow(t, &t->cache_keys, r.n * sizeof(uint64_t));
       if (rc) return rc;
       rc = grow(t, &t->sc_vals, r.n * sizeof(float));
@@ -1250,7 +1262,10 @@ int run_varlen(Batch& bt, bool push, bool pull) {
     n_largest = std::max(n_largest, it.r.n);
   }
   if (!n_largest) return PSKV_OK;
-  const int items = scan_items(n_largest);
+  // (keys per thread of the key-by-key kernels: by the keys of the whole launch, not of its largest table)
+  uint64_t n_launch = 0;
+  for (const Item& it : bt) n_launch += it.r.n;
+  const int items = scan_items(n_launch);
   const bool async_pull = pull && !push && !bt[0].r.need_total;
   for (Item& it : bt) {
     pskv_table* t = it.t;
