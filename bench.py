@@ -145,7 +145,7 @@ def wake_gpu(dev, seconds=2.0):
 
 def sampled(j, steps):
     """Whether timed step j (0-based) is one whose launches carry events: every SAMPLE_EVERY-th,
-    and no more than a quarter of a short run (but the first step always)."""
+    and no more than that share of a short run (but the first step always)."""
     return j >= 0 and j % SAMPLE_EVERY == 0 and j // SAMPLE_EVERY < max(1, steps // SAMPLE_EVERY)
 
 
