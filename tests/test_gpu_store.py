@@ -135,6 +135,30 @@ def test_growth_by_every_factor(capi, orc, dev, max_load, first, step):
     _check_dump(t, o, "growth")
 
 
+@pytest.mark.parametrize("max_load,first,second", [(0.5, 1500, 3000), (0.9, 3500, 6000)])
+def test_growth_by_eight(capi, orc, dev, max_load, first, second):
+    """A request that needs between four and eight times the slots makes the array eight times as
+    large in one streaming move (the largest factor that goes that way): 4,096 slots that hold
+    `first` keys, at a fill of 0.37 or 0.85 (long probe chains, some wrapped around the end of the
+    array), become 32,768."""
+    announce("growth_by_eight", max_load)
+    rng = np.random.default_rng(int(max_load * 10))
+    t = capi.Table(capi.MODE_SCALAR, initial_capacity=2000, max_load=max_load)
+    o = orc.Store(orc.MODE_SCALAR)
+    universe = unique_keys(rng, first + second)
+    perm = rng.permutation(universe.size)
+    a, b = np.sort(universe[perm[:first]]), np.sort(universe[perm[first:]])
+    for keys in (a, b):
+        vals = rng.integers(-50, 50, size=keys.size).astype(np.float32)
+        if keys is a:
+            assert t.counters()["slots"] == 4096
+        t.push(to_dev(keys, dev), to_dev(vals, dev))
+        o.push(keys, vals)
+    c = t.counters()
+    assert c["slots"] == 32768 and c["growths"] == 1 and c["waits"] == 0, c
+    _check_dump(t, o, "growth by eight")
+
+
 def test_growth_of_a_large_array_by_two(capi, orc, dev):
     """Arrays beyond 64 MB double: 4.6M keys take a table through 4x growths and then a 2x one."""
     announce("growth_of_a_large_array")
