@@ -290,15 +290,7 @@ struct SliceCtx {
   size_t dev_bytes = 0;
   void* pinned = nullptr;   // pinned host memory the kernels read targets from and answer into
   size_t pinned_bytes = 0;
-  void* stage = nullptr;    // device copy of host-resident keys / lens
-  size_t stage_bytes = 0;
-  void* small = nullptr;    // pinned, kSmallStage bytes: small host-resident keys / lens, read in place
 };
-
-// Host-resident keys (+ lens) up to this size are not copied to the device: the search reads
-// a few hundred of them, and the sums one pass, straight from pinned host memory.
-constexpr size_t kSmallStage = 1024u << 10;
-
 
 std::mutex g_pool_mu;
 std::vector<SliceCtx*> g_pool;
@@ -342,7 +334,7 @@ struct CtxLease {
   }
 };
 
-int ctx_reserve(SliceCtx* c, size_t dev_bytes, size_t pinned_bytes, size_t stage_bytes) {
+int ctx_reserve(SliceCtx* c, size_t dev_bytes, size_t pinned_bytes) {
   if (dev_bytes > c->dev_bytes) {
     if (c->dev) PSKV_HIP(hipFree(c->dev));
     c->dev = nullptr;
@@ -357,13 +349,6 @@ int ctx_reserve(SliceCtx* c, size_t dev_bytes, size_t pinned_bytes, size_t stage
     // coherent: never cached by the GPU, so every call sees what the host wrote for it
     PSKV_HIP(hipHostMalloc(&c->pinned, pinned_bytes, hipHostMallocCoherent));
     c->pinned_bytes = pinned_bytes;
-  }
-  if (stage_bytes > c->stage_bytes) {
-    if (c->stage) PSKV_HIP(hipFree(c->stage));
-    c->stage = nullptr;
-    c->stage_bytes = 0;
-    PSKV_HIP(hipMalloc(&c->stage, stage_bytes));
-    c->stage_bytes = stage_bytes;
   }
   return PSKV_OK;
 }
@@ -422,7 +407,7 @@ int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, 
 
   const bool do_sums = has_lens && nlens == n;
   if (n && do_sums && S > 65535) return set_error(PSKV_EINVAL, "more than 65535 ranges with lens");
-  bool sums_on_device = n != 0;  // (device-resident requests: searches and sums on the GPU)
+  bool on_device = n != 0;  // (device-resident requests: searches and sums on the GPU)
   if (n && memkind == PSKV_MEM_HOST) {
     // Keys in host memory are searched where they lie: S+1 lower bounds touch (S+1) log2 n keys,
     // and shipping all n keys over the host link for that would cost milliseconds at model size
@@ -440,7 +425,7 @@ int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, 
     }
     // The lens too: one core adds them up faster (8 MB in 0.2 ms) than pageable memory crosses the
     // host link (0.28 ms for the same 8 MB, before any kernel runs): the walk of kv_app.h:563-565.
-    sums_on_device = false;
+    on_device = false;
     if (do_sums) {
       for (size_t i = 0; i < S; ++i) {
         uint64_t sum = 0;
@@ -450,7 +435,7 @@ int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, 
     }
   }
 
-  if (sums_on_device) {
+  if (on_device) {
     DeviceGuard guard(device);
     if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", device);
     CtxLease lease(device);
@@ -459,7 +444,7 @@ int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, 
     lease.idle = false;
     // device: lb[S+1] | pos[S+1] | sums[S]      pinned: targets[S+1] | pos[S+1] | sums[S]
     const size_t arr = pad256((S + 2) * 8);  // S+1 positions and the word that says they are there
-    int rc = ctx_reserve(c, 3 * arr, 3 * arr, 0);
+    int rc = ctx_reserve(c, 3 * arr, 3 * arr);
     if (rc) return rc;
     char* d = static_cast<char*>(c->dev);
     uint64_t* d_lb = reinterpret_cast<uint64_t*>(d);
@@ -666,7 +651,7 @@ int pskv_assemble_pull(int device, const uint64_t* req_keys, size_t n, size_t R,
     // pinned, read and written by the kernels in place:
     //   key pointers[R] | nkeys[R] | targets[2R] | lower bounds[2R] | segments[2R]
     const size_t a = pad256(R * 8), b = pad256(2 * R * 8), sg = pad256(2 * R * sizeof(Segment));
-    int rc = ctx_reserve(c, 0, 2 * a + 2 * b + sg, 0);
+    int rc = ctx_reserve(c, 0, 2 * a + 2 * b + sg);
     if (rc) return rc;
     char* h = static_cast<char*>(c->pinned);
     const uint64_t** h_ptrs = reinterpret_cast<const uint64_t**>(h);
