@@ -1271,6 +1271,16 @@ def main():
         if orc is not None:
             log("extra: plumbing")
             extra["plumbing"] = extra_plumbing(capi, orc)
+        # stable key sets (the same keys every step) and the ordered match of two sorted key sets
+        log("extra: sparse_repeat")
+        sub.steps, sub.warmup = 10, 3
+        rres, rin = run_sparse_repeat(sub, capi, dev)
+        extra["sparse_repeat"] = brief(rres, cpu_sparse_repeat(orc, *rin, budget_s=3.0) if orc is not None else None)
+        del rin
+        log("extra: match")
+        mres, min_ = run_match(sub, capi, dev)
+        extra["match"] = brief(mres, cpu_match(orc, *min_, budget_s=3.0) if orc is not None else None)
+        del min_
 
     cpu = None
     if not args.no_cpu:
