@@ -177,8 +177,12 @@ int pskv_dump(pskv_table* t, uint64_t* keys, int32_t* lens, size_t cap_keys, flo
  * val_pos[S+1] so that it holds vals [val_pos[i], val_pos[i+1]), used[S] = the
  * `first` flag of the slice (0 for an empty slice). keys/lens follow memkind;
  * lens == NULL or nlens == 0 means no lens (value length k = nvals / n).
- * `device` selects the GPU for PSKV_MEM_HOST inputs and must be the device that
- * holds PSKV_MEM_DEVICE inputs. */
+ * `device` must be the device that holds PSKV_MEM_DEVICE inputs: those are searched (and their
+ * lens added up per slice) by HIP kernels, one launch and one wait. PSKV_MEM_HOST inputs are
+ * sliced where they lie, on the calling thread, with the reference's own loop: S+1 binary
+ * searches touch a few dozen keys, and shipping n keys over the host link for them would cost
+ * milliseconds at model size (this is by design, not a fallback: with PSKV_MEM_DEVICE inputs and
+ * no GPU the call fails with PSKV_EHIP). */
 int pskv_slice(int device, const uint64_t* keys, size_t n, const int32_t* lens, size_t nlens,
                size_t nvals, const uint64_t* range_begin, const uint64_t* range_end, size_t S,
                uint64_t* pos, uint64_t* val_pos, uint8_t* used, int memkind);
