@@ -495,6 +495,28 @@ def cpu_dense(orc, nk=64, k=4194304, sample_keys=16, budget_s=10.0):
 # ------------------------------------------------------------------------------------
 # varlen: configs[4]
 # ------------------------------------------------------------------------------------
+def timed_replays(rec, group, steps, ref, add):
+    """Times `steps` runs of a recorded push + pull step (after two untimed ones). `ref` holds the sums a
+    sample of the values has reached; every application of the step adds `add` to it. Returns the entry
+    for the result line and the sums the sample must have reached."""
+    ref = ref + add  # recording a request serves it once
+    for _ in range(2):
+        rec.run()
+        ref = ref + add
+    group.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        rec.run()
+    t_host = time.perf_counter() - t0
+    group.sync()
+    dt = time.perf_counter() - t0
+    for _ in range(steps):
+        ref = ref + add
+    return {"ms_per_step": dt / steps * 1e3, "host_us_per_step": t_host / steps * 1e6,
+            "note": "the same step kept as a HIP graph by pskv_replay_record and applied by pskv_replay_run: "
+                    "one call, one launch, nothing sliced, allocated or waited for per step"}, ref
+
+
 def gen_varlen(n, S):
     limit = (KMAX // S) * S
     keys = unique_sorted_keys(np.random.default_rng(0xE3B), n, limit)
@@ -573,6 +595,15 @@ def run_varlen(args, capi, dev):
     for _ in range(1 + args.warmup + args.steps):
         ref = ref + dv[idx]
     assert torch.equal(out[idx], ref), "var-len sums differ from sequential float adds"
+    replayed = None
+    if not per_table:
+        # the same step recorded once (pskv_replay_record) and replayed: no slicing, one call and one launch
+        pos, vpos, _ = capi.slice_keys(dk, rb, re, lens=dl, nvals=nvals)
+        rec = group.record(capi.REPLAY_PUSH | capi.REPLAY_PULL, dk, pos, dv, vpos, dl, out, vpos, out_lens)
+        replayed, ref = timed_replays(rec, group, args.steps, ref, dv[idx])
+        assert torch.equal(out_lens, dl), "pulled lens differ"
+        assert torch.equal(out[idx], ref), "replayed var-len sums differ from sequential float adds"
+        rec.close()
     # on request, once more with the library's default of one stream per table (launches of
     # different ranges overlap; durations are then no longer a kernel's own, hence not the headline)
     dt_own = None
@@ -607,6 +638,8 @@ def run_varlen(args, capi, dev):
                                                  traffic("rows_gather_varlen", floats_per_launch), gat[2]),
                                         bytes_per_float=8)},
     }
+    if replayed is not None:
+        res["replayed"] = dict(replayed, value=2.0 * n / (replayed["ms_per_step"] * 1e-3), unit="keys/s")
     if dt_own is not None:
         res["own_streams"] = {"value": 2.0 * n * args.steps / dt_own, "unit": "keys/s",
                               "ms_per_step": dt_own / args.steps * 1e3,
@@ -846,7 +879,8 @@ def run_sparse_repeat(args, capi, dev):
     # Room for the requests in flight: until the device has answered, the host must assume that a
     # request creates all its keys, and a table without that room makes every request wait for exact
     # counters first (the sums would be the same, the steps about a quarter slower).
-    t = capi.Table(capi.MODE_SCALAR, initial_capacity=int(n * 6))
+    group = capi.Group(1, capi.MODE_SCALAR, initial_capacity=int(n * 6))
+    t = group.tables[0]
     torch.cuda.synchronize()
     kp, vp, op = dk.data_ptr(), dv.data_ptr(), out.data_ptr()
 
@@ -875,9 +909,32 @@ def run_sparse_repeat(args, capi, dev):
         ref = ref + dv[idx]
     assert torch.equal(out[idx], ref), "sums differ from sequential float adds"
     assert t.size()[0] == n
+    # the same step as ONE request with both halves (KVWorker::PushPull, meta.push && meta.pull)
+    for _ in range(2):
+        t.pushpull_raw(kp, n, vp, n, op, n)
+    t.sync()
+    t1 = time.perf_counter()
+    for _ in range(args.steps):
+        t.pushpull_raw(kp, n, vp, n, op, n)
+    t.sync()
+    dt_pp = time.perf_counter() - t1
+    for _ in range(2 + args.steps):
+        ref = ref + dv[idx]
+    assert torch.equal(out[idx], ref), "push+pull sums differ from sequential float adds"
+    # the same step recorded once (pskv_replay_record) and replayed: one call and one launch per step
+    whole = np.array([0, n], np.uint64)
+    rec = group.record(capi.REPLAY_PUSH | capi.REPLAY_PULL, dk, whole, dv, whole, None, out)
+    replayed, ref = timed_replays(rec, group, args.steps, ref, dv[idx])
+    assert torch.equal(out[idx], ref), "replayed sums differ from sequential float adds"
+    rec.close()
     res = {
         "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
         "dtype": "f32",
+        "replayed": dict(replayed, value=2.0 * n / (replayed["ms_per_step"] * 1e-3), unit="keys/s",
+                         one_request={"ms_per_step": dt_pp / args.steps * 1e3, "value": 2.0 * n * args.steps / dt_pp,
+                                      "unit": "keys/s",
+                                      "note": "the step as one pskv_pushpull request, not recorded: what a recorded "
+                                              "SCALAR push + pull is replayed as"}),
         "config": {"workload": "sparse_repeat: the same 16M sorted unique uint64 keys pushed (fresh values) "
                                "and pulled every step, one table", "keys_per_step": n, "ranges": 1,
                    "value_len": 1, "key_dtype": "u64"},
@@ -1150,6 +1207,49 @@ def extra_plumbing(capi, orc, reps=5):
                                                        "both sides), median of %d runs" % reps}}
 
 
+def extra_replay_small(capi, dev, n=100000, S=4, steps=200):
+    """A step whose kernels are short, where the host side decides: the same 100,000 keys over 4 key
+    ranges, slice + pskv_push_multi + pskv_pull_multi per step against one pskv_replay_run per step.
+    The sums are checked against their closed form both ways."""
+    import torch
+    rng = np.random.default_rng(0x4E9)
+    keys = unique_sorted_keys(rng, n, (KMAX // S) * S)
+    dk = to_dev(keys, dev)
+    dv = torch.randn(n, device=dev) * 0.01
+    out = torch.empty(n, dtype=torch.float32, device=dev)
+    rb, re = capi.server_ranges(S)
+    group = capi.Group(S, capi.MODE_SCALAR, initial_capacity=n)
+    torch.cuda.synchronize()
+    kp, vp, op = dk.data_ptr(), dv.data_ptr(), out.data_ptr()
+
+    def step():
+        pos, _, _ = capi.slice_keys(dk, rb, re, nvals=n)
+        group.push_raw(kp, pos, vp, pos)
+        group.pull_raw(kp, pos, op)
+
+    for _ in range(5):
+        step()
+    group.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    group.sync()
+    dt = time.perf_counter() - t0
+    ref = torch.zeros(n, device=dev)
+    for _ in range(5 + steps):
+        ref = ref + dv
+    assert torch.equal(out, ref), "sums differ from sequential float adds"
+    pos, _, _ = capi.slice_keys(dk, rb, re, nvals=n)
+    rec = group.record(capi.REPLAY_PUSH | capi.REPLAY_PULL, dk, pos, dv, pos, None, out)
+    replayed, ref = timed_replays(rec, group, steps, ref, dv)
+    assert torch.equal(out, ref), "replayed sums differ from sequential float adds"
+    rec.close()
+    group.close()
+    return {"workload": "the same %d keys over %d key ranges pushed and pulled every step (SCALAR)" % (n, S),
+            "steps": steps, "ms_per_step": dt / steps * 1e3, "value": 2.0 * n * steps / dt, "unit": "keys/s",
+            "replayed": dict(replayed, value=2.0 * n / (replayed["ms_per_step"] * 1e-3), unit="keys/s")}
+
+
 def extra_host_staged(capi, reps=2, nk=64, k=4194304):
     """configs[2] from and to ordinary (pageable) host memory, as a server gets it from the
     transport: 1 GiB per push and per pull through PSKV_MEM_HOST. PCIe-inclusive, never `value`."""
@@ -1182,7 +1282,7 @@ def extra_host_staged(capi, reps=2, nk=64, k=4194304):
 
 def brief(res, cpu=None):
     """What an `extra` entry keeps of a workload's result."""
-    out = {k: res[k] for k in ("value", "unit", "ms_per_step", "gbps", "phases") if k in res}
+    out = {k: res[k] for k in ("value", "unit", "ms_per_step", "gbps", "phases", "replayed") if k in res}
     out["workload"] = res["config"]["workload"]
     out["roofline"] = res["roofline"]
     out["kernels"] = res.get("kernels")
@@ -1277,6 +1377,7 @@ def main():
         rres, rin = run_sparse_repeat(sub, capi, dev)
         extra["sparse_repeat"] = brief(rres, cpu_sparse_repeat(orc, *rin, budget_s=3.0) if orc is not None else None)
         del rin
+        extra["replay_small"] = extra_replay_small(capi, dev)
         log("extra: match")
         mres, min_ = run_match(sub, capi, dev)
         extra["match"] = brief(mres, cpu_match(orc, *min_, budget_s=3.0) if orc is not None else None)
@@ -1315,7 +1416,7 @@ def main():
         "kernel; read at run time from " + ", ".join(sorted(TRAFFIC_SOURCES))) if TRAFFIC_SOURCES else None
     if "gbps" in res:
         line["gbps"] = res["gbps"]
-    for k in ("own_streams", "presized", "per_table", "multi"):
+    for k in ("own_streams", "presized", "per_table", "multi", "replayed"):
         if k in res:
             extra[k] = res[k]
     if "phases" in res:

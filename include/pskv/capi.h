@@ -54,6 +54,7 @@ extern "C" {
 #define PSKV_EINVAL (-5)
 #define PSKV_ERANGE_GAP (-6)     /* ranges[i-1].end != ranges[i].begin: kv_app.h:533 */
 #define PSKV_ELEN_CHANGED (-7)   /* var-len push with a length that differs from the stored row */
+#define PSKV_ESTALE (-8)         /* a recorded request (pskv_replay_*) no longer fits its tables or its keys */
 
 #define PSKV_MEM_HOST 0
 #define PSKV_MEM_DEVICE 1
@@ -154,6 +155,37 @@ int pskv_pull_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, c
 /* pskv_sync for all tables of a group with one wait: returns the first deferred error (every
  * table's error state is cleared). */
 int pskv_sync_multi(pskv_table* const* tables, size_t S);
+
+/* A request that repeats, recorded once and replayed with ONE launch. The reference's own test
+ * pushes the same keys over and over (tests/test_kv_app.cc:36-44), and so does a worker that
+ * trains a dense model: per step KVWorker::Send delivers the same keys in the same slices
+ * (kv_app.h:574-613) and only the values differ. pskv_replay_record serves such a request once,
+ * exactly as pskv_push_multi (what = PSKV_REPLAY_PUSH), pskv_pull_multi (PSKV_REPLAY_PULL) or
+ * the one followed by the other (PSKV_REPLAY_PUSH | PSKV_REPLAY_PULL) would, with the same
+ * arguments (device memory only; out_vals, out_pos and out_lens as pskv_pull_multi's out,
+ * out_pos and out_lens; a PSKV_MODE_VARLEN response that does not fit is reported by the next
+ * sync), waits for it, and keeps the launches that a repeat of it takes as a HIP graph on the
+ * tables' stream (which must not be the null stream). It allocates and waits; it is a set-up call.
+ * pskv_replay_run enqueues that graph: the request is applied again, to whatever the value
+ * buffers hold by the time the stream gets to it (keys, lens, positions and addresses are part
+ * of the recording). It allocates nothing, waits for nothing and reads nothing back: the host
+ * side of a step is this one call.
+ * A replay creates no key and moves no buffer, and the host sizes nothing for it. The device
+ * therefore checks first, table by table, that the key (and lens) buffers still hold what was
+ * recorded; a table whose slice has changed is left as it is by that run, its part of a pull
+ * is not written, and the next pskv_sync / pskv_sync_multi reports PSKV_ESTALE for it.
+ * Any other request on one of the tables (pskv_push, pskv_pull, pskv_dump, another recording)
+ * may move what the recording points at, so it ends the recording's life: pskv_replay_run then
+ * returns PSKV_ESTALE and enqueues nothing; record again. pskv_sync, pskv_sync_multi and
+ * pskv_size may be called between runs. Destroy a recording before its tables. */
+typedef struct pskv_replay pskv_replay;
+#define PSKV_REPLAY_PUSH 1
+#define PSKV_REPLAY_PULL 2
+int pskv_replay_record(pskv_replay** out, pskv_table* const* tables, size_t S, int what, const uint64_t* keys,
+                       const uint64_t* pos, const float* vals, const uint64_t* val_pos, const int32_t* lens,
+                       float* out_vals, const uint64_t* out_pos, int32_t* out_lens);
+int pskv_replay_run(pskv_replay* r);
+int pskv_replay_destroy(pskv_replay* r);
 
 /* Waits for everything enqueued on the table and reports a deferred device-side
  * error (PSKV_ELEN_CHANGED) of an earlier asynchronous push, once. */

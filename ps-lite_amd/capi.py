@@ -20,6 +20,9 @@ EHIP = -4
 EINVAL = -5
 ERANGE_GAP = -6
 ELEN_CHANGED = -7
+ESTALE = -8
+REPLAY_PUSH = 1
+REPLAY_PULL = 2
 MEM_HOST = 0
 MEM_DEVICE = 1
 MODE_SCALAR = 0
@@ -33,13 +36,13 @@ KERNEL_PUSH_SCALAR, KERNEL_PULL_SCALAR, KERNEL_ROWS_ACC, KERNEL_ROWS_GATHER, KER
 ERROR_NAMES = {
     EUNCOVERED_KEY: "PSKV_EUNCOVERED_KEY", ESIZE_MISMATCH: "PSKV_ESIZE_MISMATCH",
     ENOMEM: "PSKV_ENOMEM", EHIP: "PSKV_EHIP", EINVAL: "PSKV_EINVAL",
-    ERANGE_GAP: "PSKV_ERANGE_GAP", ELEN_CHANGED: "PSKV_ELEN_CHANGED",
+    ERANGE_GAP: "PSKV_ERANGE_GAP", ELEN_CHANGED: "PSKV_ELEN_CHANGED", ESTALE: "PSKV_ESTALE",
 }
 
 # every symbol include/pskv/capi.h declares
 SYMBOLS = [
     "pskv_table_create", "pskv_table_destroy", "pskv_push", "pskv_pull", "pskv_pushpull",
-    "pskv_sync", "pskv_table_stream", "pskv_push_multi", "pskv_pull_multi", "pskv_sync_multi", "pskv_size", "pskv_dump", "pskv_slice", "pskv_slice_noalloc", "pskv_server_ranges",
+    "pskv_sync", "pskv_table_stream", "pskv_push_multi", "pskv_pull_multi", "pskv_sync_multi", "pskv_replay_record", "pskv_replay_run", "pskv_replay_destroy", "pskv_size", "pskv_dump", "pskv_slice", "pskv_slice_noalloc", "pskv_server_ranges",
     "pskv_assemble_pull", "pskv_match", "pskv_prof_enable", "pskv_prof_reset", "pskv_prof_read", "pskv_prof_samples",
     "pskv_copy_probe", "pskv_host_alloc", "pskv_host_free", "pskv_host_trim", "pskv_device_trim", "pskv_table_counters", "pskv_last_error",
     "pskv_version",
@@ -90,6 +93,9 @@ def load():
     lib.pskv_push_multi.argtypes = [vp, sz, vp, vp, vp, vp, vp, i32]
     lib.pskv_pull_multi.argtypes = [vp, sz, vp, vp, vp, vp, vp, vp, i32]
     lib.pskv_sync_multi.argtypes = [vp, sz]
+    lib.pskv_replay_record.argtypes = [ctypes.POINTER(vp), vp, sz, i32, vp, vp, vp, vp, vp, vp, vp, vp]
+    lib.pskv_replay_run.argtypes = [vp]
+    lib.pskv_replay_destroy.argtypes = [vp]
     lib.pskv_size.argtypes = [vp, ctypes.POINTER(u64), ctypes.POINTER(u64)]
     lib.pskv_dump.argtypes = [vp, vp, vp, sz, vp, sz, ctypes.POINTER(sz), ctypes.POINTER(sz)]
     lib.pskv_slice.argtypes = [i32, vp, sz, vp, sz, sz, vp, vp, sz, vp, vp, vp, i32]
@@ -237,6 +243,11 @@ class Table(_Holder):
         _check(self._lib.pskv_pull(self._h, keys_ptr, n, out_ptr, out_cap, out_lens_ptr, None,
                                    MEM_DEVICE))
 
+    def pushpull_raw(self, keys_ptr, n, vals_ptr, nvals, out_ptr, out_cap):
+        """pskv_pushpull (one request with both halves) on raw device addresses, SCALAR / FIXED tables."""
+        _check(self._lib.pskv_pushpull(self._h, keys_ptr, n, vals_ptr, nvals, None, 0, out_ptr, out_cap, None, None,
+                                       MEM_DEVICE))
+
     def sync(self):
         rc = self._lib.pskv_sync(self._h)
         self._release()
@@ -367,12 +378,55 @@ class Group(_Holder):
         self._release()
         _check(rc)
 
+    def record(self, what, keys, pos, vals=None, val_pos=None, lens=None, out=None, out_pos=None, out_lens=None):
+        """pskv_replay_record: serves the request once and returns a Replay whose run() repeats it with
+        one launch. The tensors are referenced by the Replay for as long as it lives."""
+        _memkind(MEM_DEVICE)
+        pos = np.ascontiguousarray(pos, dtype=np.uint64)
+        vp = None if val_pos is None else np.ascontiguousarray(val_pos, dtype=np.uint64)
+        op = None if out_pos is None else np.ascontiguousarray(out_pos, dtype=np.uint64)
+
+        def ptr(x):
+            return None if x is None or not x.numel() else x.data_ptr()
+
+        h = ctypes.c_void_p()
+        _check(self._lib.pskv_replay_record(ctypes.byref(h), self._arr, self.S, what, ptr(keys), pos.ctypes.data,
+                                            ptr(vals), None if vp is None else vp.ctypes.data, ptr(lens), ptr(out),
+                                            None if op is None else op.ctypes.data, ptr(out_lens)))
+        return Replay(h, (keys, vals, lens, out, out_lens))
+
     def size(self):
         nk = nv = 0
         for t in self.tables:
             a, b = t.size()
             nk, nv = nk + a, nv + b
         return nk, nv
+
+
+class Replay:
+    """A recorded request (pskv_replay_*). Close it before the tables it was recorded on."""
+
+    def __init__(self, handle, held):
+        self._h = handle
+        self._held = held
+        self._lib = load()
+
+    def run(self):
+        _check(self._lib.pskv_replay_run(self._h))
+
+    def close(self):
+        if self._h:
+            self._lib.pskv_replay_destroy(self._h)
+            self._h = None
+            self._held = None
+
+    def __del__(self):
+        if sys is None or sys.is_finalizing():
+            return
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 def server_ranges(num_servers):

@@ -51,6 +51,7 @@ constexpr unsigned kDevErrBadLen = 4u;      // negative or too long length
 constexpr unsigned kDevErrSizeMismatch = 8u;  // lens do not add up to the number of values
 constexpr unsigned kDevErrNoRoom = 16u;       // asynchronous var-len pull: response larger than the buffer
 constexpr unsigned kDevErrDuplicate = 32u;    // the same key twice in one request (row modes)
+constexpr unsigned kDevErrReplay = 64u;       // a replayed request no longer names the keys it was recorded with
 
 // Payload of a slot that has been claimed but not filled in yet (slots start as all ones).
 // No valid payload has bit 63 set.
@@ -147,7 +148,12 @@ struct Snapshot {
 struct ReqTag {
   unsigned long long epoch;  // number of the request
   unsigned int try_cache;    // the host found the key cache structurally usable for this request
-  unsigned int pad;
+  // The request is a replay of a recorded one (a node of a HIP graph, launched again and again with
+  // the same arguments, this number included): it is only ever served from the cache. When the
+  // comparison finds other keys than the cached ones, none of its kernels changes or answers
+  // anything and the table's error state says so (kDevErrReplay): the host has not sized anything
+  // for keys that it has not seen.
+  unsigned int replay;
 };
 
 // True when request `tag` carries exactly the keys (and lens) of the cached request, so that
@@ -156,6 +162,12 @@ struct ReqTag {
 // the request, so every workgroup of every later kernel sees the same answer.
 __device__ __forceinline__ bool cache_same(const DevState* st, const ReqTag& tag) {
   return st->same_epoch == tag.epoch;
+}
+
+// True in every kernel of a replayed request whose comparison has found other keys: the kernel
+// returns at once.
+__device__ __forceinline__ bool replay_blocked(const DevState* st, const ReqTag& tag) {
+  return tag.replay != 0u && st->same_epoch != tag.epoch;
 }
 
 // Records an error of request `epoch`; whatever that request left in the workspace is not

@@ -180,6 +180,12 @@ struct pskv_table {
   GrowBuf stage;      // device copies of host-resident request buffers
   GrowBuf stage_out;  // device-side response of a host-resident or undersized pull
   bool no_growth = false;  // set while dumping: every key is known to be present
+  // Recorded requests (pskv_replay_*): `gen` counts the requests that went the ordinary way, each
+  // of which may move a buffer, refill the key cache or write cached values back, so a recording
+  // only runs while `gen` is what it was when the recording was made. `capturing`: the table's
+  // stream is being captured into a HIP graph, nothing may be allocated, waited for or timed.
+  uint64_t gen = 0;
+  bool capturing = false;
 
   // Row modes: the workspace keeps the row references, offsets and tile table of the last
   // request that computed them, and the key cache keeps that request's keys and lens, so a
@@ -233,7 +239,7 @@ namespace {
 template <typename... KArgs, typename... Args>
 void launch_lds(pskv_table* t, int prof_kernel, void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds,
                 Args... args) {
-  if (t->prof && prof_kernel >= 0) {
+  if (t->prof && prof_kernel >= 0 && !t->capturing) {
     EventPair ev;
     bool have = false;
     if (!t->free_events.empty()) {
@@ -282,6 +288,7 @@ int prof_collect(pskv_table* t) {
 // ---- memory ----------------------------------------------------------------------
 int grow(pskv_table* t, GrowBuf* b, size_t bytes) {
   if (bytes <= b->bytes) return PSKV_OK;
+  if (t->capturing) return set_error(PSKV_ESTALE, "a recorded request needs a buffer that its first run did not leave");
   size_t want = std::max(bytes, b->bytes + b->bytes / 2);
   want = (want + 255) & ~(size_t)255;
   if (b == &t->ws || b == &t->tiles || b == &t->tiles_aff || b == &t->cache_keys ||
@@ -343,6 +350,9 @@ int report_device_errors(pskv_table* t) {
   PSKV_HIP(hipMemsetAsync(&t->st->error, 0, 2 * sizeof(unsigned), t->stream));
   PSKV_HIP(hipStreamSynchronize(t->stream));
   if (bits & kDevErrFull) return set_error(PSKV_ENOMEM, "slot array full (internal sizing error)");
+  if (bits & kDevErrReplay)
+    return set_error(PSKV_ESTALE, "a replayed request no longer named the keys it was recorded with: that run of it "
+                                  "changed and answered nothing on this table");
   if (bits & kDevErrBadLen)
     return set_error(PSKV_EINVAL, "a length is negative or above PSKV_MAX_VARLEN_ROW");
   if (bits & kDevErrSizeMismatch)
@@ -802,7 +812,12 @@ struct Request {
   // that it is still owed, gather_varlen which kernel it is).
   const float* vals_host;
   bool pipe_in, pipe_out, gather_deferred, gather_varlen;
+  // pskv_replay_record: kReplayPrime = the run that brings the tables into the state a repeat of the
+  // request finds (the key cache is filled whatever the size of the request and whatever earlier
+  // comparisons came to); kReplayCapture = the launches of such a repeat, recorded, not run.
+  int replay;
 };
+constexpr int kReplayPrime = 1, kReplayCapture = 2;
 
 // A request as the kernels see it: the shares of up to kMaxBatch tables that live on one device,
 // work in one mode and run on one stream, served by ONE launch per step of the pipeline. The
@@ -893,9 +908,9 @@ void note_outcomes(pskv_table* t) {
 ReqTag next_tag(pskv_table* t, const Request& r, bool back_off = false) {
   ReqTag tag;
   tag.epoch = ++t->epoch;
-  tag.pad = 0;
+  tag.replay = r.replay == kReplayCapture ? 1u : 0u;
   bool compare = t->cache_valid && t->cache_n == r.n;
-  if (back_off && compare) {
+  if (back_off && compare && !r.replay) {
     note_outcomes(t);
     const int kind = r.push ? 0 : 1;
     pskv_table::ScTrack& tr = t->sc_track[kind];
@@ -972,10 +987,23 @@ int run_scalar(Batch& bt, bool push, bool pull) {
     r.out_nvals = pull ? r.n : 0;
     it.d = TableReq{};
     if (r.n == 0) continue;
-    int rc = reserve(t, r.n, 0, 0, &it.pub);  // (a growth writes the cache back and drops it)
+    // (a growth writes the cache back and drops it; a recorded repeat creates no key)
+    int rc = r.replay == kReplayCapture ? PSKV_OK : reserve(t, r.n, 0, 0, &it.pub);
     if (rc) return rc;
     const int kind_before = t->sc_last_kind;
-    use[i] = scalar_cache_use(t, r);
+    if (r.replay) {
+      // a request that is being recorded fills the key cache, or is compared with it, whatever its size
+      if (t->cap >= (1ull << 32))
+        return set_error(PSKV_EINVAL, "a table of 2^32 slots keeps no key cache: its requests cannot be recorded");
+      const bool fits = t->cache_valid && t->cache_n == r.n;
+      if (r.replay == kReplayCapture && !fits)
+        return set_error(PSKV_ESTALE, "the key cache does not hold the request that is being recorded");
+      use[i] = fits ? kScTry : kScRecord;
+      t->sc_last_n = r.n;
+      t->sc_last_kind = r.push ? 0 : 1;
+    } else {
+      use[i] = scalar_cache_use(t, r);
+    }
     if (use[i] != kScTry) {
       // the request goes through the slots, so they must be up to date; a push then makes the
       // cached values stale, a recording replaces them
@@ -1006,10 +1034,12 @@ int run_scalar(Batch& bt, bool push, bool pull) {
       d.outcome = t->outcome;
       // A pull right behind a push, with the slots up to date (the push went through them and
       // recorded itself): the pull kernel compares key by key and needs no launch in front of it.
-      const bool per_key = use[i] == kScTry && !push && !t->sc_dirty && kind_before == 0;
+      // (not in a recording: keys that differ would go through the slots there)
+      const bool per_key = use[i] == kScTry && !push && !t->sc_dirty && kind_before == 0 && r.replay != kReplayCapture;
       d.cache_mode = per_key ? kCachePerKey : kCacheOn;
       any_cache = true;
-      it.flush_unless_same = !per_key && it.tag.try_cache && t->sc_dirty;
+      // (a recorded repeat is served from the cache or not at all: nothing to write back first)
+      it.flush_unless_same = !per_key && it.tag.try_cache && t->sc_dirty && r.replay != kReplayCapture;
     }
     d.slots = t->slots;
     d.mask = t->cap - 1;
@@ -1133,6 +1163,8 @@ int begin_row_request(Batch& bt) {
   for (Item& it : bt) {
     if (!it.r.n) continue;
     it.tag = next_tag(it.t, it.r, true);
+    if (it.r.replay == kReplayCapture && !it.tag.try_cache)
+      return set_error(PSKV_ESTALE, "the key cache does not hold the request that is being recorded");
     it.d.tag = it.tag;
     it.d.outcome = it.t->outcome;
   }
@@ -1151,7 +1183,7 @@ int run_fixed(Batch& bt, bool push, bool pull) {
     r.out_nvals = pull ? r.n * k : 0;
     it.d = TableReq{};
     if (r.n == 0) continue;
-    int rc = reserve(t, r.n, r.n, k, &it.pub);
+    int rc = r.replay == kReplayCapture ? PSKV_OK : reserve(t, r.n, r.n, k, &it.pub);
     if (rc) return rc;
     rc = grow(t, &t->ws, Carver::need(r.n, sizeof(uint64_t)));
     if (rc) return rc;
@@ -1175,7 +1207,9 @@ int run_fixed(Batch& bt, bool push, bool pull) {
   if (!n_largest) return PSKV_OK;
   int rc = begin_row_request(bt);
   if (rc) return rc;
-  if (n_largest >= kLookupLargeKeys) {
+  if (bt[0].r.replay == kReplayCapture) {
+    // a recorded repeat uses the references that are there: no lookup
+  } else if (n_largest >= kLookupLargeKeys) {
     rc = launch_batch(bt, PSKV_KERNEL_LOOKUP, k_lookup_fixed<kLookupItemsLarge>, [](const Item& it) {
       return it.r.n ? (uint64_t)grid_for(it.r.n, kBlock * kLookupItemsLarge, kMaxGrid) : 0ull;
     });
@@ -1246,6 +1280,7 @@ int make_tile_tables(Batch& bt, int items) {
     it.d.tile_aff = static_cast<TileNote*>(it.t->tiles_aff.ptr);
     it.d.ntiles = ntiles_cap;
   }
+  if (bt[0].r.replay == kReplayCapture) return PSKV_OK;  // (a recorded repeat: the tables that are there)
   return launch_batch(bt, -1, items == kScanItemsLarge ? k_var_offsets<kScanItemsLarge> : k_var_offsets<1>,
                       [](const Item& it) { return (it.r.n && it.d.total) ? it.nparts : 0ull; });
 }
@@ -1304,10 +1339,14 @@ int run_varlen(Batch& bt, bool push, bool pull) {
       Request& r = it.r;
       if (!r.n) continue;
       // every key may round its row up to a 16-byte unit, every workgroup may pad its rows' start
-      int rc = reserve(t, r.n, r.nvals / 4 + r.n + kArenaPadUnits * it.nparts, 4, &it.pub);
+      int rc = r.replay == kReplayCapture
+                   ? PSKV_OK
+                   : reserve(t, r.n, r.nvals / 4 + r.n + kArenaPadUnits * it.nparts, 4, &it.pub);
       if (rc) return rc;
       if (t->cache_nvals != r.nvals) t->cache_valid = false;  // same lens would mean the same total
       it.tag = next_tag(t, r, true);
+      if (r.replay == kReplayCapture && !it.tag.try_cache)
+        return set_error(PSKV_ESTALE, "the key cache does not hold the request that is being recorded");
       TableReq& d = it.d;
       d.outcome = t->outcome;
       d.slots = t->slots;
@@ -1326,7 +1365,9 @@ int run_varlen(Batch& bt, bool push, bool pull) {
     }
     int rc = launch_keys(bt, -1, items, k_var_push_begin<1>, k_var_push_begin<kScanItemsLarge>);
     if (rc) return rc;
-    rc = launch_keys(bt, PSKV_KERNEL_LOOKUP, items, k_var_push_lookup<1>, k_var_push_lookup<kScanItemsLarge>);
+    // (a recorded repeat uses the offsets, tile table and references that are there)
+    if (bt[0].r.replay != kReplayCapture)
+      rc = launch_keys(bt, PSKV_KERNEL_LOOKUP, items, k_var_push_lookup<1>, k_var_push_lookup<kScanItemsLarge>);
     if (rc) return rc;
     for (Item& it : bt) {
       if (!it.r.n) continue;
@@ -1432,13 +1473,16 @@ int run_varlen(Batch& bt, bool push, bool pull) {
 
 int run_batch(Batch& bt, bool push, bool pull) {
   int rc;
+  const bool capturing = bt[0].t->capturing;
+  if (!capturing)
+    for (Item& it : bt) ++it.t->gen;
   switch (bt[0].t->mode) {
     case PSKV_MODE_SCALAR: rc = run_scalar(bt, push, pull); break;
     case PSKV_MODE_FIXED: rc = run_fixed(bt, push, pull); break;
     default: rc = run_varlen(bt, push, pull); break;
   }
   // the GPU is busy with the request now: the moment to allocate ahead of a coming growth
-  if (!rc)
+  if (!rc && !capturing)
     for (Item& it : bt) prepare_growth(it.t);
   return rc;
 }
@@ -1714,12 +1758,11 @@ int check_group(pskv_table* const* tables, size_t S) {
 
 // pskv_push_multi / pskv_pull_multi: slice s of the request, keys [pos[s], pos[s+1]), goes to
 // tables[s]; slices without keys are skipped as KVWorker::Send skips them (kv_app.h:590-595).
-int request_multi(pskv_table* const* tables, size_t S, bool push, const uint64_t* keys,
+int request_multi(pskv_table* const* tables, size_t S, bool push, bool pull, const uint64_t* keys,
                   const uint64_t* pos, const float* vals, const uint64_t* val_pos, const int32_t* lens,
                   float* out, const uint64_t* out_pos, int32_t* out_lens, uint64_t* out_nvals,
-                  int memkind) {
+                  int memkind, int replay = 0) {
   clear_error();
-  const bool pull = !push;
   if (memkind != PSKV_MEM_DEVICE)
     return set_error(PSKV_EINVAL, "the multi-table entry points take device-resident buffers "
                                   "(PSKV_MEM_DEVICE); host-resident requests go table by table");
@@ -1742,6 +1785,7 @@ int request_multi(pskv_table* const* tables, size_t S, bool push, const uint64_t
     r = Request{};
     r.push = push;
     r.pull = pull;
+    r.replay = replay;
     r.n = pos[s + 1] - pos[s];
     r.keys = keys + pos[s];
     if (push) {
@@ -1971,15 +2015,121 @@ void* pskv_table_stream(pskv_table* t) { return t ? static_cast<void*>(t->stream
 
 int pskv_push_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, const uint64_t* pos,
                     const float* vals, const uint64_t* val_pos, const int32_t* lens, int memkind) {
-  return request_multi(tables, S, true, keys, pos, vals, val_pos, lens, nullptr, nullptr, nullptr,
+  return request_multi(tables, S, true, false, keys, pos, vals, val_pos, lens, nullptr, nullptr, nullptr,
                        nullptr, memkind);
 }
 
 int pskv_pull_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, const uint64_t* pos,
                     float* out, const uint64_t* out_pos, int32_t* out_lens, uint64_t* out_nvals,
                     int memkind) {
-  return request_multi(tables, S, false, keys, pos, nullptr, nullptr, nullptr, out, out_pos, out_lens,
+  return request_multi(tables, S, false, true, keys, pos, nullptr, nullptr, nullptr, out, out_pos, out_lens,
                        out_nvals, memkind);
+}
+
+struct pskv_replay {
+  std::vector<pskv_table*> tables;
+  std::vector<uint64_t> gen;  // pskv_table::gen of each when the recording was made
+  hipGraphExec_t exec = nullptr;
+  hipStream_t stream = nullptr;
+  int device = 0;
+};
+
+int pskv_replay_record(pskv_replay** out, pskv_table* const* tables, size_t S, int what, const uint64_t* keys,
+                       const uint64_t* pos, const float* vals, const uint64_t* val_pos, const int32_t* lens,
+                       float* out_vals, const uint64_t* out_pos, int32_t* out_lens) {
+  clear_error();
+  if (!out) return set_error(PSKV_EINVAL, "null argument");
+  *out = nullptr;
+  const bool push = (what & PSKV_REPLAY_PUSH) != 0, pull = (what & PSKV_REPLAY_PULL) != 0;
+  if ((!push && !pull) || (what & ~(PSKV_REPLAY_PUSH | PSKV_REPLAY_PULL)))
+    return set_error(PSKV_EINVAL, "what = %d names neither a push nor a pull", what);
+  if (S == 0) return set_error(PSKV_EINVAL, "no tables");
+  int rc = check_group(tables, S);
+  if (rc) return rc;
+  if (!pos || pos[S] == pos[0]) return set_error(PSKV_EINVAL, "a request without keys cannot be recorded");
+  auto both = [&](int replay) -> int {
+    // SCALAR: a pull of the keys just pushed is the push's own read-back, so the two go as ONE request
+    // with both halves (per key the push first, kv_app.h:451-459): one comparison and one pass
+    if (push && pull && tables[0]->mode == PSKV_MODE_SCALAR)
+      return request_multi(tables, S, true, true, keys, pos, vals, val_pos, lens, out_vals, out_pos, out_lens,
+                           nullptr, PSKV_MEM_DEVICE, replay);
+    int r = PSKV_OK;
+    if (push)
+      r = request_multi(tables, S, true, false, keys, pos, vals, val_pos, lens, nullptr, nullptr, nullptr,
+                        nullptr, PSKV_MEM_DEVICE, replay);
+    if (!r && pull)
+      r = request_multi(tables, S, false, true, keys, pos, nullptr, nullptr, nullptr, out_vals, out_pos, out_lens,
+                        nullptr, PSKV_MEM_DEVICE, replay);
+    return r;
+  };
+  // The request itself, the ordinary way: tables grow, buffers get their sizes, the key cache is
+  // filled. What the device finds wrong with it ends the recording.
+  rc = both(kReplayPrime);
+  if (rc) return rc;
+  rc = pskv_sync_multi(tables, S);
+  if (rc) return rc;
+  DeviceGuard guard(tables[0]->device);
+  if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", tables[0]->device);
+  // (an allocation that the library's own thread is making on this stream must not land in the graph)
+  for (size_t s = 0; s < S; ++s) collect_spare(tables[s], true);
+  hipStream_t stream = tables[0]->stream;
+  // The launches of a repeat, recorded instead of run. Relaxed: other threads of the process may
+  // be allocating or waiting meanwhile, which is none of this capture's business.
+  PSKV_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed));
+  for (size_t s = 0; s < S; ++s) tables[s]->capturing = true;
+  rc = both(kReplayCapture);
+  for (size_t s = 0; s < S; ++s) tables[s]->capturing = false;
+  hipGraph_t graph = nullptr;
+  const hipError_t e = hipStreamEndCapture(stream, &graph);
+  if (rc || e != hipSuccess || !graph) {
+    const std::string text = rc ? std::string(pskv_last_error()) : std::string();
+    if (graph) (void)hipGraphDestroy(graph);
+    (void)hipGetLastError();
+    for (size_t s = 0; s < S; ++s) tables[s]->cache_valid = false;
+    if (rc) return set_error(rc, "%s", text.c_str());
+    return set_error(PSKV_EHIP, "the stream of the tables could not be captured: %s", hipGetErrorString(e));
+  }
+  pskv_replay* r = new (std::nothrow) pskv_replay();
+  if (!r) {
+    (void)hipGraphDestroy(graph);
+    return set_error(PSKV_ENOMEM, "out of host memory");
+  }
+  const hipError_t ei = hipGraphInstantiate(&r->exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (ei != hipSuccess) {
+    delete r;
+    (void)hipGetLastError();
+    return set_error(PSKV_EHIP, "hipGraphInstantiate: %s", hipGetErrorString(ei));
+  }
+  r->stream = stream;
+  r->device = tables[0]->device;
+  r->tables.assign(tables, tables + S);
+  for (size_t s = 0; s < S; ++s) r->gen.push_back(tables[s]->gen);
+  *out = r;
+  return PSKV_OK;
+}
+
+int pskv_replay_run(pskv_replay* r) {
+  clear_error();
+  if (!r || !r->exec) return set_error(PSKV_EINVAL, "null recording");
+  for (size_t s = 0; s < r->tables.size(); ++s)
+    if (r->tables[s]->gen != r->gen[s])
+      return set_error(PSKV_ESTALE, "tables[%zu] has served other requests since the recording was made", s);
+  DeviceGuard guard(r->device);
+  if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", r->device);
+  PSKV_HIP(hipGraphLaunch(r->exec, r->stream));
+  return PSKV_OK;
+}
+
+int pskv_replay_destroy(pskv_replay* r) {
+  if (!r) return PSKV_OK;
+  DeviceGuard guard(r->device);
+  if (r->exec) {
+    (void)hipStreamSynchronize(r->stream);
+    (void)hipGraphExecDestroy(r->exec);
+  }
+  delete r;
+  return PSKV_OK;
 }
 
 int pskv_sync_multi(pskv_table* const* tables, size_t S) {

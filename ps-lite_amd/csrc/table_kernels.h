@@ -106,6 +106,7 @@ __global__ __launch_bounds__(kBlock) void k_scalar(ReqBatch b) {
   const float* __restrict__ vals = d.vals;
   float* __restrict__ out = d.out;
   const bool record = CACHE && d.cache_mode == kCacheOn;
+  if (CACHE && replay_blocked(st, d.tag)) return;
   if (record && cache_same(st, d.tag)) {
     // the keys are those of the cached request: position i of the request is position i of the cache
     float* __restrict__ cv = d.arena;
@@ -267,7 +268,7 @@ __global__ __launch_bounds__(kBlock) void k_scalar_flush(ReqBatch b) {
   // after every workgroup has read them
   const unsigned long long dirty = d.st->dirty_epoch;
   if (dirty <= d.st->clean_epoch) return;  // the slots are up to date
-  if (d.cache_mode == kFlushUnlessSame && cache_same(d.st, d.tag)) return;
+  if (d.cache_mode == kFlushUnlessSame && (cache_same(d.st, d.tag) || d.tag.replay)) return;
   __shared__ unsigned s_last;
   const uint64_t stride = (uint64_t)d.nblk * kBlock;
   for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < d.n; i += stride) {
@@ -296,6 +297,12 @@ __device__ __forceinline__ void decide_same(DevState* st, const ReqTag& tag, boo
   const bool usable =
       tag.try_cache && st->cache_epoch != 0ull && st->bad_epoch != st->cache_epoch;
   const bool same = !different && usable;
+  if (tag.replay && !same) {
+    // (an earlier replay of this very request may have left its number here)
+    st->same_epoch = 0ull;
+    atomicOr(&st->error, kDevErrReplay);
+    return;
+  }
   if (same) {
     st->same_epoch = tag.epoch;
   } else {
@@ -406,6 +413,7 @@ __global__ __launch_bounds__(kBlock) void k_lookup_fixed(ReqBatch b) {
     if (snap && blockIdx.x == 0 && threadIdx.x < 64) publish_snapshot(st, snap, snap_seq);
     return;
   }
+  if (tag.replay) return;
   if (blockIdx.x == 0 && threadIdx.x == 0) st->cache_epoch = cache_keys ? tag.epoch : 0ull;
   __shared__ unsigned long long red[kBlock / 64];
   __shared__ unsigned cred[kBlock / 64];
@@ -564,6 +572,7 @@ __global__ __launch_bounds__(kBlock) void k_var_push_lookup(ReqBatch b) {
     if (snap && blockIdx.x == 0 && threadIdx.x < 64) publish_snapshot(st, snap, snap_seq);
     return;
   }
+  if (tag.replay) return;
   // the request is refused as a whole when its lens are invalid or do not add up to vals.size(),
   // or when it repeats a key
   // (a refused request creates nothing, so the counter record the host may be waiting for holds
@@ -681,6 +690,7 @@ __global__ __launch_bounds__(kBlock) void k_var_pull_lookup(ReqBatch b) {
       if (base + j < n) out_lens[base + j] = cache_lens[base + j];
     return;
   }
+  if (tag.replay) return;
   // this pull rewrites the references and offsets in the workspace: the cached push is gone
   if (blockIdx.x == 0 && threadIdx.x == 0) st->bad_epoch = st->cache_epoch;
   unsigned long long s = 0;
@@ -718,7 +728,7 @@ __global__ __launch_bounds__(kBlock) void k_var_offsets(ReqBatch b) {
   constexpr uint64_t tile = PSKV_TILE_VAR;
   const DevState* st = d.st;
   const ReqTag tag = d.tag;
-  if (cache_same(st, tag)) return;  // offsets and tile table of the cached request hold
+  if (cache_same(st, tag) || tag.replay) return;  // offsets and tile table of the cached request hold
   __shared__ unsigned long long wsum[kBlock / 64];
   uint64_t ntiles = (st->scan_total + tile - 1) / tile;
   if (ntiles > ntiles_cap) ntiles = ntiles_cap;
@@ -1153,6 +1163,7 @@ __global__ __launch_bounds__(kBlock) void k_rows(ReqBatch b) {
     if (!scalar) rows_wave_ask<OP, 4, STREAM, kTileVar>(p, p.total, x4, aff);
     // a request served from the cached references creates nothing and cannot have been refused
     const bool same = facts.same_epoch == p.tag.epoch;
+    if (p.tag.replay && !same) return;
     if (same) p.ignore_new = 1;
     const unsigned err = same ? 0u : facts.req_error;
     if (err & (kDevErrBadLen | kDevErrSizeMismatch | kDevErrDuplicate)) return;
@@ -1175,6 +1186,7 @@ __global__ __launch_bounds__(kBlock) void k_rows(ReqBatch b) {
       rows_wave_varlen<OP, 4, STREAM, kTileVar>(p, total, s_off, s_ref, rejected, same, x4);
     }
   } else {
+    if (p.tag.replay && facts.same_epoch != p.tag.epoch) return;
     if (facts.same_epoch == p.tag.epoch) p.ignore_new = 1;
     if (scalar) {
       rows_tile_fixed<OP, 1, STREAM, kTileFixed>(p, total);
