@@ -1239,6 +1239,22 @@ def extra_replay_small(capi, dev, n=100000, S=4, steps=200):
     for _ in range(5 + steps):
         ref = ref + dv
     assert torch.equal(out, ref), "sums differ from sequential float adds"
+
+    def step_one():
+        pos, _, _ = capi.slice_keys(dk, rb, re, nvals=n)
+        group.pushpull_raw(kp, pos, vp, pos, op)
+
+    for _ in range(5):
+        step_one()
+    group.sync()
+    t1 = time.perf_counter()
+    for _ in range(steps):
+        step_one()
+    group.sync()
+    dt_one = time.perf_counter() - t1
+    for _ in range(5 + steps):
+        ref = ref + dv
+    assert torch.equal(out, ref), "push+pull sums differ from sequential float adds"
     pos, _, _ = capi.slice_keys(dk, rb, re, nvals=n)
     rec = group.record(capi.REPLAY_PUSH | capi.REPLAY_PULL, dk, pos, dv, pos, None, out)
     replayed, ref = timed_replays(rec, group, steps, ref, dv)
@@ -1247,6 +1263,8 @@ def extra_replay_small(capi, dev, n=100000, S=4, steps=200):
     group.close()
     return {"workload": "the same %d keys over %d key ranges pushed and pulled every step (SCALAR)" % (n, S),
             "steps": steps, "ms_per_step": dt / steps * 1e3, "value": 2.0 * n * steps / dt, "unit": "keys/s",
+            "one_request": {"ms_per_step": dt_one / steps * 1e3, "value": 2.0 * n * steps / dt_one, "unit": "keys/s",
+                            "note": "slice + ONE pskv_pushpull_multi request per step, not recorded"},
             "replayed": dict(replayed, value=2.0 * n / (replayed["ms_per_step"] * 1e-3), unit="keys/s")}
 
 

@@ -125,7 +125,7 @@ int pskv_pushpull(pskv_table* t, const uint64_t* keys, size_t n, const float* va
 
 /* One process, several logical servers on one GPU. KVWorker::Send turns a sliced request into
  * one message per server range (kv_app.h:590-612); when the tables of those ranges live in one
- * process on one GPU, the three calls below serve all of them with ONE launch per step of the
+ * process on one GPU, the calls below serve all of them with ONE launch per step of the
  * pipeline instead of one per table (a launch over 1/S of a request leaves most of the GPU
  * idle). pos[S+1] and val_pos[S+1] are HOST arrays, exactly what pskv_slice returns: slice s
  * holds keys [pos[s], pos[s+1]) and vals [val_pos[s], val_pos[s+1]) (and lens [pos[s],
@@ -152,6 +152,12 @@ int pskv_push_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, c
 int pskv_pull_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, const uint64_t* pos,
                     float* out, const uint64_t* out_pos, int32_t* out_lens, uint64_t* out_nvals,
                     int memkind);
+/* A request with push and pull both set (kv_app.h:451-459) over all slices at once: what S calls of
+ * pskv_pushpull would give, arguments as in the two calls above. In PSKV_MODE_VARLEN the call waits for
+ * the device between the two halves, as pskv_pushpull does (a refused push is not followed by its pull). */
+int pskv_pushpull_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, const uint64_t* pos,
+                        const float* vals, const uint64_t* val_pos, const int32_t* lens, float* out,
+                        const uint64_t* out_pos, int32_t* out_lens, uint64_t* out_nvals, int memkind);
 /* pskv_sync for all tables of a group with one wait: returns the first deferred error (every
  * table's error state is cleared). */
 int pskv_sync_multi(pskv_table* const* tables, size_t S);

@@ -7,6 +7,7 @@ memory here; every computation happens inside libpskv.so.
 import ctypes
 import os
 import sys
+import weakref
 
 import numpy as np
 
@@ -42,7 +43,7 @@ ERROR_NAMES = {
 # every symbol include/pskv/capi.h declares
 SYMBOLS = [
     "pskv_table_create", "pskv_table_destroy", "pskv_push", "pskv_pull", "pskv_pushpull",
-    "pskv_sync", "pskv_table_stream", "pskv_push_multi", "pskv_pull_multi", "pskv_sync_multi", "pskv_replay_record", "pskv_replay_run", "pskv_replay_destroy", "pskv_size", "pskv_dump", "pskv_slice", "pskv_slice_noalloc", "pskv_server_ranges",
+    "pskv_sync", "pskv_table_stream", "pskv_push_multi", "pskv_pull_multi", "pskv_pushpull_multi", "pskv_sync_multi", "pskv_replay_record", "pskv_replay_run", "pskv_replay_destroy", "pskv_size", "pskv_dump", "pskv_slice", "pskv_slice_noalloc", "pskv_server_ranges",
     "pskv_assemble_pull", "pskv_match", "pskv_prof_enable", "pskv_prof_reset", "pskv_prof_read", "pskv_prof_samples",
     "pskv_copy_probe", "pskv_host_alloc", "pskv_host_free", "pskv_host_trim", "pskv_device_trim", "pskv_table_counters", "pskv_last_error",
     "pskv_version",
@@ -92,6 +93,7 @@ def load():
     lib.pskv_table_stream.restype = vp
     lib.pskv_push_multi.argtypes = [vp, sz, vp, vp, vp, vp, vp, i32]
     lib.pskv_pull_multi.argtypes = [vp, sz, vp, vp, vp, vp, vp, vp, i32]
+    lib.pskv_pushpull_multi.argtypes = [vp, sz, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32]
     lib.pskv_sync_multi.argtypes = [vp, sz]
     lib.pskv_replay_record.argtypes = [ctypes.POINTER(vp), vp, sz, i32, vp, vp, vp, vp, vp, vp, vp, vp]
     lib.pskv_replay_run.argtypes = [vp]
@@ -322,6 +324,12 @@ class Group(_Holder):
         self._lib = load()
 
     def close(self):
+        # recordings go before the tables they point at
+        for ref in self.__dict__.get("_recordings", []):
+            rec = ref()
+            if rec is not None:
+                rec.close()
+        self.__dict__["_recordings"] = []
         # the first table owns the stream the others run on: it goes last
         for t in reversed(self.tables):
             t.close()
@@ -356,6 +364,32 @@ class Group(_Holder):
                                        out_lens_ptr, sizes.ctypes.data if want_sizes else None, MEM_DEVICE)
         self.last_sizes = sizes
         _check(rc)
+        return sizes[:self.S] if want_sizes else None
+
+    def pushpull_raw(self, keys_ptr, pos, vals_ptr, val_pos, out_ptr, out_pos=None, lens_ptr=None, out_lens_ptr=None):
+        pos = np.ascontiguousarray(pos, dtype=np.uint64)
+        val_pos = np.ascontiguousarray(val_pos, dtype=np.uint64)
+        op = None if out_pos is None else np.ascontiguousarray(out_pos, dtype=np.uint64)
+        _check(self._lib.pskv_pushpull_multi(self._arr, self.S, keys_ptr, pos.ctypes.data, vals_ptr,
+                                             val_pos.ctypes.data, lens_ptr, out_ptr,
+                                             None if op is None else op.ctypes.data, out_lens_ptr, None, MEM_DEVICE))
+
+    def pushpull(self, keys, pos, vals, val_pos, out, lens=None, out_pos=None, out_lens=None, want_sizes=False):
+        """pskv_pushpull_multi: one request with both halves over all slices."""
+        _memkind(MEM_DEVICE)
+        self._hold(keys, vals, lens, out, out_lens)
+        pos = np.ascontiguousarray(pos, dtype=np.uint64)
+        val_pos = np.ascontiguousarray(val_pos, dtype=np.uint64)
+        op = None if out_pos is None else np.ascontiguousarray(out_pos, dtype=np.uint64)
+        sizes = np.zeros(max(self.S, 1), np.uint64) if want_sizes else None
+
+        def ptr(x):
+            return None if x is None or not x.numel() else x.data_ptr()
+
+        _check(self._lib.pskv_pushpull_multi(self._arr, self.S, ptr(keys), pos.ctypes.data, ptr(vals),
+                                             val_pos.ctypes.data, ptr(lens), ptr(out),
+                                             None if op is None else op.ctypes.data, ptr(out_lens),
+                                             sizes.ctypes.data if want_sizes else None, MEM_DEVICE))
         return sizes[:self.S] if want_sizes else None
 
     def push(self, keys, pos, vals, val_pos, lens=None):
@@ -393,7 +427,9 @@ class Group(_Holder):
         _check(self._lib.pskv_replay_record(ctypes.byref(h), self._arr, self.S, what, ptr(keys), pos.ctypes.data,
                                             ptr(vals), None if vp is None else vp.ctypes.data, ptr(lens), ptr(out),
                                             None if op is None else op.ctypes.data, ptr(out_lens)))
-        return Replay(h, (keys, vals, lens, out, out_lens))
+        rec = Replay(h, (keys, vals, lens, out, out_lens))
+        self.__dict__.setdefault("_recordings", []).append(weakref.ref(rec))
+        return rec
 
     def size(self):
         nk = nv = 0

@@ -2019,6 +2019,13 @@ int pskv_push_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, c
                        nullptr, memkind);
 }
 
+int pskv_pushpull_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, const uint64_t* pos,
+                        const float* vals, const uint64_t* val_pos, const int32_t* lens, float* out,
+                        const uint64_t* out_pos, int32_t* out_lens, uint64_t* out_nvals, int memkind) {
+  return request_multi(tables, S, true, true, keys, pos, vals, val_pos, lens, out, out_pos, out_lens, out_nvals,
+                       memkind);
+}
+
 int pskv_pull_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, const uint64_t* pos,
                     float* out, const uint64_t* out_pos, int32_t* out_lens, uint64_t* out_nvals,
                     int memkind) {

@@ -108,6 +108,45 @@ def test_multi_matches_the_oracle(capi, orc, dev, mode, S, n):
     g.close()
 
 
+@pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
+@pytest.mark.parametrize("S,n", [(4, 10000), (19, 30000), (3, 300000)])
+def test_pushpull_multi_matches_the_oracle(capi, orc, dev, mode, S, n):
+    """One request with both halves over all slices (KVWorker::PushPull through kv_app.h:451-459):
+    per key the push first, then the value read back; keys the store has never seen among them; the
+    third request repeats the second's keys."""
+    import torch
+    announce("pushpull_multi", mode, S, n)
+    rng = np.random.default_rng(S + n)
+    rb, re = capi.server_ranges(S)
+    k = 12
+    g = capi.Group(S, MODES[mode], initial_capacity=16, row_len=k if mode == "fixed" else 0)
+    o = orc.Store(MODES[mode], k if mode == "fixed" else 0)
+    universe = unique_keys(rng, 2 * n, S)
+    len_of = dict(zip(universe.tolist(), rng.choice(np.array([0, 4, 8, 20, 64], np.int32), size=universe.size).tolist()))
+    keys = None
+    for rep in range(4):
+        if rep != 2:
+            keys = np.sort(rng.choice(universe, size=n, replace=False))
+        lens = np.array([len_of[x] for x in keys.tolist()], np.int32) if mode == "varlen" else None
+        nvals = {"scalar": n, "fixed": k * n}.get(mode, int(lens.sum()) if lens is not None else 0)
+        vals = rng.normal(0, 1, size=nvals).astype(np.float32)
+        dk, dv = to_dev(keys, dev), to_dev(vals, dev)
+        dl = None if lens is None else to_dev(lens, dev)
+        pos, vpos = _slice(capi, dk, rb, re, dl, nvals)
+        out = torch.full((nvals + 4,), 7.0, dtype=torch.float32, device=dev)
+        out_lens = torch.full((n,), -1, dtype=torch.int32, device=dev) if mode == "varlen" else None
+        sizes = g.pushpull(dk, pos, dv, vpos, out, dl, vpos, out_lens, want_sizes=True)
+        rc, want, want_lens, _ = o.handle(True, True, keys, vals, lens)
+        assert rc == 0
+        g.sync()
+        assert np.array_equal(sizes.astype(np.int64), np.diff(vpos.astype(np.int64)))
+        assert_bits_equal(from_dev(out)[:nvals], want, "push+pull %d" % rep)
+        if mode == "varlen":
+            assert np.array_equal(from_dev(out_lens), want_lens)
+    _check_dump(g, o, "after the push+pulls")
+    g.close()
+
+
 def test_multi_equals_single_table_calls(capi, dev):
     """The same requests through pskv_push_multi and through one pskv_push per table leave
     identical stores, key for key and bit for bit (var-len rows of mixed lengths)."""
