@@ -80,6 +80,7 @@ struct AllocJob {
   void* ptr = nullptr;
   bool pooled = false;
   int rc = PSKV_OK;
+  double took_us = 0;  // what the allocation cost the allocating thread
   bool done = false;  // guarded by AllocWorker::mu
 };
 
@@ -141,6 +142,7 @@ struct pskv_table {
   struct Stats {
     uint64_t requests = 0, waits = 0, growths = 0, growths_unasked = 0, spare_used = 0, records = 0, catch_ups = 0;
     double alloc_us = 0, release_us = 0, catch_up_us = 0;  // host time spent allocating, releasing, catching up
+    double ahead_us = 0;  // time the allocating thread spent on this table's arrays
   } stats;
   uint64_t count = 0;      // key count at the last read_state()
 
@@ -289,8 +291,11 @@ int prof_collect(pskv_table* t) {
 int grow(pskv_table* t, GrowBuf* b, size_t bytes) {
   if (bytes <= b->bytes) return PSKV_OK;
   if (t->capturing) return set_error(PSKV_ESTALE, "a recorded request needs a buffer that its first run did not leave");
-  size_t want = std::max(bytes, b->bytes + b->bytes / 2);
-  want = (want + 255) & ~(size_t)255;
+  // An eighth to spare (up to 32 MB): the slices of a worker's requests differ by a few keys from one
+  // request to the next, and a reallocation waits for the stream and costs 100-350 us, several
+  // requests' worth, every time a table sees its largest slice so far.
+  size_t want = std::max(bytes + std::min<size_t>(bytes / 8, (size_t)32 << 20), b->bytes + b->bytes / 2);
+  want = (want + 4095) & ~(size_t)4095;
   if (b == &t->ws || b == &t->tiles || b == &t->tiles_aff || b == &t->cache_keys ||
       b == &t->cache_lens || b == &t->sc_vals || b == &t->sc_slots)
     t->cache_valid = false;  // the contents do not survive a reallocation
@@ -471,12 +476,14 @@ class AllocWorker {
         job = jobs_.front();
         jobs_.pop_front();
       }
+      const auto a0 = std::chrono::steady_clock::now();
       if (hipSetDevice(job->device) != hipSuccess) {
         (void)hipGetLastError();
         job->rc = PSKV_EHIP;
       } else {
         job->rc = alloc_for_growth(&job->ptr, job->bytes, job->stream, &job->pooled);
       }
+      job->took_us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - a0).count();
       {
         std::lock_guard<std::mutex> lk(mu_);
         job->done = true;
@@ -568,6 +575,7 @@ void collect_spare(pskv_table* t, bool wait) {
   } else if (!AllocWorker::get().finished(t->spare_job)) {
     return;
   }
+  t->stats.ahead_us += t->spare_job->took_us;
   if (t->spare_job->rc == PSKV_OK && t->spare_job->ptr) {
     t->spare = static_cast<Slot*>(t->spare_job->ptr);
     t->spare_pooled = t->spare_job->pooled;
@@ -1935,12 +1943,12 @@ int pskv_table_destroy(pskv_table* t) {
   if (std::getenv("PSKV_STATS"))
     fprintf(stderr, "[pskv] table %p mode %d: %llu requests, %llu slots at the end, %llu growths (%llu without asking "
             "the device, %llu into an array allocated ahead), %llu waits for exact counters, %llu for the newest record (%.0f us), %llu counter records; host time "
-            "allocating %.0f us, releasing %.0f us\n",
+            "allocating %.0f us (%.0f us on the allocating thread), releasing %.0f us\n",
             (void*)t, t->mode, (unsigned long long)t->stats.requests, (unsigned long long)t->cap,
             (unsigned long long)t->stats.growths, (unsigned long long)t->stats.growths_unasked,
             (unsigned long long)t->stats.spare_used, (unsigned long long)t->stats.waits,
             (unsigned long long)t->stats.catch_ups, t->stats.catch_up_us, (unsigned long long)t->stats.records,
-            t->stats.alloc_us, t->stats.release_us);
+            t->stats.alloc_us, t->stats.ahead_us, t->stats.release_us);
   if (t->stream) (void)hipStreamSynchronize(t->stream);
   for (int k = 0; k < PSKV_KERNEL_COUNT; ++k)
     for (const EventPair& ev : t->pending[k]) t->free_events.push_back(ev);
