@@ -23,6 +23,8 @@ def test_kv_app_through_adapters(num_servers):
     assert "test_kv_app_gpu: ok" in r.stdout
     # the two workers of tests/test_kv_app_multi_workers.cc ran, each on its own thread
     assert "two workers, customer 0: error 0, 0" in r.stdout and "two workers, customer 1: error 0, 0" in r.stdout
+    # the reference test's 50 pushes of one key set, recorded once and replayed through the C ABI alone
+    assert "ranges replayed, 0 + 0 floats differ" in r.stdout
 
 
 def test_kv_app_with_32_bit_keys():

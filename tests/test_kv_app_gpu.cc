@@ -223,6 +223,87 @@ static void RunDeviceBufferContract() {
   std::printf("device buffers: %d pushes of %zu keys from one buffer, %zu floats differ\n", pushes, n, bad);
 }
 
+// The reference's test pushes one key set `repeat` times and pulls it once (tests/test_kv_app.cc:36-60).
+// Here with the servers' tables and the worker's buffers on one GPU: the request is recorded once
+// (pskv_replay_record) and every repeat is one pskv_replay_run; closed forms as in the reference's check.
+static void RunRecordedRequests(int num_servers) {
+  const size_t S = static_cast<size_t>(num_servers), n = 200000;
+  const int repeat = 50;
+  std::vector<uint64_t> rb(S), re(S), pos(S + 1), val_pos(S + 1);
+  std::vector<uint8_t> used(S);
+  EXPECT(pskv_server_ranges(S, rb.data(), re.data()) == PSKV_OK);
+  std::vector<pskv_table*> t(S, nullptr);
+  pskv_opts o = {};
+  o.mode = PSKV_MODE_SCALAR;
+  for (size_t s = 0; s < S; ++s) {
+    EXPECT(pskv_table_create(&t[s], &o) == PSKV_OK);
+    o.stream = pskv_table_stream(t[0]);
+  }
+  std::vector<uint64_t> keys(n);
+  std::vector<float> vals(n), got(n, -1.0f);
+  for (size_t i = 0; i < n; ++i) {
+    keys[i] = (re[S - 1] / n) * i;  // tests/test_kv_app.cc:27
+    vals[i] = static_cast<float>(i % 1000) * 0.5f;
+  }
+  uint64_t* d_keys = nullptr;
+  float *d_vals = nullptr, *d_out = nullptr;
+  EXPECT(hipMalloc(reinterpret_cast<void**>(&d_keys), n * 8) == hipSuccess);
+  EXPECT(hipMalloc(reinterpret_cast<void**>(&d_vals), n * 4) == hipSuccess);
+  EXPECT(hipMalloc(reinterpret_cast<void**>(&d_out), n * 4) == hipSuccess);
+  EXPECT(hipMemcpy(d_keys, keys.data(), n * 8, hipMemcpyHostToDevice) == hipSuccess);
+  EXPECT(hipMemcpy(d_vals, vals.data(), n * 4, hipMemcpyHostToDevice) == hipSuccess);
+  EXPECT(pskv_slice(0, d_keys, n, nullptr, 0, n, rb.data(), re.data(), S, pos.data(), val_pos.data(), used.data(),
+                    PSKV_MEM_DEVICE) == PSKV_OK);
+  pskv_replay* push = nullptr;
+  EXPECT(pskv_replay_record(&push, t.data(), S, PSKV_REPLAY_PUSH, d_keys, pos.data(), d_vals, val_pos.data(), nullptr,
+                            nullptr, nullptr, nullptr) == PSKV_OK);  // push 1 of `repeat`
+  for (int r = 1; r < repeat; ++r) EXPECT(pskv_replay_run(push) == PSKV_OK);
+  EXPECT(pskv_pull_multi(t.data(), S, d_keys, pos.data(), d_out, nullptr, nullptr, nullptr, PSKV_MEM_DEVICE) == PSKV_OK);
+  EXPECT(pskv_sync_multi(t.data(), S) == PSKV_OK);
+  // the pull was another request: the recording is over
+  EXPECT(pskv_replay_run(push) == PSKV_ESTALE);
+  EXPECT(pskv_replay_destroy(push) == PSKV_OK);
+  EXPECT(hipMemcpy(got.data(), d_out, n * 4, hipMemcpyDeviceToHost) == hipSuccess);
+  size_t bad = 0;
+  for (size_t i = 0; i < n; ++i) {
+    float want = 0.0f;
+    for (int r = 0; r < repeat; ++r) want = want + vals[i];  // sequential float adds, as the store makes them
+    bad += got[i] != want;
+  }
+  EXPECT(bad == 0);
+  // push + pull recorded as one step; a key that changes under the recording stops its slice, and only that
+  pskv_replay* step = nullptr;
+  EXPECT(pskv_replay_record(&step, t.data(), S, PSKV_REPLAY_PUSH | PSKV_REPLAY_PULL, d_keys, pos.data(), d_vals,
+                            val_pos.data(), nullptr, d_out, nullptr, nullptr) == PSKV_OK);
+  EXPECT(pskv_replay_run(step) == PSKV_OK);
+  EXPECT(pskv_sync_multi(t.data(), S) == PSKV_OK);
+  EXPECT(hipMemcpy(got.data(), d_out, n * 4, hipMemcpyDeviceToHost) == hipSuccess);
+  size_t bad2 = 0;
+  for (size_t i = 0; i < n; ++i) {
+    float want = 0.0f;
+    for (int r = 0; r < repeat + 2; ++r) want = want + vals[i];
+    bad2 += got[i] != want;
+  }
+  EXPECT(bad2 == 0);
+  const uint64_t other = keys[n - 1] + 1;  // the last key of the last slice becomes another key of its range
+  EXPECT(hipMemcpy(d_keys + (n - 1), &other, 8, hipMemcpyHostToDevice) == hipSuccess);
+  EXPECT(pskv_replay_run(step) == PSKV_OK);  // enqueued; the device finds the difference
+  EXPECT(pskv_sync_multi(t.data(), S) == PSKV_ESTALE);
+  uint64_t held = 0, total = 0;
+  for (size_t s = 0; s < S; ++s) {
+    EXPECT(pskv_size(t[s], &held, nullptr) == PSKV_OK);
+    total += held;
+  }
+  EXPECT(total == n);  // the other key was not created
+  EXPECT(pskv_replay_destroy(step) == PSKV_OK);
+  EXPECT(hipFree(d_vals) == hipSuccess);
+  EXPECT(hipFree(d_out) == hipSuccess);
+  EXPECT(hipFree(d_keys) == hipSuccess);
+  for (size_t s = S; s-- > 0;) EXPECT(pskv_table_destroy(t[s]) == PSKV_OK);  // the owner of the stream last
+  std::printf("recorded requests: %d pushes of %zu keys over %zu ranges replayed, %zu + %zu floats differ\n", repeat, n,
+              S, bad, bad2);
+}
+
 static void RunTwoWorkers(int app_id) {
   std::thread t0(RunOneOfTwoWorkers, app_id, 0);
   std::thread t1(RunOneOfTwoWorkers, app_id, 1);
@@ -410,6 +491,7 @@ int main(int argc, char** argv) {
     RunFailures(num_servers);
     RunOrderedMatch();
     RunDeviceBufferContract();
+    RunRecordedRequests(num_servers);
     auto s6 = StartServers(6, num_servers, PSKV_MODE_SCALAR);
     RunTwoWorkers(6);
     if (argc > 2) {  // floats per key of the dense run from host memory (4194304 is the configuration's)
