@@ -529,6 +529,29 @@ def timed_replays(rec, group, steps, ref, add):
                     "one call, one launch, nothing sliced, allocated or waited for per step"}, ref
 
 
+def with_rates(replayed, n):
+    """Adds keys/s (pushed + pulled keys per step) to a `replayed` entry and to its `as_launches` part."""
+    out = dict(replayed, value=2.0 * n / (replayed["ms_per_step"] * 1e-3), unit="keys/s")
+    out["as_launches"] = dict(replayed["as_launches"], value=2.0 * n / (replayed["as_launches"]["ms_per_step"] * 1e-3),
+                              unit="keys/s")
+    return out
+
+
+def replay_both(capi, group, steps, ref, add, *record_args):
+    """Records the push + pull step with `record_args` (after the flags) as a HIP graph and as its launches,
+    times `steps` runs of each; returns the `replayed` entry and the sums the sample must have reached."""
+    rec = group.record(capi.REPLAY_PUSH | capi.REPLAY_PULL, *record_args)
+    replayed, ref = timed_replays(rec, group, steps, ref, add)
+    rec.close()
+    rec = group.record(capi.REPLAY_PUSH | capi.REPLAY_PULL | capi.REPLAY_LAUNCHES, *record_args)
+    relaunched, ref = timed_replays(rec, group, steps, ref, add)
+    rec.close()
+    relaunched["note"] = ("the same recording kept as its launches (PSKV_REPLAY_LAUNCHES), made again one by one by "
+                          "pskv_replay_run")
+    replayed["as_launches"] = relaunched
+    return replayed, ref
+
+
 def gen_varlen(n, S):
     limit = (KMAX // S) * S
     keys = unique_sorted_keys(np.random.default_rng(0xE3B), n, limit)
@@ -611,11 +634,9 @@ def run_varlen(args, capi, dev):
     if not per_table:
         # the same step recorded once (pskv_replay_record) and replayed: no slicing, one call and one launch
         pos, vpos, _ = capi.slice_keys(dk, rb, re, lens=dl, nvals=nvals)
-        rec = group.record(capi.REPLAY_PUSH | capi.REPLAY_PULL, dk, pos, dv, vpos, dl, out, vpos, out_lens)
-        replayed, ref = timed_replays(rec, group, args.steps, ref, dv[idx])
+        replayed, ref = replay_both(capi, group, args.steps, ref, dv[idx], dk, pos, dv, vpos, dl, out, vpos, out_lens)
         assert torch.equal(out_lens, dl), "pulled lens differ"
         assert torch.equal(out[idx], ref), "replayed var-len sums differ from sequential float adds"
-        rec.close()
     # on request, once more with the library's default of one stream per table (launches of
     # different ranges overlap; durations are then no longer a kernel's own, hence not the headline)
     dt_own = None
@@ -651,7 +672,7 @@ def run_varlen(args, capi, dev):
                                         bytes_per_float=8)},
     }
     if replayed is not None:
-        res["replayed"] = dict(replayed, value=2.0 * n / (replayed["ms_per_step"] * 1e-3), unit="keys/s")
+        res["replayed"] = with_rates(replayed, n)
     if dt_own is not None:
         res["own_streams"] = {"value": 2.0 * n * args.steps / dt_own, "unit": "keys/s",
                               "ms_per_step": dt_own / args.steps * 1e3,
@@ -935,14 +956,12 @@ def run_sparse_repeat(args, capi, dev):
     assert torch.equal(out[idx], ref), "push+pull sums differ from sequential float adds"
     # the same step recorded once (pskv_replay_record) and replayed: one call and one launch per step
     whole = np.array([0, n], np.uint64)
-    rec = group.record(capi.REPLAY_PUSH | capi.REPLAY_PULL, dk, whole, dv, whole, None, out)
-    replayed, ref = timed_replays(rec, group, args.steps, ref, dv[idx])
+    replayed, ref = replay_both(capi, group, args.steps, ref, dv[idx], dk, whole, dv, whole, None, out)
     assert torch.equal(out[idx], ref), "replayed sums differ from sequential float adds"
-    rec.close()
     res = {
         "value": 2.0 * n * args.steps / dt, "unit": "keys/s", "ms_per_step": dt / args.steps * 1e3,
         "dtype": "f32",
-        "replayed": dict(replayed, value=2.0 * n / (replayed["ms_per_step"] * 1e-3), unit="keys/s",
+        "replayed": dict(with_rates(replayed, n),
                          one_request={"ms_per_step": dt_pp / args.steps * 1e3, "value": 2.0 * n * args.steps / dt_pp,
                                       "unit": "keys/s",
                                       "note": "the step as one pskv_pushpull request, not recorded: what a recorded "
@@ -1268,16 +1287,14 @@ def extra_replay_small(capi, dev, n=100000, S=4, steps=200):
         ref = ref + dv
     assert torch.equal(out, ref), "push+pull sums differ from sequential float adds"
     pos, _, _ = capi.slice_keys(dk, rb, re, nvals=n)
-    rec = group.record(capi.REPLAY_PUSH | capi.REPLAY_PULL, dk, pos, dv, pos, None, out)
-    replayed, ref = timed_replays(rec, group, steps, ref, dv)
+    replayed, ref = replay_both(capi, group, steps, ref, dv, dk, pos, dv, pos, None, out)
     assert torch.equal(out, ref), "replayed sums differ from sequential float adds"
-    rec.close()
     group.close()
     return {"workload": "the same %d keys over %d key ranges pushed and pulled every step (SCALAR)" % (n, S),
             "steps": steps, "ms_per_step": dt / steps * 1e3, "value": 2.0 * n * steps / dt, "unit": "keys/s",
             "one_request": {"ms_per_step": dt_one / steps * 1e3, "value": 2.0 * n * steps / dt_one, "unit": "keys/s",
                             "note": "slice + ONE pskv_pushpull_multi request per step, not recorded"},
-            "replayed": dict(replayed, value=2.0 * n / (replayed["ms_per_step"] * 1e-3), unit="keys/s")}
+            "replayed": with_rates(replayed, n)}
 
 
 def extra_host_staged(capi, reps=2, nk=64, k=4194304):

@@ -171,8 +171,9 @@ int pskv_sync_multi(pskv_table* const* tables, size_t S);
  * arguments (device memory only; out_vals, out_pos and out_lens as pskv_pull_multi's out,
  * out_pos and out_lens; a PSKV_MODE_VARLEN response that does not fit is reported by the next
  * sync), waits for it, and keeps the launches that a repeat of it takes as a HIP graph on the
- * tables' stream (which must not be the null stream). It allocates and waits; it is a set-up call.
- * pskv_replay_run enqueues that graph: the request is applied again, to whatever the value
+ * tables' stream (which must not be the null stream), or, with PSKV_REPLAY_LAUNCHES, as the
+ * launches themselves. It allocates and waits; it is a set-up call.
+ * pskv_replay_run enqueues that graph (makes those launches again): the request is applied again, to whatever the value
  * buffers hold by the time the stream gets to it (keys, lens, positions and addresses are part
  * of the recording). It allocates nothing, waits for nothing and reads nothing back: the host
  * side of a step is this one call.
@@ -187,6 +188,9 @@ int pskv_sync_multi(pskv_table* const* tables, size_t S);
 typedef struct pskv_replay pskv_replay;
 #define PSKV_REPLAY_PUSH 1
 #define PSKV_REPLAY_PULL 2
+/* or-ed into `what`: keep the launches themselves instead of a graph; pskv_replay_run then makes them
+ * again one by one (same kernels, same arguments, same checks on the device). */
+#define PSKV_REPLAY_LAUNCHES 4
 int pskv_replay_record(pskv_replay** out, pskv_table* const* tables, size_t S, int what, const uint64_t* keys,
                        const uint64_t* pos, const float* vals, const uint64_t* val_pos, const int32_t* lens,
                        float* out_vals, const uint64_t* out_pos, int32_t* out_lens);

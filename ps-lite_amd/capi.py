@@ -24,6 +24,7 @@ ELEN_CHANGED = -7
 ESTALE = -8
 REPLAY_PUSH = 1
 REPLAY_PULL = 2
+REPLAY_LAUNCHES = 4
 MEM_HOST = 0
 MEM_DEVICE = 1
 MODE_SCALAR = 0

@@ -853,6 +853,16 @@ pskv_table* lead_of(Batch& bt) {
   return bt[0].t;
 }
 
+// A launch as pskv_replay_record keeps it: everything hipLaunchKernelGGL needs to make it again.
+struct SavedLaunch {
+  void (*kernel)(ReqBatch);
+  dim3 grid;
+  ReqBatch rb;
+};
+// Where launch_batch leaves a copy of its launches while a request is being recorded (the thread
+// that records is the thread that launches).
+thread_local std::vector<SavedLaunch>* g_recording = nullptr;
+
 // One launch for the whole batch: blockIdx.y selects the table, `nblk_of` says how many
 // workgroups serve each (0: none, the table sits this step out).
 template <typename F>
@@ -870,6 +880,7 @@ int launch_batch(Batch& bt, int prof_kernel, void (*kernel)(ReqBatch), F nblk_of
   if (!gx) return PSKV_OK;
   launch(lead_of(bt), prof_kernel, kernel, dim3((unsigned)gx, (unsigned)bt.size()), dim3(kBlock), rb);
   PSKV_HIP(hipGetLastError());
+  if (g_recording) g_recording->push_back(SavedLaunch{kernel, dim3((unsigned)gx, (unsigned)bt.size()), rb});
   return PSKV_OK;
 }
 
@@ -2044,6 +2055,7 @@ int pskv_pull_multi(pskv_table* const* tables, size_t S, const uint64_t* keys, c
 struct pskv_replay {
   std::vector<pskv_table*> tables;
   std::vector<uint64_t> gen;  // pskv_table::gen of each when the recording was made
+  std::vector<SavedLaunch> launches;  // PSKV_REPLAY_LAUNCHES: made again one by one instead of as a graph
   hipGraphExec_t exec = nullptr;
   hipStream_t stream = nullptr;
   int device = 0;
@@ -2056,7 +2068,8 @@ int pskv_replay_record(pskv_replay** out, pskv_table* const* tables, size_t S, i
   if (!out) return set_error(PSKV_EINVAL, "null argument");
   *out = nullptr;
   const bool push = (what & PSKV_REPLAY_PUSH) != 0, pull = (what & PSKV_REPLAY_PULL) != 0;
-  if ((!push && !pull) || (what & ~(PSKV_REPLAY_PUSH | PSKV_REPLAY_PULL)))
+  const bool as_graph = (what & PSKV_REPLAY_LAUNCHES) == 0;
+  if ((!push && !pull) || (what & ~(PSKV_REPLAY_PUSH | PSKV_REPLAY_PULL | PSKV_REPLAY_LAUNCHES)))
     return set_error(PSKV_EINVAL, "what = %d names neither a push nor a pull", what);
   if (S == 0) return set_error(PSKV_EINVAL, "no tables");
   int rc = check_group(tables, S);
@@ -2091,8 +2104,11 @@ int pskv_replay_record(pskv_replay** out, pskv_table* const* tables, size_t S, i
   // The launches of a repeat, recorded instead of run. Relaxed: other threads of the process may
   // be allocating or waiting meanwhile, which is none of this capture's business.
   PSKV_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed));
+  std::vector<SavedLaunch> saved;
   for (size_t s = 0; s < S; ++s) tables[s]->capturing = true;
+  g_recording = &saved;
   rc = both(kReplayCapture);
+  g_recording = nullptr;
   for (size_t s = 0; s < S; ++s) tables[s]->capturing = false;
   hipGraph_t graph = nullptr;
   const hipError_t e = hipStreamEndCapture(stream, &graph);
@@ -2109,13 +2125,14 @@ int pskv_replay_record(pskv_replay** out, pskv_table* const* tables, size_t S, i
     (void)hipGraphDestroy(graph);
     return set_error(PSKV_ENOMEM, "out of host memory");
   }
-  const hipError_t ei = hipGraphInstantiate(&r->exec, graph, nullptr, nullptr, 0);
+  const hipError_t ei = as_graph ? hipGraphInstantiate(&r->exec, graph, nullptr, nullptr, 0) : hipSuccess;
   (void)hipGraphDestroy(graph);
   if (ei != hipSuccess) {
     delete r;
     (void)hipGetLastError();
     return set_error(PSKV_EHIP, "hipGraphInstantiate: %s", hipGetErrorString(ei));
   }
+  if (!as_graph) r->launches.swap(saved);
   r->stream = stream;
   r->device = tables[0]->device;
   r->tables.assign(tables, tables + S);
@@ -2126,23 +2143,26 @@ int pskv_replay_record(pskv_replay** out, pskv_table* const* tables, size_t S, i
 
 int pskv_replay_run(pskv_replay* r) {
   clear_error();
-  if (!r || !r->exec) return set_error(PSKV_EINVAL, "null recording");
+  if (!r || (!r->exec && r->launches.empty())) return set_error(PSKV_EINVAL, "null recording");
   for (size_t s = 0; s < r->tables.size(); ++s)
     if (r->tables[s]->gen != r->gen[s])
       return set_error(PSKV_ESTALE, "tables[%zu] has served other requests since the recording was made", s);
   DeviceGuard guard(r->device);
   if (!guard.ok()) return set_error(PSKV_EHIP, "cannot select device %d", r->device);
-  PSKV_HIP(hipGraphLaunch(r->exec, r->stream));
+  if (r->exec) {
+    PSKV_HIP(hipGraphLaunch(r->exec, r->stream));
+    return PSKV_OK;
+  }
+  for (const SavedLaunch& l : r->launches) hipLaunchKernelGGL(l.kernel, l.grid, dim3(kBlock), 0, r->stream, l.rb);
+  PSKV_HIP(hipGetLastError());
   return PSKV_OK;
 }
 
 int pskv_replay_destroy(pskv_replay* r) {
   if (!r) return PSKV_OK;
   DeviceGuard guard(r->device);
-  if (r->exec) {
-    (void)hipStreamSynchronize(r->stream);
-    (void)hipGraphExecDestroy(r->exec);
-  }
+  (void)hipStreamSynchronize(r->stream);
+  if (r->exec) (void)hipGraphExecDestroy(r->exec);
   delete r;
   return PSKV_OK;
 }

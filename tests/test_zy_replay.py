@@ -69,9 +69,10 @@ class _Step:
 @pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
 @pytest.mark.parametrize("S,n", [(4, 400000), (1, 1000), (16, 40000), (37, 9000)])
 @pytest.mark.parametrize("what", ["push+pull", "push", "pull"])
-def test_replays_equal_the_oracle(capi, orc, dev, mode, S, n, what):
+@pytest.mark.parametrize("how", ["graph", "launches"])
+def test_replays_equal_the_oracle(capi, orc, dev, mode, S, n, what, how):
     import torch
-    announce("replay", mode, S, n, what)
+    announce("replay", mode, S, n, what, how)
     rng = np.random.default_rng(S * 7 + n + len(what))
     g = capi.Group(S, MODES[mode], initial_capacity=16, row_len=K if mode == "fixed" else 0)
     o = orc.Store(MODES[mode], K if mode == "fixed" else 0)
@@ -95,6 +96,8 @@ def test_replays_equal_the_oracle(capi, orc, dev, mode, S, n, what):
         o.push(keys, first, lens)
         g.sync()
     flags = {"push+pull": capi.REPLAY_PUSH | capi.REPLAY_PULL, "push": capi.REPLAY_PUSH, "pull": capi.REPLAY_PULL}[what]
+    if how == "launches":
+        flags |= capi.REPLAY_LAUNCHES
 
     def reference(vals):
         if "push" in what:
@@ -138,9 +141,10 @@ def test_replays_equal_the_oracle(capi, orc, dev, mode, S, n, what):
 
 
 @pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
-def test_a_replay_whose_keys_have_changed_applies_nothing(capi, orc, dev, mode):
+@pytest.mark.parametrize("how", [0, 4])  # a graph / the launches one by one (PSKV_REPLAY_LAUNCHES)
+def test_a_replay_whose_keys_have_changed_applies_nothing(capi, orc, dev, mode, how):
     import torch
-    announce("replay_changed_keys", mode)
+    announce("replay_changed_keys", mode, how)
     rng = np.random.default_rng(11)
     S, n = 4, 50000
     g = capi.Group(S, MODES[mode], initial_capacity=16, row_len=K if mode == "fixed" else 0)
@@ -150,7 +154,7 @@ def test_a_replay_whose_keys_have_changed_applies_nothing(capi, orc, dev, mode):
     st = _Step(capi, dev, rng, mode, S, keys, lens, nvals)
     vals = rng.normal(0, 1, size=nvals).astype(np.float32)
     st.set_vals(vals)
-    rec = g.record(capi.REPLAY_PUSH | capi.REPLAY_PULL, st.dk, st.pos, st.dv, st.vpos, st.dl, st.out, st.out_pos,
+    rec = g.record(capi.REPLAY_PUSH | capi.REPLAY_PULL | how, st.dk, st.pos, st.dv, st.vpos, st.dl, st.out, st.out_pos,
                    st.out_lens)
     o.push(keys, vals, lens)
     g.sync()
@@ -283,7 +287,7 @@ def test_replay_misuse_is_a_status_code(capi, dev):
     keys = torch.arange(10, dtype=torch.int64, device=dev)
     vals = torch.ones(10, dtype=torch.float32, device=dev)
     pos = np.array([0, 10, 10], np.uint64)
-    for what in (0, 4, 7):
+    for what in (0, 4, 8, 15):
         with pytest.raises(capi.PskvError) as e:
             g.record(what, keys, pos, vals, pos)
         assert e.value.code == capi.EINVAL
