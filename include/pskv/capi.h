@@ -181,6 +181,8 @@ int pskv_sync_multi(pskv_table* const* tables, size_t S);
  * therefore checks first, table by table, that the key (and lens) buffers still hold what was
  * recorded; a table whose slice has changed is left as it is by that run, its part of a pull
  * is not written, and the next pskv_sync / pskv_sync_multi reports PSKV_ESTALE for it.
+ * A PSKV_MODE_VARLEN pull on its own can only be recorded right behind a push of the same keys (a
+ * var-len pull creates nothing and leaves no key cache behind; PSKV_ESTALE otherwise).
  * Any other request on one of the tables (pskv_push, pskv_pull, pskv_dump, another recording)
  * may move what the recording points at, so it ends the recording's life: pskv_replay_run then
  * returns PSKV_ESTALE and enqueues nothing; record again. pskv_sync, pskv_sync_multi and

@@ -1183,7 +1183,10 @@ int begin_row_request(Batch& bt) {
     if (!it.r.n) continue;
     it.tag = next_tag(it.t, it.r, true);
     if (it.r.replay == kReplayCapture && !it.tag.try_cache)
-      return set_error(PSKV_ESTALE, "the key cache does not hold the request that is being recorded");
+      return set_error(PSKV_ESTALE, "the key cache does not hold the request that is being recorded%s",
+                       it.t->mode == PSKV_MODE_VARLEN ? " (a PSKV_MODE_VARLEN pull leaves no key cache behind: record "
+                                                        "it together with the push of its keys, or right behind one)"
+                                                      : "");
     it.d.tag = it.tag;
     it.d.outcome = it.t->outcome;
   }

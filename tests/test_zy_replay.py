@@ -299,3 +299,20 @@ def test_replay_misuse_is_a_status_code(capi, dev):
     assert e.value.code == capi.EINVAL
     g.sync()
     g.close()
+    # a var-len pull leaves no key cache behind: on its own it can only be recorded behind a push of its keys
+    g = capi.Group(2, capi.MODE_VARLEN)
+    lens = torch.full((10,), 4, dtype=torch.int32, device=dev)
+    vals = torch.ones(40, dtype=torch.float32, device=dev)
+    out = torch.zeros(40, dtype=torch.float32, device=dev)
+    out_lens = torch.zeros(10, dtype=torch.int32, device=dev)
+    vpos = np.array([0, 40, 40], np.uint64)
+    with pytest.raises(capi.PskvError) as e:
+        g.record(capi.REPLAY_PULL, keys, pos, None, None, None, out, vpos, out_lens)
+    assert e.value.code == capi.ESTALE and "PSKV_MODE_VARLEN pull" in str(e.value)
+    g.push(keys, pos, vals, vpos, lens)
+    rec = g.record(capi.REPLAY_PULL, keys, pos, None, None, None, out, vpos, out_lens)
+    rec.run()
+    g.sync()
+    assert torch.equal(out, vals) and torch.equal(out_lens, lens)
+    rec.close()
+    g.close()
