@@ -87,7 +87,9 @@ typedef struct pskv_opts {
   uint64_t initial_capacity; /* keys the table should hold before its first growth; 0 = default */
   uint64_t row_len;          /* PSKV_MODE_FIXED: floats per key, 0 = taken from the first push */
   uint64_t arena_floats;     /* row modes: initial value storage in floats, 0 = default */
-  float max_load;            /* highest fill of the slot array, 0 = 0.5 */
+  float max_load;            /* the fill the slot array is kept below, 0 = 0.5 (a table whose requests have
+                                mostly been naming keys it holds may run up to 0.85 rather than grow for the
+                                keys of requests in flight that are unlikely to be new) */
   uint32_t reserved;
   void* stream;              /* hipStream_t to run on, NULL = the table creates its own */
 } pskv_opts;

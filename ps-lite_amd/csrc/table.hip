@@ -61,6 +61,8 @@ constexpr int kSmallParts = 8;  // (128 KiB each: a SCALAR push of up to 10,000 
 // Host-resident buffers from this size on travel piece by piece through the ring of pinned memory
 // (stager.h), copying, transfer and kernels overlapping; smaller ones take one copy command.
 constexpr size_t kPipeBytes = 4u << 20;
+// The fill a slot array never exceeds, whatever the host assumed about the requests in flight (reserve()).
+constexpr double kHardLoad = 0.85;
 
 // A device buffer that only grows. Contents are not kept across growth.
 struct GrowBuf {
@@ -159,6 +161,7 @@ struct pskv_table {
   Snapshot* snap = nullptr;  // pinned host memory the device publishes into
   uint64_t record_seq = ~0ull;  // the newest request that was asked to publish its counters (all ones: none yet)
   double new_share = 0.0;  // share of the keys named by requests that were new, over the latest records
+  bool share_known = false;  // (a record has said so)
   DevState* st = nullptr;  // device
   StateView* st_host = nullptr;  // pinned: what read_state() last read of the device state
 
@@ -536,7 +539,8 @@ void adopt_snapshot(pskv_table* t) {
   // which share of the keys that requests named turned out to be new, lately (a moving average)
   if (named) {
     const double share = c > t->base_count ? std::min(1.0, (double)(c - t->base_count) / (double)named) : 0.0;
-    t->new_share = 0.5 * t->new_share + 0.5 * share;
+    t->new_share = t->share_known ? 0.5 * t->new_share + 0.5 * share : share;
+    t->share_known = true;
   }
   t->base_seq = s1 + 1;
   t->base_count = c;
@@ -706,8 +710,21 @@ struct PublishReq {
 
 int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit, PublishReq* pub) {
   if (t->no_growth) return PSKV_OK;
+  // Two limits. `limit` is the fill the table is kept below; `hard` (0.85 unless max_load is higher) is
+  // the fill it must never exceed. The keys in flight count in full against the second, and against the
+  // first with the share of them that is going to be new if requests go on as the latest records say
+  // (twice that share plus a tenth, to be on the safe side; in full while no record has said anything).
+  // A server whose requests mostly name keys it holds, the steady state of a parameter server, then does
+  // not grow, or wait, for keys that are not coming, however far ahead of the device its caller runs; if
+  // the requests change their ways the table runs fuller than `limit` for as long as it takes the next
+  // records to say so, never fuller than `hard`.
   const double limit = (double)t->max_load * (double)t->cap;
-  auto slots_short = [&]() { return (double)(t->base_count + t->pend_keys + n) > limit; };
+  const double hard = std::max((double)t->max_load, kHardLoad) * (double)t->cap;
+  const double share = t->share_known ? std::min(1.0, 2.0 * t->new_share + 0.1) : 1.0;
+  auto slots_short = [&]() {
+    const double in_flight = (double)(t->pend_keys + n);
+    return (double)t->base_count + in_flight > hard || (double)t->base_count + share * in_flight > limit;
+  };
   auto arena_short = [&]() {
     return units && (t->base_top + t->pend_units + units) * floats_per_unit > t->arena_cap;
   };

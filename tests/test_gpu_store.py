@@ -206,6 +206,77 @@ def test_device_trim_between_growths(capi, orc, dev):
     capi.device_trim()
 
 
+@pytest.mark.parametrize("mode", ["scalar", "fixed"])
+def test_a_table_does_not_grow_for_keys_that_are_not_coming(capi, orc, dev, mode):
+    """A table at a fill of 0.33 whose caller keeps many large requests in flight that name keys it
+    holds: counted in full, the keys in flight would take the table over its fill limit (0.7M held + two
+    requests of 0.2M unaccounted for + the request at hand = 1.3M against 1.05M), so it used to double
+    for nothing. The host now counts them with the share that the device's records say is new, and in
+    full only against a limit the array must never cross. When the requests then bring new keys after
+    all, the table grows in time: the slots never fill beyond 0.85 and every value matches the oracle."""
+    import torch
+    announce("no_growth_for_hits", mode)
+    rng = np.random.default_rng(77)
+    k = 4
+    m = {"scalar": capi.MODE_SCALAR, "fixed": capi.MODE_FIXED}[mode]
+    om = {"scalar": orc.MODE_SCALAR, "fixed": orc.MODE_FIXED}[mode]
+    width = 1 if mode == "scalar" else k
+    held = 700000
+    # (row storage for every row of the test up front: this is about the slots)
+    t = capi.Table(m, initial_capacity=1000000, row_len=k if mode == "fixed" else 0,
+                   arena_floats=(held + 700000) * k if mode == "fixed" else 0)
+    o = orc.Store(om, k if mode == "fixed" else 0)
+    universe = unique_keys(rng, held + 600000)
+    base = np.sort(universe[:held])
+    fresh = np.sort(universe[held:])
+    vals = rng.standard_normal(held * width).astype(np.float32)
+    t.push(to_dev(base, dev), to_dev(vals, dev))
+    o.push(base, vals)
+    t.sync()
+    assert t.counters()["slots"] == 1 << 21 and t.counters()["growths"] == 0
+    keep = []
+
+    def hits():
+        idx = np.sort(rng.choice(held, size=200000, replace=False))
+        keys = base[idx]
+        v = rng.standard_normal(keys.size * width).astype(np.float32)
+        dk, dv = to_dev(keys, dev), to_dev(v, dev)
+        keep.append((dk, dv))
+        t.push(dk, dv)
+        o.push(keys, v)
+
+    # two requests whose records the device has written by the time the next request looks (the GPU is
+    # idle, but the table has not been asked to wait): the host has learnt that such requests bring nothing new
+    for _ in range(2):
+        hits()
+        torch.cuda.synchronize()
+    for _ in range(80):  # never waited for
+        hits()
+    c = t.counters()
+    assert c["growths"] == 0 and c["waits"] == 0, c
+    # now the requests bring new keys after all, 100,000 at a time, still never waited for
+    for rep in range(6):
+        keys = fresh[rep * 100000:(rep + 1) * 100000]
+        v = rng.standard_normal(keys.size * width).astype(np.float32)
+        dk, dv = to_dev(keys, dev), to_dev(v, dev)
+        keep.append((dk, dv))
+        t.push(dk, dv)
+        o.push(keys, v)
+        assert t.counters()["slots"] * 0.85 >= held + (rep + 1) * 100000  # what the array may hold covers it
+    t.sync()
+    # the table may have run fuller than its fill limit for those few requests; the next request sees it
+    hits()
+    t.sync()
+    c = t.counters()
+    assert c["growths"] >= 1 and c["slots"] * 0.5 >= held + 600000, c
+    assert t.size()[0] == o.size()[0] == held + 600000
+    gk, gl, gv = t.dump()
+    ok, ol, ov = o.dump()
+    assert np.array_equal(gk, ok)
+    assert_bits_equal(gv, ov, "dump")
+    t.close()
+
+
 @pytest.mark.parametrize("mode", ["scalar", "fixed", "varlen"])
 def test_many_requests_in_flight_while_the_table_grows(capi, orc, dev, mode):
     """Device-resident requests are enqueued without waiting, so the host only has bounds on the
