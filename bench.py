@@ -909,9 +909,9 @@ def run_sparse_repeat(args, capi, dev):
     vals = rng.normal(0.0, 0.01, size=n).astype(np.float32)
     dk, dv = to_dev(keys, dev), to_dev(vals, dev)
     out = torch.empty(n, dtype=torch.float32, device=dev)
-    # Room for the requests in flight: until the device has answered, the host must assume that a
-    # request creates all its keys, and a table without that room makes every request wait for exact
-    # counters first (the sums would be the same, the steps about a quarter slower).
+    # Room for the requests in flight: until the device's first records have arrived, the host must
+    # assume that a request creates all its keys. (A table created with the default capacity grows to
+    # that room by itself during the first requests and then runs the same steps at the same speed.)
     group = capi.Group(1, capi.MODE_SCALAR, initial_capacity=int(n * 6))
     t = group.tables[0]
     torch.cuda.synchronize()
