@@ -720,8 +720,9 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
   // records to say so, never fuller than `hard`.
   const double limit = (double)t->max_load * (double)t->cap;
   const double hard = std::max((double)t->max_load, kHardLoad) * (double)t->cap;
-  const double share = t->share_known ? std::min(1.0, 2.0 * t->new_share + 0.1) : 1.0;
   auto slots_short = [&]() {
+    // (looked up on every call: a record adopted further down may have changed it)
+    const double share = t->share_known ? std::min(1.0, 2.0 * t->new_share + 0.1) : 1.0;
     const double in_flight = (double)(t->pend_keys + n);
     return (double)t->base_count + in_flight > hard || (double)t->base_count + share * in_flight > limit;
   };
