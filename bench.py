@@ -1427,6 +1427,10 @@ def main():
         extra["sparse_repeat"] = brief(rres, cpu_sparse_repeat(orc, *rin, budget_s=3.0) if orc is not None else None)
         del rin
         extra["replay_small"] = extra_replay_small(capi, dev)
+        log("extra: embed")
+        eres, ein = run_embed(sub, capi, dev)
+        extra["embed"] = brief(eres, cpu_embed(orc, *ein, budget_s=3.0) if orc is not None else None)
+        del ein
         log("extra: match")
         mres, min_ = run_match(sub, capi, dev)
         extra["match"] = brief(mres, cpu_match(orc, *min_, budget_s=3.0) if orc is not None else None)
