@@ -164,19 +164,20 @@ int pskv_pushpull_multi(pskv_table* const* tables, size_t S, const uint64_t* key
  * table's error state is cleared). */
 int pskv_sync_multi(pskv_table* const* tables, size_t S);
 
-/* A request that repeats, recorded once and replayed with ONE launch. The reference's own test
+/* A request that repeats, recorded once and replayed with ONE call. The reference's own test
  * pushes the same keys over and over (tests/test_kv_app.cc:36-44), and so does a worker that
  * trains a dense model: per step KVWorker::Send delivers the same keys in the same slices
  * (kv_app.h:574-613) and only the values differ. pskv_replay_record serves such a request once,
  * exactly as pskv_push_multi (what = PSKV_REPLAY_PUSH), pskv_pull_multi (PSKV_REPLAY_PULL) or
- * the one followed by the other (PSKV_REPLAY_PUSH | PSKV_REPLAY_PULL) would, with the same
+ * the one followed by the other (PSKV_REPLAY_PUSH | PSKV_REPLAY_PULL; PSKV_MODE_SCALAR tables serve
+ * the two as one request with both halves, which gives the same values) would, with the same
  * arguments (device memory only; out_vals, out_pos and out_lens as pskv_pull_multi's out,
  * out_pos and out_lens; a PSKV_MODE_VARLEN response that does not fit is reported by the next
  * sync), waits for it, and keeps the launches that a repeat of it takes as a HIP graph on the
  * tables' stream (which must not be the null stream), or, with PSKV_REPLAY_LAUNCHES, as the
  * launches themselves. It allocates and waits; it is a set-up call.
- * pskv_replay_run enqueues that graph (makes those launches again): the request is applied again, to whatever the value
- * buffers hold by the time the stream gets to it (keys, lens, positions and addresses are part
+ * pskv_replay_run enqueues that graph (makes those launches again): the request is applied
+ * again, to whatever the value buffers hold by the time the stream gets to it (keys, lens, positions and addresses are part
  * of the recording). It allocates nothing, waits for nothing and reads nothing back: the host
  * side of a step is this one call.
  * A replay creates no key and moves no buffer, and the host sizes nothing for it. The device
