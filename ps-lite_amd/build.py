@@ -78,7 +78,8 @@ def build_host_test():
 def build_oracle():
     """Compiles the CPU oracle (test infrastructure) and, when the reference tree is
     present, the reference's own slicer into oracle/_ref/."""
-    subprocess.run(["make", "-C", os.path.join(REPO, "oracle")], check=True,
+    # (-B: compiled on every call, like the library, so that a call says whether it still builds)
+    subprocess.run(["make", "-B", "-C", os.path.join(REPO, "oracle")], check=True,
                    stdout=subprocess.DEVNULL)
 
 
