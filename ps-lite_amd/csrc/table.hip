@@ -53,6 +53,8 @@ constexpr uint64_t kSlackBytes = 256ull << 20;  // tables up to this size trade 
 // one stays below this size; beyond it the host waits for exact counters before it spends the memory.
 constexpr uint64_t kGrowUnaskedBytes = 4096ull << 20;
 constexpr uint64_t kKeepInFlight = 2;  // requests the host leaves unaccounted for when it lets the device catch up
+// ... unless the array that the uncertainty would cost is this large: then it lets the device catch up all the way
+constexpr uint64_t kLargeArrayBytes = 1024ull << 20;
 constexpr uint64_t kSpareMaxBytes = 16384ull << 20;  // no array larger than this is allocated ahead of need
 // Host-resident requests up to this size (per direction) skip the copy commands: the kernels
 // read the request from, and write the response to, pinned host memory mapped into the GPU.
@@ -734,19 +736,23 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
   if (slots_short() || arena_short() || t->seq - t->base_seq >= (uint64_t)pskv_table::kLog - 1) {
     adopt_snapshot(t);
     const bool old_log = t->seq - t->base_seq >= (uint64_t)pskv_table::kLog - 1;
+    // (two requests of 16M keys that are left unaccounted for would make a 1 GiB array a 2 GiB one;
+    // the host's lead is worth less than that: a few tens of microseconds of idle GPU, once)
+    const uint64_t keep =
+        grown_cap(t, t->base_count + t->pend_keys + n) * sizeof(Slot) >= kLargeArrayBytes ? 0 : kKeepInFlight;
     if (slots_short() && !arena_short() && !old_log && (double)(t->base_count + n) <= limit &&
-        t->record_seq != ~0ull && t->record_seq >= t->base_seq && t->seq - t->base_seq > kKeepInFlight) {
+        t->record_seq != ~0ull && t->record_seq >= t->base_seq && t->seq - t->base_seq > keep) {
       // The array is only short if the requests in flight create most of their keys, and some of
       // them are going to say how many they did create: the host lets the device catch up, but not
-      // all the way. A caller that runs many requests ahead is held back until only kKeepInFlight
-      // requests are unaccounted for (so the device never runs dry, as it would in a wait for the
+      // all the way (unless a large array is at stake). A caller that runs many requests ahead is held
+      // back until only kKeepInFlight requests are unaccounted for (so the device never runs dry, as it would in a wait for the
       // stream, and the steps that follow do not run in lock-step with the host); if the array
       // still looks short then, it is replaced, at most that many requests early and sized for
       // at most that many requests of uncertainty.
       const auto t0 = std::chrono::steady_clock::now();
       unsigned spins = 0;
       while (slots_short() && (double)(t->base_count + n) <= limit && t->record_seq >= t->base_seq &&
-             t->seq - t->base_seq > kKeepInFlight) {
+             t->seq - t->base_seq > keep) {
         adopt_snapshot(t);
         if ((++spins & 63u) == 0) {
           if (std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(20)) break;
@@ -762,7 +768,8 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
       // sized for what the requests in flight could create at most, without asking the device how
       // many keys they did create. The move is queued behind them; nothing waits.
       const uint64_t most = t->base_count + t->pend_keys + n;
-      const uint64_t slack_n = t->cap * sizeof(Slot) <= kSlackBytes ? 2 * n : 0;
+      // (room for two more such requests while that keeps the array a small one)
+      const uint64_t slack_n = grown_cap(t, most + 2 * n) * sizeof(Slot) <= kSlackBytes ? 2 * n : 0;
       int rc = grow_slots(t, most + slack_n);
       if (rc) return rc;
       ++t->stats.growths_unasked;
@@ -774,7 +781,7 @@ int reserve(pskv_table* t, uint64_t n, uint64_t units, uint64_t floats_per_unit,
       // keys. Small tables get room for two more such requests, so that a caller who keeps
       // requests of this size in flight does not wait again on every one of them; for large
       // tables the wait is short next to their kernels and the memory is not.
-      const uint64_t slack_n = t->cap * sizeof(Slot) <= kSlackBytes ? 2 * n : 0;
+      const uint64_t slack_n = grown_cap(t, t->base_count + 3 * n) * sizeof(Slot) <= kSlackBytes ? 2 * n : 0;
       const uint64_t slack_u = t->arena_cap * sizeof(float) <= kSlackBytes ? 2 * units : 0;
       if ((double)(t->base_count + n + slack_n) > limit) {
         rc = grow_slots(t, t->base_count + n + slack_n);
