@@ -50,6 +50,16 @@ def test_errors_without_a_device(capi):
     b, e_ = capi.server_ranges(4)
     assert int(e_[-1]) == ((1 << 64) - 1) // 4 * 4
     assert capi.version().startswith("pskv")
+    # the recorded-request entry points refuse what they can refuse without a table
+    import ctypes
+    lib = capi.load()
+    h = ctypes.c_void_p()
+    assert lib.pskv_replay_record(ctypes.byref(h), None, 0, capi.REPLAY_PUSH, None, None, None, None, None, None,
+                                  None, None) == capi.EINVAL
+    assert lib.pskv_replay_record(None, None, 0, capi.REPLAY_PUSH, None, None, None, None, None, None, None,
+                                  None) == capi.EINVAL
+    assert lib.pskv_replay_run(None) == capi.EINVAL
+    assert lib.pskv_replay_destroy(None) == capi.OK
 
 
 def test_adapters_compile_with_in_process_surface(tmp_path):
